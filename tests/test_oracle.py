@@ -1,0 +1,246 @@
+"""Pins for the CPU oracle.  The reference stores no golden vectors for this path
+(its tests are closed forms and invariants: tests/test_moe.py, ablate/common/test_eager_radial.py),
+so each oracle function is pinned by library routines, special cases, invariants and tiny brute force
+written independently of the oracle's own expressions."""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import bibo_moe_oracle as O
+
+
+def _ulp_diff(a, b):
+    return np.abs(a.view(np.int32).astype(np.int64) - b.view(np.int32).astype(np.int64))
+
+
+# ------------------------------------------------------------------ sigmoid
+def test_canonical_exp_matches_libm():
+    y = np.linspace(-200, 200, 200001)
+    assert np.max(np.abs(O.exp64_canonical(y) - np.exp(y)) / np.exp(y)) < 1e-15
+
+
+def test_canonical_sigmoid_is_the_correctly_rounded_one():
+    rng = np.random.default_rng(0)
+    x = np.concatenate([rng.standard_normal(200000).astype(np.float32) * 4,
+                        np.linspace(-110, 110, 50001).astype(np.float32)])
+    s = O.sigmoid32(x)
+    # Python's math.exp on doubles, one rounding to float32: an independent evaluation
+    sample = x[::97]
+    ref = np.array([1.0 / (1.0 + math.exp(-float(v))) for v in sample]).astype(np.float32)
+    assert np.array_equal(s[::97], ref)
+    # the reference's torch.sigmoid (router.py:31) is within 2 ulp wherever the result is normal
+    m = np.abs(x) <= 80
+    assert _ulp_diff(s[m], torch.sigmoid(torch.from_numpy(x[m])).numpy()).max() <= 2
+
+
+def test_sigmoid_special_values_and_monotonicity():
+    x = np.array([0.0, -0.0, np.inf, -np.inf, 1e38, -1e38, 200.0, -200.0], dtype=np.float32)
+    assert O.sigmoid32(x).tolist() == [0.5, 0.5, 1.0, 0.0, 1.0, 0.0, 1.0, 0.0]
+    xs = np.sort(np.random.default_rng(1).standard_normal(100000).astype(np.float32) * 6)
+    assert (np.diff(O.sigmoid32(xs)) >= 0).all()
+    a = np.linspace(-30, 30, 10001).astype(np.float32)      # s(x) + s(-x) = 1
+    assert np.max(np.abs(O.sigmoid32(a).astype(np.float64) + O.sigmoid32(-a) - 1.0)) < 1.2e-7
+
+
+# ------------------------------------------------------------------ router
+def _brute_topk(sel_row, k):
+    order = sorted(range(len(sel_row)), key=lambda e: (-float(sel_row[e]), e))
+    return sorted(order[:k])
+
+
+@pytest.mark.parametrize("E,k", [(64, 6), (8, 2), (22, 2), (4, 1), (5, 5)])
+def test_selection_matches_brute_force_and_torch_topk(E, k):
+    rng = np.random.default_rng(E * 10 + k)
+    logits = (rng.standard_normal((257, E)) * 2).astype(np.float32)
+    bias = (rng.uniform(-0.05, 0.05, E)).astype(np.float32)
+    idx, w, scores = O.route_from_logits(logits, bias, k)
+    sel = scores + bias[None]
+    for t in range(logits.shape[0]):
+        assert idx[t].tolist() == _brute_topk(sel[t], k)
+    # torch.topk (router.py:39) picks the same SET whenever the boundary is not tied
+    tk = torch.topk(torch.from_numpy(sel), k, dim=-1, sorted=False).indices.sort(-1).values.numpy()
+    assert np.array_equal(tk, idx)
+    # reference invariants (tests/test_moe.py:138-145): fp32, positive, unit mass, indices in range
+    assert w.dtype == np.float32 and idx.dtype == np.int32
+    assert (w > 0).all() and idx.min() >= 0 and idx.max() < E
+    if k > 1:
+        assert np.allclose(w.sum(-1), 1.0, atol=1e-6)
+
+
+def test_ties_go_to_the_lowest_expert_index():
+    E, k = 8, 3
+    logits = np.zeros((4, E), dtype=np.float32)          # all scores equal -> experts 0,1,2
+    logits[1, 5] = 1.0                                    # one winner then lowest indices
+    logits[2, [6, 7]] = 1.0
+    logits[3, :] = [0.5, 0.7, 0.7, 0.7, 0.7, 0.2, 0.9, 0.7]
+    idx, w, _ = O.route_from_logits(logits, np.zeros(E, np.float32), k)
+    assert idx.tolist() == [[0, 1, 2], [0, 1, 5], [0, 6, 7], [1, 2, 6]]
+    # a tie created by the bias is broken the same way
+    b = np.zeros(E, np.float32); b[4] = 0.25
+    lg = np.zeros((1, E), np.float32)
+    idx, w, sc = O.route_from_logits(lg, b, 2)
+    assert idx.tolist() == [[0, 4]]
+
+
+def test_bias_moves_selection_but_never_weights():
+    """tests/test_moe.py:177-185, plus: weights are the unbiased scores of the chosen experts."""
+    rng = np.random.default_rng(3)
+    logits = rng.standard_normal((64, 16)).astype(np.float32)
+    bias = np.zeros(16, np.float32); bias[0] = 5.0
+    idx, w, scores = O.route_from_logits(logits, bias, 4, norm=False)
+    assert (idx == 0).any(axis=1).all()
+    assert np.array_equal(w, np.take_along_axis(scores, idx.astype(np.int64), 1))
+    assert w.max() <= 1.0
+    _, wn, _ = O.route_from_logits(logits, bias, 4)
+    assert np.allclose(wn, w / w.sum(-1, keepdims=True), rtol=1e-6)
+    _, ws, _ = O.route_from_logits(logits, bias, 4, norm="softmax")
+    assert np.allclose(ws, torch.softmax(torch.from_numpy(w), -1).numpy())
+
+
+def test_router_logits_and_gap():
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(33, 48, generator=g).bfloat16()
+    wr = (torch.randn(10, 48, generator=g) * 0.1).bfloat16()
+    lg = O.router_logits(x, wr)
+    assert lg.dtype == np.float32 and lg.shape == (33, 10)
+    ref = np.einsum("th,eh->te", x.double().numpy(), wr.double().numpy())   # experts are the ROW dim
+    assert np.max(np.abs(lg - ref)) < 1e-5
+    _, _, scores = O.route_from_logits(lg, np.zeros(10, np.float32), 3)
+    tk = torch.from_numpy(scores).topk(4, dim=-1).values                     # router.py:35-36
+    assert np.allclose(O.boundary_gap(scores, 3), (tk[:, 2] - tk[:, 3]).numpy())
+
+
+# ------------------------------------------------------------------ permutation
+@pytest.mark.parametrize("T,E,k", [(1, 4, 1), (37, 8, 2), (300, 64, 6), (64, 64, 6)])
+def test_permutation_matches_brute_force(T, E, k):
+    rng = np.random.default_rng(T)
+    idx = np.stack([np.sort(rng.choice(E, k, replace=False)) for _ in range(T)]).astype(np.int32)
+    counts, offsets, perm_slot, perm_token = O.permute(idx, E)
+    flat = idx.reshape(-1)
+    brute = sorted(range(T * k), key=lambda s: (int(flat[s]), s // k, s % k))
+    assert perm_slot.tolist() == brute
+    assert perm_token.tolist() == [s // k for s in brute]
+    assert counts.tolist() == [int((flat == e).sum()) for e in range(E)]
+    assert offsets[0] == 0 and offsets[-1] == T * k and (np.diff(offsets) == counts).all()
+    assert sorted(perm_slot.tolist()) == list(range(T * k))
+    assert (np.bincount(perm_token, minlength=T) == k).all()        # every token exactly k times
+
+
+def test_permutation_with_repeated_experts_and_empty_experts():
+    idx = np.array([[2, 2], [0, 2], [2, 0]], dtype=np.int32)     # legal at the experts seam
+    counts, offsets, perm_slot, perm_token = O.permute(idx, 4)
+    assert counts.tolist() == [2, 0, 4, 0]
+    assert offsets.tolist() == [0, 2, 2, 6, 6]
+    assert perm_slot.tolist() == [2, 5, 0, 1, 3, 4]
+    with pytest.raises(ValueError):
+        O.permute(np.array([[4]], dtype=np.int32), 4)
+
+
+# ------------------------------------------------------------------ experts
+def _tiny(E=4, H=16, I=8, T=5, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(T, H, generator=g, dtype=torch.float64)
+    wgu = torch.randn(E, 2 * I, H, generator=g, dtype=torch.float64) * 0.3
+    wd = torch.randn(E, H, I, generator=g, dtype=torch.float64) * 0.3
+    return x, wgu, wd
+
+
+def _scalar_expert(xrow, wgu_e, wd_e, theta):
+    """Pure-Python scalar evaluation of one expert on one row, written from the definition
+    r^p * SiLU(g/r) with r = rms(gate), p = sigmoid(theta) (tests/test_moe.py:36-37)."""
+    two_i, H = len(wgu_e), len(xrow)
+    I = two_i // 2
+    gu = [sum(wgu_e[j][h] * xrow[h] for h in range(H)) for j in range(two_i)]
+    gate, up = gu[:I], gu[I:]
+    r = math.sqrt(sum(v * v for v in gate) / I + 1e-6)
+    p = 1.0 / (1.0 + math.exp(-theta))
+    hid = [(r ** p) * (v / r) / (1.0 + math.exp(-v / r)) * u for v, u in zip(gate, up)]
+    return [sum(wd_e[o][i] * hid[i] for i in range(I)) for o in range(len(wd_e))]
+
+
+def test_experts_match_scalar_brute_force():
+    E, H, I, T, k = 4, 16, 8, 5, 2
+    x, wgu, wd = _tiny(E, H, I, T)
+    theta = torch.tensor([-2.0, 0.0, 1.5, 3.0], dtype=torch.float64)   # p = .12/.50/.82/.95
+    idx = np.array([[0, 1], [1, 3], [2, 3], [0, 2], [0, 3]], dtype=np.int32)
+    w = torch.tensor(np.random.default_rng(0).uniform(0.1, 1, (T, k)))
+    out = O.experts_forward(x, idx, w, wgu, wd, theta, dtype=torch.float64)
+    for t in range(T):
+        acc = [0.0] * H
+        for j in range(k):
+            e = int(idx[t, j])
+            y = _scalar_expert(x[t].tolist(), wgu[e].tolist(), wd[e].tolist(), float(theta[e]))
+            acc = [a + float(w[t, j]) * v for a, v in zip(acc, y)]
+        assert np.allclose(out[t].numpy(), acc, rtol=1e-10, atol=1e-12)
+
+
+def test_radial_special_cases():
+    x, wgu, wd = _tiny(seed=1)
+    g = (x @ wgu[0].t())[:, :8]
+    # p -> 0 is NormSiLU: SiLU(g * rsqrt(mean g^2 + eps)) (tests/test_moe.py:66-78)
+    a0 = O.radial_normsilu(g, torch.tensor(-40.0))
+    assert torch.allclose(a0, F.silu(g * torch.rsqrt(g.square().mean(-1, keepdim=True) + 1e-6)), rtol=1e-9)
+    # p -> 1: r * SiLU(g/r) = g * sigmoid(g/r)
+    r = (g.square().mean(-1, keepdim=True) + 1e-6).sqrt()
+    assert torch.allclose(O.radial_normsilu(g, torch.tensor(40.0)), g * torch.sigmoid(g / r), rtol=1e-9)
+    # degree-p homogeneity: act(a*g) = a^p act(g) for a > 0 (eps negligible) -- fails for r^theta
+    for theta in (-2.0, 0.0, 1.5):
+        p = 1 / (1 + math.exp(-theta))
+        lhs = O.radial_normsilu(3.0 * g, torch.tensor(theta))
+        assert torch.allclose(lhs, (3.0 ** p) * O.radial_normsilu(g, torch.tensor(theta)), rtol=1e-5)
+    # the mean is over the LAST dim only: rows are independent
+    assert torch.allclose(O.radial_normsilu(g[:2], torch.tensor(0.3)), O.radial_normsilu(g, torch.tensor(0.3))[:2])
+
+
+def test_gate_is_the_first_half_of_gate_up_rows():
+    """moe.py:85 chunk(2): rows 0..I-1 gate, I..2I-1 up.  Zeroing the up half must zero the output;
+    zeroing the gate half must too (SiLU(0) = 0)."""
+    x, wgu, wd = _tiny(E=1, seed=2)
+    idx = np.zeros((5, 1), np.int32); w = torch.ones(5, 1, dtype=torch.float64); th = torch.zeros(1)
+    a = wgu.clone(); a[:, 8:, :] = 0
+    assert O.experts_forward(x, idx, w, a, wd, th, dtype=torch.float64).abs().max() == 0
+    b = wgu.clone(); b[:, :8, :] = 0
+    assert O.experts_forward(x, idx, w, b, wd, th, dtype=torch.float64).abs().max() == 0
+    # swapping the halves changes the result (the activation is on the gate only)
+    c = torch.cat([wgu[:, 8:], wgu[:, :8]], 1)
+    o1 = O.experts_forward(x, idx, w, wgu, wd, th, dtype=torch.float64)
+    assert (O.experts_forward(x, idx, w, c, wd, th, dtype=torch.float64) - o1).abs().max() > 1e-3
+
+
+def test_combine_is_linear_in_the_weights_and_order_free():
+    x, wgu, wd = _tiny(seed=3)
+    th = torch.tensor([0.1, -0.3, 0.7, 0.0], dtype=torch.float64)
+    one = lambda e: O.experts_forward(x, np.full((5, 1), e, np.int32), torch.ones(5, 1, dtype=torch.float64),
+                                      wgu, wd, th, dtype=torch.float64)
+    idx = np.tile(np.array([[1, 3]], np.int32), (5, 1))
+    w = torch.tensor([[0.3, 0.7]], dtype=torch.float64).repeat(5, 1)
+    both = O.experts_forward(x, idx, w, wgu, wd, th, dtype=torch.float64)
+    assert torch.allclose(both, 0.3 * one(1) + 0.7 * one(3), rtol=1e-12)
+    swapped = O.experts_forward(x, idx[:, ::-1].copy(), w.flip(-1), wgu, wd, th, dtype=torch.float64)
+    assert torch.allclose(both, swapped, rtol=1e-12)
+
+
+def test_fp32_oracle_tracks_fp64_and_eager_loop_tracks_oracle():
+    p = O.make_inputs(T=96, H=64, E=8, k=2, I=32, bias="uniform", theta="normal", seed=7)
+    out32, idx, w = O.moe_forward(**p)
+    out64 = O.experts_forward(p["x"], idx, w, p["w_gate_up"], p["w_down"], p["theta"], dtype=torch.float64)
+    assert ((out32.double() - out64).abs().max() / out64.abs().max()) < 1e-5     # test_eager_radial.py:61
+    # the timed bf16 eager loop agrees with the fp32 oracle at the bf16 tolerance (test_act_silu.py:65-66)
+    eager = O.eager_loop_forward(**p)
+    assert eager.dtype == torch.bfloat16
+    assert ((eager.double() - out64).abs().max() / out64.abs().max()) < 2e-2
+    # fp32 eager loop == fp32 oracle to rounding (same routing: no ties in this draw)
+    pf = {k_: (v.float() if isinstance(v, torch.Tensor) else v) for k_, v in p.items()}
+    assert ((O.eager_loop_forward(**pf).double() - out64).abs().max() / out64.abs().max()) < 1e-5
+
+
+def test_workload_table_matches_the_named_shapes():
+    c = O.CONFIGS
+    assert (c["c2"]["T"], c["c2"]["H"], c["c2"]["I"]) == (8192, 768, 384)
+    assert (c["c3"]["T"], c["c3"]["H"], c["c3"]["I"]) == (64, 1024, 512)
+    p = O.make_inputs(**{**c["c4"], "T": 32})
+    assert (p["bias"][:4] == 2.0).all() and p["bias"][4:].abs().max() <= 0.01
+    assert p["x"].dtype == torch.bfloat16 and p["bias"].dtype == torch.float32
