@@ -1,0 +1,229 @@
+"""Benchmark of the BiBo sparse-MoE layer forward on one MI355X.
+
+One step = one forward of the whole layer (router, permutation, gate/up + Radial NormSiLU, down +
+combine) over one batch of the prefill workload (T=8192, H=768, E=64, k=6, I=384, bf16), inputs and
+weights resident in HBM.  Prints one JSON line; see --help for the flags."""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import pathlib
+import sys
+import time
+
+ROOT = pathlib.Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
+
+
+def flops_layer(T, H, E, k, I):
+    return 2 * T * H * E + 6 * T * k * H * I
+
+
+def bytes_layer(T, H, E, k, I, e_active):
+    return 2 * (3 * H * I * e_active + E * H + 2 * T * H) + 8 * E
+
+
+class Layer:
+    """Pre-allocated operands and a direct ctypes call per stage, so the timed loop does no allocation."""
+
+    def __init__(self, name, dev, algo="auto"):
+        import torch
+        from bibo_amd import _lib as L
+        from bibo_amd import ops
+        from oracle import bibo_moe_oracle as O
+        self.torch, self.L, self.ops = torch, L, ops
+        self.cfg = cfg = O.CONFIGS[name]
+        self.name = name
+        p = O.make_inputs(**cfg)
+        self.host = p
+        self.dev = dev
+        self.T, self.H, self.E, self.k, self.I = cfg["T"], cfg["H"], cfg["E"], cfg["k"], cfg["I"]
+        self.S = self.T * self.k
+        self.x = p["x"].to(dev)
+        self.wr = p["w_router"].to(dev)
+        self.bias = p["bias"].to(dev)
+        self.wgu = p["w_gate_up"].to(dev)
+        self.wd = p["w_down"].to(dev)
+        self.theta = p["theta"].to(dev)
+        T, H, E, k, I, S = self.T, self.H, self.E, self.k, self.I, self.S
+        self.out = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+        self.idx = torch.empty(T, k, dtype=torch.int32, device=dev)
+        self.w = torch.empty(T, k, dtype=torch.float32, device=dev)
+        self.counts = torch.empty(E, dtype=torch.int32, device=dev)
+        self.offsets = torch.empty(E + 1, dtype=torch.int32, device=dev)
+        self.perm_slot = torch.empty(S, dtype=torch.int32, device=dev)
+        self.perm_token = torch.empty(S, dtype=torch.int32, device=dev)
+        self.hidden = torch.empty(S, I, dtype=torch.bfloat16, device=dev)
+        self.ws = torch.empty(ops.workspace_bytes(T, H, E, k, I, L.DTYPE_BF16), dtype=torch.uint8, device=dev)
+        self.shape = L.Shape(T, H, E, k, I, L.DTYPE_BF16)
+        self.algo = ops.algo_code(algo)
+        self.lib = L.lib()
+        self.stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+        P = lambda t: ctypes.c_void_p(t.data_ptr())
+        self._fwd_args = (P(self.x), P(self.wr), P(self.bias), P(self.wgu), P(self.wd), P(self.theta),
+                          ctypes.byref(self.shape), L.NORM_SUM, self.algo, P(self.out), P(self.idx), P(self.w),
+                          P(self.counts), None, P(self.ws), self.ws.numel(), self.stream)
+        self._stages = {
+            "router": (self.lib.bibo_moe_router_fwd,
+                       (P(self.x), P(self.wr), P(self.bias), T, H, E, k, L.DTYPE_BF16, L.NORM_SUM, None, P(self.idx),
+                        P(self.w), None, self.stream)),
+            "permute": (self.lib.bibo_moe_permute,
+                        (P(self.idx), T, E, k, P(self.counts), P(self.offsets), P(self.perm_slot), P(self.perm_token),
+                         P(self.ws), self.ws.numel(), self.stream)),
+            "gateup": (self.lib.bibo_moe_gateup_fwd,
+                       (P(self.x), P(self.wgu), P(self.theta), P(self.offsets), P(self.perm_token), T, H, E, k, I,
+                        L.DTYPE_BF16, self.algo, P(self.hidden), self.stream)),
+            "down_combine": (self.lib.bibo_moe_down_combine_fwd,
+                             (P(self.hidden), P(self.wd), P(self.w), P(self.offsets), P(self.perm_slot), T, H, E, k, I,
+                              L.DTYPE_BF16, self.algo, P(self.out), P(self.ws), self.ws.numel(), self.stream)),
+        }
+
+    def forward(self):
+        rc = self.lib.bibo_moe_forward(*self._fwd_args)
+        if rc != 0:
+            self.L.check(rc, "bibo_moe_forward")
+
+    def stage(self, name):
+        fn, args = self._stages[name]
+        rc = fn(*args)
+        if rc != 0:
+            self.L.check(rc, name)
+
+    def time_forward(self, steps, warmup):
+        torch = self.torch
+        for _ in range(warmup):
+            self.forward()
+        torch.cuda.synchronize(self.dev)
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            self.forward()
+        torch.cuda.synchronize(self.dev)
+        return (time.perf_counter() - t0) / steps
+
+    def time_stages(self, steps):
+        """Average duration of each stage, HIP events on the launch stream around every call."""
+        torch = self.torch
+        names = list(self._stages)
+        for n in names:
+            self.stage(n)
+        torch.cuda.synchronize(self.dev)
+        acc = {n: 0.0 for n in names}
+        for _ in range(steps):
+            evs = [torch.cuda.Event(enable_timing=True) for _ in range(len(names) + 1)]
+            evs[0].record()
+            for i, n in enumerate(names):
+                self.stage(n)
+                evs[i + 1].record()
+            torch.cuda.synchronize(self.dev)
+            for i, n in enumerate(names):
+                acc[n] += evs[i].elapsed_time(evs[i + 1]) * 1e-3
+        return {n: v / steps for n, v in acc.items()}
+
+    def check(self):
+        """Parity of the benchmarked configuration against the oracle on a token sample."""
+        import numpy as np
+        from oracle import bibo_moe_oracle as O
+        torch = self.torch
+        self.forward()
+        torch.cuda.synchronize(self.dev)
+        idx = self.idx.cpu().numpy()
+        w = self.w.cpu().numpy()
+        rng = np.random.default_rng(0)
+        sample = rng.choice(self.T, min(self.T, 128), replace=False)
+        p = self.host
+        ref = O.experts_forward(p["x"][sample], idx[sample], w[sample], p["w_gate_up"], p["w_down"], p["theta"])
+        got = self.out.cpu()[sample].double()
+        return ((got - ref.double()).abs().max() / ref.double().abs().max()).item(), int((self.counts > 0).sum())
+
+
+def cpu_baseline(name, budget_s=20.0, sample_tokens=2048):
+    """The reference's eager CPU path (oracle restatement) timed on this box's host cores."""
+    import torch
+    from oracle import bibo_moe_oracle as O
+    cfg = dict(O.CONFIGS[name])
+    T = min(cfg["T"], sample_tokens)
+    p = O.make_inputs(**{**cfg, "T": T})
+    cores = torch.get_num_threads()
+    best = None
+    for label, cast in (("bf16", lambda t: t), ("fp32", lambda t: t.float())):
+        q = {k_: (cast(v) if isinstance(v, torch.Tensor) and v.dtype == torch.bfloat16 else v) for k_, v in p.items()}
+        O.eager_loop_forward(**q)                       # warm-up
+        t0 = time.perf_counter()
+        reps = 0
+        while reps < 5 and (time.perf_counter() - t0) < budget_s / 2:
+            O.eager_loop_forward(**q)
+            reps += 1
+        dt = (time.perf_counter() - t0) / max(reps, 1)
+        tps = T / dt
+        if best is None or tps > best[0]:
+            best = (tps, label, reps, dt)
+    return {"value": best[0], "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": f"first {T} tokens of the {name} workload (same weights), eager per-expert loop in {best[1]}, "
+                      f"{best[2]} timed forwards of {best[3]:.2f} s after one warm-up"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4"])
+    ap.add_argument("--algo", default="auto", choices=["auto", "generic", "mfma", "stream"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-decode", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+
+    import torch
+    from bibo_amd import _lib
+    if not _lib.LIB_PATH.exists():
+        import __graft_entry__
+        __graft_entry__.build()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    layer = Layer(args.workload, dev, args.algo)
+    rel, e_active = layer.check()
+    sec = layer.time_forward(args.steps, args.warmup)
+    stages = layer.time_stages(max(10, min(args.steps, 100)))
+    T, H, E, k, I, S = layer.T, layer.H, layer.E, layer.k, layer.I, layer.S
+    fl = flops_layer(T, H, E, k, I)
+    gateup_flops = 2 * S * H * 2 * I
+    out = {
+        "metric": "moe_layer_tokens_per_s", "value": T / sec, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": sec * 1e3, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: MoE layer forward T={T} H={H} E={E} k={k} I={I} bf16, seeded synthetic",
+                   "algo": args.algo},
+        "tflops": fl / sec / 1e12, "pct_bf16_mfma_peak": 100.0 * fl / sec / 1e12 / PEAK_BF16_TFLOPS,
+        "parity_rel_err_sample": rel, "experts_active": e_active,
+        "stage_us": {n: v * 1e6 for n, v in stages.items()},
+        "roofline": {"kernel": "gateup_mfma_kernel (grouped gate/up GEMM + Radial NormSiLU)", "bound": "mfma",
+                     "achieved": gateup_flops / stages["gateup"] / 1e12, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": gateup_flops / stages["gateup"] / 1e12 / PEAK_BF16_TFLOPS, "traffic": None},
+    }
+    if not args.no_decode and args.workload == "c2":
+        d = Layer("c3", dev, args.algo)
+        drel, dact = d.check()
+        dsec = d.time_forward(args.steps, args.warmup)
+        dst = d.time_stages(max(10, min(args.steps, 100)))
+        db = bytes_layer(d.T, d.H, d.E, d.k, d.I, dact)
+        out["decode"] = {"workload": f"c3: T={d.T} H={d.H} E={d.E} k={d.k} I={d.I} bf16", "tokens_per_s": d.T / dsec,
+                         "us_per_step": dsec * 1e6, "algorithmic_bytes": db, "hbm_gbs": db / dsec / 1e9,
+                         "pct_hbm_peak": 100.0 * db / dsec / 1e9 / PEAK_HBM_GBS, "experts_active": dact,
+                         "parity_rel_err_sample": drel, "stage_us": {n: v * 1e6 for n, v in dst.items()},
+                         "note": "single weight set: 201 MB of weights can sit in the 256 MB Infinity Cache"}
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(args.workload)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,227 @@
+// extern "C" entry points: host-side argument checks, workspace carving and kernel dispatch.
+// Nothing here allocates or synchronises; see include/bibo_moe.h for the contract.
+#include "common.h"
+
+namespace {
+
+using namespace bibo;
+
+constexpr size_t kAlign = 256;
+inline size_t align_up(size_t v) { return (v + kAlign - 1) & ~(kAlign - 1); }
+inline size_t elt_size(int dtype) { return dtype == BIBO_DTYPE_BF16 ? 2 : 4; }
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+int check_dims(int T, int H, int E, int k, int I, int dtype) {
+  if (dtype != BIBO_DTYPE_BF16 && dtype != BIBO_DTYPE_F32) return BIBO_ERR_BAD_DTYPE;
+  if (T < 0 || H < 1 || I < 1 || E < 1 || E > kMaxE || k < 1 || k > kMaxK || k > E) return BIBO_ERR_BAD_SHAPE;
+  if ((long long)T * k > 0x3fffffffLL) return BIBO_ERR_BAD_SHAPE;
+  return BIBO_OK;
+}
+
+int resolve_algo(int algo, int H, int I, int dtype, int* out) {
+  switch (algo) {
+    case BIBO_ALGO_AUTO: *out = mfma_supported(H, I, dtype) ? BIBO_ALGO_MFMA : BIBO_ALGO_GENERIC; break;
+    case BIBO_ALGO_GENERIC: *out = BIBO_ALGO_GENERIC; break;
+    case BIBO_ALGO_MFMA:
+      if (!mfma_supported(H, I, dtype)) return BIBO_ERR_UNSUPPORTED;
+      *out = BIBO_ALGO_MFMA;
+      break;
+    default: return BIBO_ERR_UNSUPPORTED;
+  }
+  // the generic kernels keep one activation row (H + 2I floats) in LDS
+  if (*out == BIBO_ALGO_GENERIC && (size_t)(H + 2 * I) * sizeof(float) > 64 * 1024) return BIBO_ERR_UNSUPPORTED;
+  return BIBO_OK;
+}
+
+struct Workspace {
+  size_t hist, idx, w, counts, offsets, perm_slot, perm_token, hidden, yw, total;
+};
+
+Workspace carve(int T, int H, int E, int k, int I, int dtype) {
+  (void)E;
+  const size_t S = (size_t)T * k;
+  Workspace ws;
+  size_t o = 0;
+  ws.hist = o;       o += align_up(permute_workspace_bytes(T));
+  ws.idx = o;        o += align_up(S * sizeof(int32_t));
+  ws.w = o;          o += align_up(S * sizeof(float));
+  ws.counts = o;     o += align_up(kMaxE * sizeof(int32_t));
+  ws.offsets = o;    o += align_up((kMaxE + 1) * sizeof(int32_t));
+  ws.perm_slot = o;  o += align_up(S * sizeof(int32_t));
+  ws.perm_token = o; o += align_up(S * sizeof(int32_t));
+  ws.hidden = o;     o += align_up(S * (size_t)I * elt_size(dtype));
+  ws.yw = o;         o += align_up(S * (size_t)H * sizeof(float));
+  ws.total = o;
+  return ws;
+}
+
+inline int hip_rc(hipError_t e) { return e == hipSuccess ? BIBO_OK : (int)e; }
+
+int gateup_dispatch(const void* x, const void* wgu, const float* theta, const int32_t* offsets,
+                    const int32_t* perm_token, int T, int H, int E, int k, int I, int dtype, int algo, void* hidden,
+                    hipStream_t s) {
+  if (algo == BIBO_ALGO_MFMA) {
+    if (!aligned16(x) || !aligned16(wgu) || !aligned16(hidden)) return BIBO_ERR_MISALIGNED;
+    return hip_rc(launch_gateup_mfma(x, wgu, theta, offsets, perm_token, T, H, E, k, I, hidden, s));
+  }
+  return hip_rc(launch_gateup_generic(x, wgu, theta, offsets, perm_token, T, H, E, k, I, dtype, hidden, s));
+}
+
+int down_dispatch(const void* hidden, const void* wd, const float* w, const int32_t* offsets, const int32_t* perm_slot,
+                  int T, int H, int E, int k, int I, int dtype, int algo, void* out, float* yw, hipStream_t s) {
+  hipError_t e;
+  if (algo == BIBO_ALGO_MFMA) {
+    if (!aligned16(hidden) || !aligned16(wd)) return BIBO_ERR_MISALIGNED;
+    e = launch_down_mfma(hidden, wd, w, offsets, perm_slot, T, H, E, k, I, yw, /*yw_is_bf16=*/0, s);
+  } else {
+    e = launch_down_generic(hidden, wd, w, offsets, perm_slot, T, H, E, k, I, dtype, yw, s);
+  }
+  if (e != hipSuccess) return (int)e;
+  return hip_rc(launch_combine(yw, 0, T, H, k, dtype, out, s));
+}
+
+}  // namespace
+
+extern "C" {
+
+int bibo_moe_abi_version(void) { return BIBO_MOE_ABI_VERSION; }
+
+const char* bibo_moe_strerror(int code) {
+  switch (code) {
+    case BIBO_OK: return "success";
+    case BIBO_ERR_NULL_POINTER: return "a required pointer is NULL";
+    case BIBO_ERR_BAD_SHAPE: return "bad shape: need T >= 0, H, I >= 1, 1 <= E <= 64, 1 <= k <= min(E, 8)";
+    case BIBO_ERR_BAD_DTYPE: return "dtype must be BIBO_DTYPE_BF16 or BIBO_DTYPE_F32";
+    case BIBO_ERR_WORKSPACE_TOO_SMALL: return "workspace smaller than bibo_moe_workspace_bytes() for this shape";
+    case BIBO_ERR_MISALIGNED: return "tensor base pointers must be 16-byte aligned";
+    case BIBO_ERR_UNSUPPORTED: return "requested kernel family does not support this shape or dtype";
+    default: break;
+  }
+  if (code > 0) return hipGetErrorString((hipError_t)code);
+  return "unknown error code";
+}
+
+int bibo_moe_workspace_bytes(const bibo_moe_shape* sh, size_t* bytes) {
+  if (sh == nullptr || bytes == nullptr) return BIBO_ERR_NULL_POINTER;
+  const int rc = check_dims(sh->T, sh->H, sh->E, sh->k, sh->I, sh->dtype);
+  if (rc != BIBO_OK) return rc;
+  *bytes = carve(sh->T, sh->H, sh->E, sh->k, sh->I, sh->dtype).total;
+  return BIBO_OK;
+}
+
+int bibo_moe_router_fwd(const void* x, const void* w_router, const float* bias, int T, int H, int E, int k, int dtype,
+                        int norm_mode, float* logits, int32_t* idx, float* w, float* gap, void* stream) {
+  const int rc = check_dims(T, H, E, k, 1, dtype);
+  if (rc != BIBO_OK) return rc;
+  if (norm_mode < BIBO_NORM_NONE || norm_mode > BIBO_NORM_SOFTMAX) return BIBO_ERR_UNSUPPORTED;
+  if (T == 0) return BIBO_OK;
+  if (!x || !w_router || !bias || !idx || !w) return BIBO_ERR_NULL_POINTER;
+  return hip_rc(launch_router(x, w_router, bias, T, H, E, k, dtype, norm_mode, logits, idx, w, gap,
+                              static_cast<hipStream_t>(stream)));
+}
+
+int bibo_moe_permute(const int32_t* idx, int T, int E, int k, int32_t* counts, int32_t* offsets, int32_t* perm_slot,
+                     int32_t* perm_token, void* workspace, size_t workspace_bytes, void* stream) {
+  const int rc = check_dims(T, 1, E, k, 1, BIBO_DTYPE_BF16);
+  if (rc != BIBO_OK) return rc;
+  if (!counts || !offsets || !workspace) return BIBO_ERR_NULL_POINTER;
+  if (T > 0 && (!idx || !perm_slot || !perm_token)) return BIBO_ERR_NULL_POINTER;
+  if (workspace_bytes < permute_workspace_bytes(T)) return BIBO_ERR_WORKSPACE_TOO_SMALL;
+  return hip_rc(launch_permute(idx, T, E, k, counts, offsets, perm_slot, perm_token, workspace,
+                               static_cast<hipStream_t>(stream)));
+}
+
+int bibo_moe_gateup_fwd(const void* x, const void* w_gate_up, const float* theta, const int32_t* offsets,
+                        const int32_t* perm_token, int T, int H, int E, int k, int I, int dtype, int algo, void* hidden,
+                        void* stream) {
+  int rc = check_dims(T, H, E, k, I, dtype);
+  if (rc != BIBO_OK) return rc;
+  int a;
+  if ((rc = resolve_algo(algo, H, I, dtype, &a)) != BIBO_OK) return rc;
+  if (T == 0) return BIBO_OK;
+  if (!x || !w_gate_up || !theta || !offsets || !perm_token || !hidden) return BIBO_ERR_NULL_POINTER;
+  return gateup_dispatch(x, w_gate_up, theta, offsets, perm_token, T, H, E, k, I, dtype, a, hidden,
+                         static_cast<hipStream_t>(stream));
+}
+
+int bibo_moe_down_combine_fwd(const void* hidden, const void* w_down, const float* w, const int32_t* offsets,
+                              const int32_t* perm_slot, int T, int H, int E, int k, int I, int dtype, int algo,
+                              void* out, void* workspace, size_t workspace_bytes, void* stream) {
+  int rc = check_dims(T, H, E, k, I, dtype);
+  if (rc != BIBO_OK) return rc;
+  int a;
+  if ((rc = resolve_algo(algo, H, I, dtype, &a)) != BIBO_OK) return rc;
+  if (T == 0) return BIBO_OK;
+  if (!hidden || !w_down || !w || !offsets || !perm_slot || !out || !workspace) return BIBO_ERR_NULL_POINTER;
+  if (workspace_bytes < (size_t)T * k * H * sizeof(float)) return BIBO_ERR_WORKSPACE_TOO_SMALL;
+  return down_dispatch(hidden, w_down, w, offsets, perm_slot, T, H, E, k, I, dtype, a, out,
+                       static_cast<float*>(workspace), static_cast<hipStream_t>(stream));
+}
+
+int bibo_moe_experts_fwd(const void* x, const int32_t* idx, const float* w, const void* w_gate_up, const void* w_down,
+                         const float* theta, const bibo_moe_shape* sh, int algo, void* out, int32_t* counts_out,
+                         void* workspace, size_t workspace_bytes, void* stream) {
+  if (sh == nullptr) return BIBO_ERR_NULL_POINTER;
+  const int T = sh->T, H = sh->H, E = sh->E, k = sh->k, I = sh->I, dtype = sh->dtype;
+  int rc = check_dims(T, H, E, k, I, dtype);
+  if (rc != BIBO_OK) return rc;
+  int a;
+  if ((rc = resolve_algo(algo, H, I, dtype, &a)) != BIBO_OK) return rc;
+  if (!workspace) return BIBO_ERR_NULL_POINTER;
+  if (T > 0 && (!x || !idx || !w || !w_gate_up || !w_down || !theta || !out)) return BIBO_ERR_NULL_POINTER;
+  const Workspace ws = carve(T, H, E, k, I, dtype);
+  if (workspace_bytes < ws.total) return BIBO_ERR_WORKSPACE_TOO_SMALL;
+  char* base = static_cast<char*>(workspace);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  int32_t* counts = counts_out ? counts_out : reinterpret_cast<int32_t*>(base + ws.counts);
+  int32_t* offsets = reinterpret_cast<int32_t*>(base + ws.offsets);
+  int32_t* perm_slot = reinterpret_cast<int32_t*>(base + ws.perm_slot);
+  int32_t* perm_token = reinterpret_cast<int32_t*>(base + ws.perm_token);
+  if ((rc = hip_rc(launch_permute(idx, T, E, k, counts, offsets, perm_slot, perm_token, base + ws.hist, s))) != BIBO_OK)
+    return rc;
+  if (T == 0) return BIBO_OK;
+  if ((rc = gateup_dispatch(x, w_gate_up, theta, offsets, perm_token, T, H, E, k, I, dtype, a, base + ws.hidden, s)) !=
+      BIBO_OK)
+    return rc;
+  return down_dispatch(base + ws.hidden, w_down, w, offsets, perm_slot, T, H, E, k, I, dtype, a, out,
+                       reinterpret_cast<float*>(base + ws.yw), s);
+}
+
+int bibo_moe_forward(const void* x, const void* w_router, const float* bias, const void* w_gate_up, const void* w_down,
+                     const float* theta, const bibo_moe_shape* sh, int norm_mode, int algo, void* out, int32_t* idx_out,
+                     float* w_out, int32_t* counts_out, float* logits_out, void* workspace, size_t workspace_bytes,
+                     void* stream) {
+  if (sh == nullptr) return BIBO_ERR_NULL_POINTER;
+  const int T = sh->T, H = sh->H, E = sh->E, k = sh->k, I = sh->I, dtype = sh->dtype;
+  int rc = check_dims(T, H, E, k, I, dtype);
+  if (rc != BIBO_OK) return rc;
+  if (norm_mode < BIBO_NORM_NONE || norm_mode > BIBO_NORM_SOFTMAX) return BIBO_ERR_UNSUPPORTED;
+  int a;
+  if ((rc = resolve_algo(algo, H, I, dtype, &a)) != BIBO_OK) return rc;
+  if (!workspace) return BIBO_ERR_NULL_POINTER;
+  if (T > 0 && (!x || !w_router || !bias || !w_gate_up || !w_down || !theta || !out)) return BIBO_ERR_NULL_POINTER;
+  const Workspace ws = carve(T, H, E, k, I, dtype);
+  if (workspace_bytes < ws.total) return BIBO_ERR_WORKSPACE_TOO_SMALL;
+  char* base = static_cast<char*>(workspace);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  int32_t* idx = idx_out ? idx_out : reinterpret_cast<int32_t*>(base + ws.idx);
+  float* w = w_out ? w_out : reinterpret_cast<float*>(base + ws.w);
+  if (T > 0 &&
+      (rc = hip_rc(launch_router(x, w_router, bias, T, H, E, k, dtype, norm_mode, logits_out, idx, w, nullptr, s))) !=
+          BIBO_OK)
+    return rc;
+  int32_t* counts = counts_out ? counts_out : reinterpret_cast<int32_t*>(base + ws.counts);
+  int32_t* offsets = reinterpret_cast<int32_t*>(base + ws.offsets);
+  int32_t* perm_slot = reinterpret_cast<int32_t*>(base + ws.perm_slot);
+  int32_t* perm_token = reinterpret_cast<int32_t*>(base + ws.perm_token);
+  if ((rc = hip_rc(launch_permute(idx, T, E, k, counts, offsets, perm_slot, perm_token, base + ws.hist, s))) != BIBO_OK)
+    return rc;
+  if (T == 0) return BIBO_OK;
+  if ((rc = gateup_dispatch(x, w_gate_up, theta, offsets, perm_token, T, H, E, k, I, dtype, a, base + ws.hidden, s)) !=
+      BIBO_OK)
+    return rc;
+  return down_dispatch(base + ws.hidden, w_down, w, offsets, perm_slot, T, H, E, k, I, dtype, a, out,
+                       reinterpret_cast<float*>(base + ws.yw), s);
+}
+
+}  // extern "C"

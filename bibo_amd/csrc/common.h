@@ -1,0 +1,114 @@
+// Shared device helpers and host-side launcher declarations for the BiBo MoE kernels (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/bibo_moe.h"
+
+namespace bibo {
+
+constexpr int kWave = 64;
+constexpr int kMaxE = BIBO_MOE_MAX_EXPERTS;
+constexpr int kMaxK = BIBO_MOE_MAX_TOPK;
+constexpr float kNormSiluEps = 1e-6f;   // src/modeling/ffn/moe.py:16
+constexpr float kSumNormEps = 1e-20f;   // src/modeling/ffn/router.py:45
+
+// tokens handled by one workgroup of the histogram / permutation kernels
+constexpr int kPermTokens = 64;
+
+typedef __bf16 bf16_t;
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float to_float(float v) { return v; }
+__device__ __forceinline__ float to_float(bf16_t v) { return (float)v; }
+template <typename T> __device__ __forceinline__ T from_float(float v);
+template <> __device__ __forceinline__ float from_float<float>(float v) { return v; }
+template <> __device__ __forceinline__ bf16_t from_float<bf16_t>(float v) { return (bf16_t)v; }
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+  return v;
+}
+
+__device__ __forceinline__ int wave_inclusive_scan(int v) {
+  const int lane = lane_id();
+#pragma unroll
+  for (int o = 1; o < kWave; o <<= 1) {
+    int u = __shfl_up(v, o, kWave);
+    if (lane >= o) v += u;
+  }
+  return v;
+}
+
+// Routing sigmoid: float32(1 / (1 + exp64(-x))) with exp64 a fixed sequence of IEEE double
+// multiplies and adds (never fused), so that every platform produces the same bits.
+//   y = clamp(-x, -200, 200); n = floor(y*log2e + 0.5); r = (y - n*LN2_HI) - n*LN2_LO;
+//   p = Horner over 1/13! .. 1/0!; e = p * 2^n.
+// Reference operation: torch.sigmoid on the fp32 logits, src/modeling/ffn/router.py:31.
+__device__ __forceinline__ float sigmoid32_canonical(float x) {
+#pragma clang fp contract(off)
+  double y = -(double)x;
+  y = fmin(fmax(y, -200.0), 200.0);
+  const double t = y * 1.4426950408889634;
+  const double n = floor(t + 0.5);
+  double r = y - n * 0.693147180369123816490;
+  r = r - n * 1.90821492927058770002e-10;
+  double p = 1.0 / 6227020800.0;
+  p = p * r; p = p + 1.0 / 479001600.0;
+  p = p * r; p = p + 1.0 / 39916800.0;
+  p = p * r; p = p + 1.0 / 3628800.0;
+  p = p * r; p = p + 1.0 / 362880.0;
+  p = p * r; p = p + 1.0 / 40320.0;
+  p = p * r; p = p + 1.0 / 5040.0;
+  p = p * r; p = p + 1.0 / 720.0;
+  p = p * r; p = p + 1.0 / 120.0;
+  p = p * r; p = p + 1.0 / 24.0;
+  p = p * r; p = p + 1.0 / 6.0;
+  p = p * r; p = p + 0.5;
+  p = p * r; p = p + 1.0;
+  p = p * r; p = p + 1.0;
+  const long long bits = ((long long)((int)n + 1023)) << 52;
+  const double e = p * __longlong_as_double(bits);
+  const double d = 1.0 + e;
+  return (float)(1.0 / d);
+}
+
+// Map a workgroup id to a tile so that the workgroups of one XCD (ids congruent mod 8 are dispatched
+// to the same XCD) walk a contiguous range of tiles: tiles of one expert then share that XCD's L2.
+__device__ __forceinline__ int xcd_tile(int bid, int total) {
+  const int per = (total + 7) >> 3;
+  const int slot = bid >> 3;
+  if (slot >= per) return total;   // no tile
+  return (bid & 7) * per + slot;
+}
+
+// ---- host-side launchers (one per translation unit) -------------------------------------------
+hipError_t launch_router(const void* x, const void* w_router, const float* bias, int T, int H, int E, int k, int dtype,
+                         int norm_mode, float* logits, int32_t* idx, float* w, float* gap, hipStream_t s);
+size_t permute_workspace_bytes(int T);
+hipError_t launch_permute(const int32_t* idx, int T, int E, int k, int32_t* counts, int32_t* offsets,
+                          int32_t* perm_slot, int32_t* perm_token, void* ws, hipStream_t s);
+hipError_t launch_gateup_generic(const void* x, const void* wgu, const float* theta, const int32_t* offsets,
+                                 const int32_t* perm_token, int T, int H, int E, int k, int I, int dtype, void* hidden,
+                                 hipStream_t s);
+hipError_t launch_down_generic(const void* hidden, const void* wd, const float* w, const int32_t* offsets,
+                               const int32_t* perm_slot, int T, int H, int E, int k, int I, int dtype, float* yw,
+                               hipStream_t s);
+hipError_t launch_combine(const void* yw, int yw_is_bf16, int T, int H, int k, int dtype, void* out, hipStream_t s);
+bool mfma_supported(int H, int I, int dtype);
+hipError_t launch_gateup_mfma(const void* x, const void* wgu, const float* theta, const int32_t* offsets,
+                              const int32_t* perm_token, int T, int H, int E, int k, int I, void* hidden, hipStream_t s);
+hipError_t launch_down_mfma(const void* hidden, const void* wd, const float* w, const int32_t* offsets,
+                            const int32_t* perm_slot, int T, int H, int E, int k, int I, void* yw, int yw_is_bf16,
+                            hipStream_t s);
+
+}  // namespace bibo

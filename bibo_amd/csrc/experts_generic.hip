@@ -1,0 +1,155 @@
+// Generic expert kernels: one workgroup per routed row, any H and I, bf16 or fp32 operands, fp32
+// accumulation.  They serve shapes the MFMA tiles do not cover and fp32 modules, and double as an
+// independent implementation the MFMA kernels are cross-checked against.
+// Follow BiBoFusedExperts.forward, src/modeling/ffn/moe.py:73-101 of the reference.
+#include "common.h"
+
+namespace bibo {
+namespace {
+
+__device__ __forceinline__ int find_expert(const int32_t* __restrict__ offsets, int E, int row, int* sh) {
+  // offsets is non-decreasing; the owner is the last expert with offsets[e] <= row < offsets[e+1]
+  const int tid = threadIdx.x;
+  if (tid < E && offsets[tid] <= row && row < offsets[tid + 1]) *sh = tid;
+  __syncthreads();
+  return *sh;
+}
+
+// hidden[row, :] = r^p * SiLU(g/r) * up   (moe.py:84-92)
+template <typename TIn>
+__global__ __launch_bounds__(256) void gateup_generic_kernel(const TIn* __restrict__ x, const TIn* __restrict__ wgu,
+                                                             const float* __restrict__ theta,
+                                                             const int32_t* __restrict__ offsets,
+                                                             const int32_t* __restrict__ perm_token, int H, int E,
+                                                             int I, TIn* __restrict__ hidden) {
+  extern __shared__ float smem[];
+  float* xs = smem;            // [H]
+  float* gu = smem + H;        // [2I]
+  __shared__ int sh_e;
+  __shared__ float red[4];
+  const int row = blockIdx.x;
+  if (row >= offsets[E]) return;
+  const int e = find_expert(offsets, E, row, &sh_e);
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const TIn* xr = x + (size_t)perm_token[row] * H;                     // moe.py:81
+  for (int h = tid; h < H; h += 256) xs[h] = to_float(xr[h]);
+  __syncthreads();
+  const TIn* wbase = wgu + (size_t)e * 2 * I * H;
+  for (int j = wave; j < 2 * I; j += 4) {                              // moe.py:84
+    const TIn* wrow = wbase + (size_t)j * H;
+    float acc = 0.f;
+    for (int h = lane; h < H; h += kWave) acc = fmaf(xs[h], to_float(wrow[h]), acc);
+    acc = wave_sum(acc);
+    if (lane == 0) gu[j] = acc;
+  }
+  __syncthreads();
+  float ss = 0.f;
+  for (int i = tid; i < I; i += 256) ss = fmaf(gu[i], gu[i], ss);
+  ss = wave_sum(ss);
+  if (lane == 0) red[wave] = ss;
+  __syncthreads();
+  const float ms = ((red[0] + red[1]) + red[2]) + red[3];
+  const float r = sqrtf(ms / (float)I + kNormSiluEps);                 // moe.py:88
+  const float p = 1.f / (1.f + expf(-theta[e]));                       // moe.py:89
+  const float gain = powf(r, p);
+  for (int i = tid; i < I; i += 256) {
+    const float z = gu[i] / r;
+    const float act = z / (1.f + expf(-z)) * gain;                     // SiLU(g/r) * r^p
+    hidden[(size_t)row * I + i] = from_float<TIn>(act * gu[I + i]);    // * up (moe.py:92)
+  }
+}
+
+// yw[slot, :] = w[slot] * (hidden[row, :] @ w_down[e]^T)   (moe.py:92-93)
+template <typename TIn>
+__global__ __launch_bounds__(256) void down_generic_kernel(const TIn* __restrict__ hidden, const TIn* __restrict__ wd,
+                                                           const float* __restrict__ w,
+                                                           const int32_t* __restrict__ offsets,
+                                                           const int32_t* __restrict__ perm_slot, int H, int E, int I,
+                                                           float* __restrict__ yw) {
+  extern __shared__ float smem[];
+  float* hs = smem;            // [I]
+  __shared__ int sh_e;
+  const int row = blockIdx.x;
+  if (row >= offsets[E]) return;
+  const int e = find_expert(offsets, E, row, &sh_e);
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  for (int i = tid; i < I; i += 256) hs[i] = to_float(hidden[(size_t)row * I + i]);
+  __syncthreads();
+  const int slot = perm_slot[row];
+  const float ws = w[slot];
+  const TIn* wbase = wd + (size_t)e * H * I;
+  for (int h = wave; h < H; h += 4) {
+    const TIn* wrow = wbase + (size_t)h * I;
+    float acc = 0.f;
+    for (int i = lane; i < I; i += kWave) acc = fmaf(hs[i], to_float(wrow[i]), acc);
+    acc = wave_sum(acc);
+    if (lane == 0) yw[(size_t)slot * H + h] = ws * acc;
+  }
+}
+
+// out[t, :] = round(sum_j yw[t*k + j, :])  in fp32, ascending j   (moe.py:93,101)
+template <typename TY, typename TOut>
+__global__ __launch_bounds__(256) void combine_kernel(const TY* __restrict__ yw, int T, int H, int k,
+                                                      TOut* __restrict__ out) {
+  const size_t n = (size_t)T * H;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
+    const size_t t = i / H, h = i - t * H;
+    float acc = 0.f;
+    for (int j = 0; j < k; ++j) acc += to_float(yw[(t * k + j) * H + h]);
+    out[i] = from_float<TOut>(acc);
+  }
+}
+
+}  // namespace
+
+hipError_t launch_gateup_generic(const void* x, const void* wgu, const float* theta, const int32_t* offsets,
+                                 const int32_t* perm_token, int T, int H, int E, int k, int I, int dtype, void* hidden,
+                                 hipStream_t s) {
+  const int S = T * k;
+  if (S == 0) return hipSuccess;
+  const size_t shm = (size_t)(H + 2 * I) * sizeof(float);
+  if (dtype == BIBO_DTYPE_BF16)
+    hipLaunchKernelGGL(gateup_generic_kernel<bf16_t>, dim3(S), dim3(256), shm, s, static_cast<const bf16_t*>(x),
+                       static_cast<const bf16_t*>(wgu), theta, offsets, perm_token, H, E, I,
+                       static_cast<bf16_t*>(hidden));
+  else
+    hipLaunchKernelGGL(gateup_generic_kernel<float>, dim3(S), dim3(256), shm, s, static_cast<const float*>(x),
+                       static_cast<const float*>(wgu), theta, offsets, perm_token, H, E, I,
+                       static_cast<float*>(hidden));
+  return hipGetLastError();
+}
+
+hipError_t launch_down_generic(const void* hidden, const void* wd, const float* w, const int32_t* offsets,
+                               const int32_t* perm_slot, int T, int H, int E, int k, int I, int dtype, float* yw,
+                               hipStream_t s) {
+  const int S = T * k;
+  if (S == 0) return hipSuccess;
+  const size_t shm = (size_t)I * sizeof(float);
+  if (dtype == BIBO_DTYPE_BF16)
+    hipLaunchKernelGGL(down_generic_kernel<bf16_t>, dim3(S), dim3(256), shm, s, static_cast<const bf16_t*>(hidden),
+                       static_cast<const bf16_t*>(wd), w, offsets, perm_slot, H, E, I, yw);
+  else
+    hipLaunchKernelGGL(down_generic_kernel<float>, dim3(S), dim3(256), shm, s, static_cast<const float*>(hidden),
+                       static_cast<const float*>(wd), w, offsets, perm_slot, H, E, I, yw);
+  return hipGetLastError();
+}
+
+hipError_t launch_combine(const void* yw, int yw_is_bf16, int T, int H, int k, int dtype, void* out, hipStream_t s) {
+  const size_t n = (size_t)T * H;
+  if (n == 0) return hipSuccess;
+  const int grid = (int)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
+  if (yw_is_bf16) {
+    if (dtype != BIBO_DTYPE_BF16) return hipErrorInvalidValue;
+    hipLaunchKernelGGL((combine_kernel<bf16_t, bf16_t>), dim3(grid), dim3(256), 0, s,
+                       static_cast<const bf16_t*>(yw), T, H, k, static_cast<bf16_t*>(out));
+  } else if (dtype == BIBO_DTYPE_BF16) {
+    hipLaunchKernelGGL((combine_kernel<float, bf16_t>), dim3(grid), dim3(256), 0, s, static_cast<const float*>(yw), T,
+                       H, k, static_cast<bf16_t*>(out));
+  } else {
+    hipLaunchKernelGGL((combine_kernel<float, float>), dim3(grid), dim3(256), 0, s, static_cast<const float*>(yw), T,
+                       H, k, static_cast<float*>(out));
+  }
+  return hipGetLastError();
+}
+
+}  // namespace bibo

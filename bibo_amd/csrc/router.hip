@@ -1,0 +1,224 @@
+// Kernel 1: fused router.  fp32 logits x @ w_router^T, canonical sigmoid, selection on score + bias
+// (ties to the lowest expert index), gather of the unbiased scores, normalisation.
+// Follows BiBoMoERouter.forward, src/modeling/ffn/router.py:25-51 of the reference.
+#include "common.h"
+
+namespace bibo {
+namespace {
+
+constexpr int kRowPad = kMaxE + 1;   // LDS row stride (floats): lane = token reads are conflict-free
+
+// One lane owns one token: scan the E scores in ascending expert order and keep the k best
+// (score + bias) in a sorted register list.  Strict '>' keeps the earlier, i.e. lower-index, expert
+// ahead of an equal later one, which is the tie rule.  Emits experts in ascending index order.
+__device__ __forceinline__ void select_row(const float* __restrict__ sc, const float* __restrict__ bias_s, int E,
+                                           int k, int norm_mode, int32_t* __restrict__ idx_out,
+                                           float* __restrict__ w_out, float* __restrict__ gap_out) {
+  float sel[kMaxK];
+  int id[kMaxK];
+#pragma unroll
+  for (int j = 0; j < kMaxK; ++j) { sel[j] = -INFINITY; id[j] = j; }
+  for (int e = 0; e < E; ++e) {
+    const float v = sc[e] + bias_s[e];                       // router.py:38
+#pragma unroll
+    for (int j = kMaxK - 1; j >= 0; --j) {
+      if (j < k) {
+        const bool gt_prev = (j > 0) && (v > sel[j > 0 ? j - 1 : 0]);
+        if (gt_prev) { sel[j] = sel[j - (j > 0)]; id[j] = id[j - (j > 0)]; }
+        else if (v > sel[j]) { sel[j] = v; id[j] = e; }
+      }
+    }
+  }
+  unsigned long long mask = 0;
+#pragma unroll
+  for (int j = 0; j < kMaxK; ++j)
+    if (j < k) mask |= 1ull << id[j];
+  // ascending expert order; weights are the UNBIASED scores (router.py:41)
+  float raw[kMaxK];
+  float sum = 0.f, mx = -INFINITY;
+  unsigned long long m = mask;
+#pragma unroll
+  for (int j = 0; j < kMaxK; ++j) {
+    raw[j] = 0.f;
+    if (j < k) {
+      const int e = __ffsll((long long)m) - 1;
+      m &= m - 1;
+      idx_out[j] = e;
+      raw[j] = sc[e];
+      sum += raw[j];                                         // sequential fp32 adds, ascending expert
+      mx = fmaxf(mx, raw[j]);
+    }
+  }
+  if (k > 1 && norm_mode == BIBO_NORM_SOFTMAX) {             // router.py:42-43
+    float ex[kMaxK];
+    float es = 0.f;
+#pragma unroll
+    for (int j = 0; j < kMaxK; ++j) { ex[j] = (j < k) ? expf(raw[j] - mx) : 0.f; es += ex[j]; }
+#pragma unroll
+    for (int j = 0; j < kMaxK; ++j) if (j < k) w_out[j] = ex[j] / es;
+  } else if (k > 1 && norm_mode == BIBO_NORM_SUM) {          // router.py:44-45
+    const float den = sum + kSumNormEps;
+#pragma unroll
+    for (int j = 0; j < kMaxK; ++j) if (j < k) w_out[j] = raw[j] / den;
+  } else {                                                   // router.py:46-47
+#pragma unroll
+    for (int j = 0; j < kMaxK; ++j) if (j < k) w_out[j] = raw[j];
+  }
+  if (gap_out != nullptr) {                                  // router.py:33-36, unbiased scores
+    float top[kMaxK + 1];
+#pragma unroll
+    for (int j = 0; j <= kMaxK; ++j) top[j] = -INFINITY;
+    for (int e = 0; e < E; ++e) {
+      const float v = sc[e];
+#pragma unroll
+      for (int j = kMaxK; j >= 0; --j) {
+        if (j <= k) {
+          const bool gt_prev = (j > 0) && (v > top[j > 0 ? j - 1 : 0]);
+          if (gt_prev) top[j] = top[j - (j > 0)];
+          else if (v > top[j]) top[j] = v;
+        }
+      }
+    }
+    float a = 0.f, b = 0.f;
+#pragma unroll
+    for (int j = 0; j <= kMaxK; ++j) { if (j == k - 1) a = top[j]; if (j == k) b = top[j]; }
+    *gap_out = (k < E) ? (a - b) : 0.f;
+  }
+}
+
+// ---- generic router: any H, bf16 or fp32 inputs, plain FMA -------------------------------------
+constexpr int kGenTokens = 64;
+
+template <typename TIn>
+__global__ __launch_bounds__(256) void router_generic_kernel(const TIn* __restrict__ x, const TIn* __restrict__ wr,
+                                                             const float* __restrict__ bias, int T, int H, int E, int k,
+                                                             int norm_mode, float* __restrict__ logits,
+                                                             int32_t* __restrict__ idx, float* __restrict__ w,
+                                                             float* __restrict__ gap) {
+  __shared__ float sc[kGenTokens * kRowPad];
+  __shared__ float bias_s[kMaxE];
+  const int tid = threadIdx.x;
+  const int t0 = blockIdx.x * kGenTokens;
+  if (tid < kMaxE) bias_s[tid] = (tid < E) ? bias[tid] : 0.f;
+  {
+    const int tl = tid >> 2, q = tid & 3;
+    const int t = min(t0 + tl, T - 1);
+    float acc[kMaxE / 4];
+#pragma unroll
+    for (int j = 0; j < kMaxE / 4; ++j) acc[j] = 0.f;
+    const TIn* xr = x + (size_t)t * H;
+    for (int h = 0; h < H; ++h) {
+      const float xv = to_float(xr[h]);
+#pragma unroll
+      for (int j = 0; j < kMaxE / 4; ++j) {
+        const int e = q + 4 * j;
+        if (e < E) acc[j] = fmaf(xv, to_float(wr[(size_t)e * H + h]), acc[j]);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < kMaxE / 4; ++j) {
+      const int e = q + 4 * j;
+      if (e < E) sc[tl * kRowPad + e] = acc[j];
+    }
+  }
+  __syncthreads();
+  const int ntok = min(kGenTokens, T - t0);
+  for (int i = tid; i < ntok * E; i += 256) {
+    const int tl = i / E, e = i - tl * E;
+    const float lg = sc[tl * kRowPad + e];
+    if (logits != nullptr) logits[(size_t)(t0 + tl) * E + e] = lg;
+    sc[tl * kRowPad + e] = sigmoid32_canonical(lg);          // router.py:31
+  }
+  __syncthreads();
+  if (tid < ntok) {
+    const int t = t0 + tid;
+    select_row(sc + tid * kRowPad, bias_s, E, k, norm_mode, idx + (size_t)t * k, w + (size_t)t * k,
+               gap ? gap + t : nullptr);
+  }
+}
+
+// ---- MFMA router: bf16, H % 32 == 0 -------------------------------------------------------------
+// One workgroup = 16 tokens, 4 waves.  The waves split K (32-wide steps round-robin); each keeps
+// four 16x16 fp32 accumulators (64 experts), partials are summed through LDS in wave order.
+constexpr int kMfmaTokens = 16;
+
+__global__ __launch_bounds__(256) void router_mfma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wr,
+                                                          const float* __restrict__ bias, int T, int H, int E, int k,
+                                                          int norm_mode, float* __restrict__ logits,
+                                                          int32_t* __restrict__ idx, float* __restrict__ w,
+                                                          float* __restrict__ gap) {
+  __shared__ float part[4 * kMfmaTokens * kRowPad];
+  __shared__ float sc[kMfmaTokens * kRowPad];
+  __shared__ float bias_s[kMaxE];
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63;
+  const int t0 = blockIdx.x * kMfmaTokens;
+  if (tid < kMaxE) bias_s[tid] = (tid < E) ? bias[tid] : 0.f;
+
+  const int r16 = lane & 15, kc = lane >> 4;                 // fragment row, 8-wide k chunk
+  const bf16_t* xa = x + (size_t)min(t0 + r16, T - 1) * H + kc * 8;
+  const bf16_t* wb[4];
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt) wb[nt] = wr + (size_t)min(nt * 16 + r16, E - 1) * H + kc * 8;
+  floatx4 acc[4];
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt) acc[nt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  const int nsteps = H / 32;
+  for (int s = wave; s < nsteps; s += 4) {
+    const int k0 = s * 32;
+    const bf16x8 a = *reinterpret_cast<const bf16x8*>(xa + k0);
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+      const bf16x8 b = *reinterpret_cast<const bf16x8*>(wb[nt] + k0);
+      acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[nt], 0, 0, 0);
+    }
+  }
+  // D layout of the 16x16 tile: lane holds column (expert) lane%16, rows (tokens) 4*(lane/16)+i
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      part[(wave * kMfmaTokens + kc * 4 + i) * kRowPad + nt * 16 + r16] = acc[nt][i];
+  __syncthreads();
+  const int ntok = min(kMfmaTokens, T - t0);
+  for (int i = tid; i < kMfmaTokens * kMaxE; i += 256) {
+    const int tl = i >> 6, e = i & 63;
+    if (tl < ntok && e < E) {
+      const int o = tl * kRowPad + e;
+      const float lg = ((part[o] + part[kMfmaTokens * kRowPad + o]) + part[2 * kMfmaTokens * kRowPad + o]) +
+                       part[3 * kMfmaTokens * kRowPad + o];
+      if (logits != nullptr) logits[(size_t)(t0 + tl) * E + e] = lg;
+      sc[o] = sigmoid32_canonical(lg);                       // router.py:31
+    }
+  }
+  __syncthreads();
+  if (tid < ntok) {
+    const int t = t0 + tid;
+    select_row(sc + tid * kRowPad, bias_s, E, k, norm_mode, idx + (size_t)t * k, w + (size_t)t * k,
+               gap ? gap + t : nullptr);
+  }
+}
+
+}  // namespace
+
+hipError_t launch_router(const void* x, const void* w_router, const float* bias, int T, int H, int E, int k, int dtype,
+                         int norm_mode, float* logits, int32_t* idx, float* w, float* gap, hipStream_t s) {
+  if (T == 0) return hipSuccess;
+  const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w_router)) & 15) == 0;
+  if (dtype == BIBO_DTYPE_BF16 && (H % 32) == 0 && aligned) {
+    const int grid = (T + kMfmaTokens - 1) / kMfmaTokens;
+    hipLaunchKernelGGL(router_mfma_kernel, dim3(grid), dim3(256), 0, s, static_cast<const bf16_t*>(x),
+                       static_cast<const bf16_t*>(w_router), bias, T, H, E, k, norm_mode, logits, idx, w, gap);
+  } else {
+    const int grid = (T + kGenTokens - 1) / kGenTokens;
+    if (dtype == BIBO_DTYPE_BF16)
+      hipLaunchKernelGGL(router_generic_kernel<bf16_t>, dim3(grid), dim3(256), 0, s, static_cast<const bf16_t*>(x),
+                         static_cast<const bf16_t*>(w_router), bias, T, H, E, k, norm_mode, logits, idx, w, gap);
+    else
+      hipLaunchKernelGGL(router_generic_kernel<float>, dim3(grid), dim3(256), 0, s, static_cast<const float*>(x),
+                         static_cast<const float*>(w_router), bias, T, H, E, k, norm_mode, logits, idx, w, gap);
+  }
+  return hipGetLastError();
+}
+
+}  // namespace bibo

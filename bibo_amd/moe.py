@@ -1,0 +1,238 @@
+"""Drop-in modules for the reference's sparse-MoE block, running on the HIP kernels of libbibo_moe.so.
+
+Class names, constructor argument, attribute names, parameter shapes and state_dict keys follow
+src/modeling/ffn/router.py and src/modeling/ffn/moe.py of the reference, so a reference checkpoint
+loads with strict=True and code that pokes at `layer.gate.bias` or `layer.experts.radial_theta`
+keeps working.  Forward only: outputs carry no autograd graph."""
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+
+from . import _lib as L
+from . import ops
+
+__all__ = ["BiBoMoERouter", "BiBoFusedExperts", "BiBoMoELayer"]
+
+try:
+    _no_compile = torch.compiler.disable
+except AttributeError:                                    # older torch
+    _no_compile = torch._dynamo.disable
+
+
+def _forward_only_guard(*tensors):
+    if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors):
+        raise RuntimeError(
+            "bibo_amd implements the forward pass only; call it under torch.no_grad() or torch.inference_mode() "
+            "(an input or parameter requires grad and autograd is enabled, so gradients would silently be lost)")
+
+
+class _CastCache:
+    """Device copies of parameters in the dtype the kernels want, refreshed when the parameter changes."""
+
+    def __init__(self):
+        self._store = {}
+
+    def get(self, name: str, p: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+        if p.dtype == dtype and p.is_contiguous():
+            return p.detach()
+        key = (name, dtype)
+        tag = (p.data_ptr(), p._version, p.device, p.dtype)
+        hit = self._store.get(key)
+        if hit is None or hit[0] != tag:
+            hit = (tag, p.detach().to(dtype).contiguous())
+            self._store[key] = hit
+        return hit[1]
+
+
+def _compute_dtype(x: torch.Tensor) -> torch.dtype:
+    """bf16 activations, or fp32 activations under bf16 autocast, run the bf16 kernels; plain fp32 runs the
+    fp32 generic kernels (the regimes of ablate/common/train.py:589,677 and tests/test_moe.py:252-259)."""
+    if x.dtype == torch.bfloat16:
+        return torch.bfloat16
+    if x.dtype == torch.float32:
+        if torch.is_autocast_enabled() and torch.get_autocast_gpu_dtype() == torch.bfloat16:
+            return torch.bfloat16
+        return torch.float32
+    raise TypeError(f"hidden states must be bfloat16 or float32, got {x.dtype}")
+
+
+class BiBoMoERouter(nn.Module):
+    """Sigmoid router with a non-grad selection bias (src/modeling/ffn/router.py:10-51)."""
+
+    def __init__(self, config):
+        super().__init__()
+        self.num_routed_experts = config.num_routed_experts
+        self.top_k = config.num_experts_per_tok
+        self.norm_topk_prob = config.norm_topk_prob
+        if self.num_routed_experts > L.MAX_EXPERTS or self.top_k > L.MAX_TOPK:
+            raise NotImplementedError(f"the HIP router supports at most {L.MAX_EXPERTS} experts and top-{L.MAX_TOPK}")
+        self.bias = nn.Parameter(torch.zeros(self.num_routed_experts), requires_grad=False)
+        self._probe_gap = False
+        self.boundary_gap = None
+        self.gate_proj = nn.Linear(config.hidden_size, self.num_routed_experts, bias=False)
+        nn.init.normal_(self.gate_proj.weight, mean=0.0, std=getattr(config, "initializer_range", 0.02))
+        self._cache = _CastCache()
+
+    def _operands(self, hidden_states):
+        cd = _compute_dtype(hidden_states)
+        x = hidden_states.detach().reshape(-1, hidden_states.shape[-1])
+        x = x.to(cd) if x.dtype != cd else x
+        return (x.contiguous(), self._cache.get("w", self.gate_proj.weight, cd),
+                self._cache.get("b", self.bias, torch.float32))
+
+    @_no_compile
+    def router_logits(self, hidden_states: torch.Tensor) -> torch.Tensor:
+        """fp32 logits [B*S, E] (router.py:25-26); kept in fp32, never rounded to the model dtype."""
+        x, w, b = self._operands(hidden_states)
+        return ops.router_fwd(x, w, b, self.top_k, self.norm_topk_prob, want_logits=True)[2]
+
+    @_no_compile
+    def forward(self, hidden_states: torch.Tensor):
+        _forward_only_guard(hidden_states, self.gate_proj.weight)
+        bsz, seq, _ = hidden_states.shape
+        x, w, b = self._operands(hidden_states)
+        probe = self._probe_gap and self.top_k < self.num_routed_experts
+        idx, wgt, _, gap = ops.router_fwd(x, w, b, self.top_k, self.norm_topk_prob, want_gap=probe)
+        if probe:
+            self.boundary_gap = gap.mean()                                   # router.py:33-36
+        return idx.view(bsz, seq, -1).long(), wgt.view(bsz, seq, -1)
+
+
+class BiBoFusedExperts(nn.Module):
+    """Stacked GLU experts with the Radial NormSiLU activation (src/modeling/ffn/moe.py:19-101)."""
+
+    def __init__(self, config):
+        super().__init__()
+        self.num_glu_experts = config.num_glu_experts
+        self.special_expert_pairs = config.special_expert_pairs
+        self.num_routed_experts = config.num_routed_experts
+        self.hidden_size = config.hidden_size
+        self.intermediate_size = config.moe_intermediate_size
+        num_pos = getattr(config, "num_pos_identity_experts", self.special_expert_pairs)
+        num_neg = getattr(config, "num_neg_identity_experts", self.special_expert_pairs)
+        self.pos_start = self.num_glu_experts
+        self.pos_end = self.pos_start + num_pos
+        self.neg_start = self.pos_end
+        self.neg_end = self.neg_start + num_neg
+        if self.num_glu_experts != self.num_routed_experts:
+            raise NotImplementedError(
+                "+/-Identity special experts are not implemented by the HIP kernels: configure "
+                "special_expert_pairs=0 (num_glu_experts must equal num_routed_experts)")
+        if self.num_routed_experts > L.MAX_EXPERTS:
+            raise NotImplementedError(f"the HIP kernels support at most {L.MAX_EXPERTS} experts")
+        std = getattr(config, "initializer_range", 0.02)
+        self.gate_up_proj = nn.Parameter(torch.empty(self.num_glu_experts, 2 * self.intermediate_size, self.hidden_size))
+        self.down_proj = nn.Parameter(torch.empty(self.num_glu_experts, self.hidden_size, self.intermediate_size))
+        nn.init.normal_(self.gate_up_proj, mean=0.0, std=std)
+        nn.init.normal_(self.down_proj, mean=0.0, std=std)
+        self.radial_theta = nn.Parameter(torch.zeros(self.num_glu_experts))
+        self.algo = "auto"
+        self._cache = _CastCache()
+
+    def _weights(self, cd):
+        return (self._cache.get("gu", self.gate_up_proj, cd), self._cache.get("dn", self.down_proj, cd),
+                self._cache.get("th", self.radial_theta, torch.float32))
+
+    @_no_compile
+    def forward(self, hidden_states: torch.Tensor, top_k_indices: torch.Tensor, top_k_weights: torch.Tensor,
+                _want_counts: bool = False):
+        _forward_only_guard(hidden_states, top_k_weights, self.gate_up_proj)
+        cd = _compute_dtype(hidden_states)
+        x = hidden_states.detach()
+        x = (x.to(cd) if x.dtype != cd else x).contiguous()
+        idx = top_k_indices.detach().to(torch.int32).contiguous()
+        w = top_k_weights.detach().to(torch.float32).contiguous()
+        gu, dn, th = self._weights(cd)
+        out, counts = ops.experts_fwd(x, idx, w, gu, dn, th, algo=self.algo, want_counts=_want_counts)
+        out = out if out.dtype == hidden_states.dtype else out.to(hidden_states.dtype)   # moe.py:101
+        return (out, counts) if _want_counts else out
+
+
+class BiBoMoELayer(nn.Module):
+    """Router + experts + balancing state (src/modeling/ffn/moe.py:104-183)."""
+
+    def __init__(self, config):
+        super().__init__()
+        self.hidden_size = config.hidden_size
+        self.num_routed_experts = config.num_routed_experts
+        self.num_experts_per_tok = config.num_experts_per_tok
+        self.bias_update_factor = config.bias_update_factor
+        self.bias_update_threshold = config.bias_update_threshold
+        self.register_buffer("accumulated_tpe", torch.zeros(config.num_routed_experts, dtype=torch.float))
+        self._fwd_step = 0
+        self._update_every = None
+        self.experts = BiBoFusedExperts(config)
+        self.use_shared_expert = getattr(config, "use_shared_expert", False)
+        self.shared_experts_list = nn.ModuleList()
+        if self.use_shared_expert:
+            raise NotImplementedError("use_shared_expert=True is not implemented by the HIP MoE layer")
+        self.gate = BiBoMoERouter(config)
+
+    # ---- balancing (host logic over device tensors, moe.py:131-155) ----
+    @torch.no_grad()
+    def update_bias(self, tokens_per_expert: torch.Tensor):
+        u = self.bias_update_factor
+        if u <= 0:
+            return
+        load = tokens_per_expert.detach().float()
+        load = load / load.sum().clamp_min(1.0)
+        self.gate.bias.add_(u * (load.mean() - load))        # proportional step; deviations sum to zero
+
+    @_no_compile
+    @torch.no_grad()
+    def _balance_step(self, top_k_indices, num_tokens, counts=None):
+        """Accumulate this forward's per-expert token counts; every `_update_every` forwards hand the
+        accumulated vector back (all-reduced across ranks when a process group exists) and reset it.
+        `counts` lets the caller pass the histogram the permutation kernel already produced."""
+        if counts is None:
+            counts = torch.bincount(top_k_indices.reshape(-1), minlength=self.num_routed_experts)
+        self.accumulated_tpe += counts.to(self.accumulated_tpe.dtype)
+        if self._update_every is None:
+            self._update_every = max(1, round(self.bias_update_threshold / max(num_tokens, 1)))
+        self._fwd_step += 1
+        if self._fwd_step % self._update_every != 0:
+            return None
+        import torch.distributed as dist
+        if dist.is_available() and dist.is_initialized():
+            dist.all_reduce(self.accumulated_tpe, op=dist.ReduceOp.SUM)
+        tpe = self.accumulated_tpe.clone()
+        self.accumulated_tpe.zero_()
+        return tpe
+
+    def _hooks_present(self) -> bool:
+        g, e = self.gate, self.experts
+        return bool(g._forward_hooks or g._forward_pre_hooks or e._forward_hooks or e._forward_pre_hooks
+                    or g._probe_gap or nn.modules.module._global_forward_hooks
+                    or nn.modules.module._global_forward_pre_hooks)
+
+    @_no_compile
+    def forward(self, hidden_states: torch.Tensor) -> torch.Tensor:
+        bsz, seq, hdim = hidden_states.shape
+        num_tokens = bsz * seq
+        balancing = self.training and self.bias_update_factor > 0
+        if self._hooks_present():
+            # module-by-module, so hooks on `gate` and `experts` observe exactly what the reference's
+            # would (ablate/common/router_trace.py hooks both)
+            top_idx, top_w = self.gate(hidden_states)
+            res = self.experts(hidden_states.reshape(num_tokens, hdim), top_idx.view(num_tokens, -1),
+                               top_w.view(num_tokens, -1), _want_counts=balancing)
+            out, counts = res if balancing else (res, None)
+        else:
+            _forward_only_guard(hidden_states, self.gate.gate_proj.weight, self.experts.gate_up_proj)
+            cd = _compute_dtype(hidden_states)
+            x = hidden_states.detach().reshape(num_tokens, hdim)
+            x = (x.to(cd) if x.dtype != cd else x).contiguous()
+            gu, dn, th = self.experts._weights(cd)
+            wr = self.gate._cache.get("w", self.gate.gate_proj.weight, cd)
+            b = self.gate._cache.get("b", self.gate.bias, torch.float32)
+            out, _, _, counts, _ = ops.moe_forward(x, wr, b, gu, dn, th, self.num_experts_per_tok,
+                                                   norm=self.gate.norm_topk_prob, algo=self.experts.algo,
+                                                   want_counts=balancing)
+            out = out if out.dtype == hidden_states.dtype else out.to(hidden_states.dtype)
+            top_idx = None
+        if balancing:                                          # exactly once per training forward
+            tpe = self._balance_step(top_idx, num_tokens, counts=counts)
+            if tpe is not None:
+                self.update_bias(tpe)
+        return out.view(bsz, seq, hdim)

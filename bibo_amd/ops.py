@@ -1,0 +1,188 @@
+"""Tensor-level wrappers over the C ABI: torch supplies device memory and the stream, nothing else."""
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from . import _lib as L
+
+_NORM = {"sum": L.NORM_SUM, True: L.NORM_SUM, "softmax": L.NORM_SOFTMAX, False: L.NORM_NONE, None: L.NORM_NONE}
+_ALGO = {"auto": L.ALGO_AUTO, "generic": L.ALGO_GENERIC, "mfma": L.ALGO_MFMA, "stream": L.ALGO_STREAM}
+
+
+def norm_mode(v) -> int:
+    if isinstance(v, str) or isinstance(v, bool) or v is None:
+        if v in _NORM:
+            return _NORM[v]
+    raise ValueError(f"norm_topk_prob must be 'sum', 'softmax' or False, got {v!r}")
+
+
+def algo_code(v) -> int:
+    if isinstance(v, int):
+        return v
+    return _ALGO[v]
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    if t.dtype == torch.bfloat16:
+        return L.DTYPE_BF16
+    if t.dtype == torch.float32:
+        return L.DTYPE_F32
+    raise TypeError(f"hidden states and weights must be bfloat16 or float32, got {t.dtype}")
+
+
+def _chk(t: torch.Tensor, name: str, dtype=None, shape=None):
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must live on the GPU (got {t.device}); bibo_amd has no CPU path")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")   # a strided view would be silently misread
+    if dtype is not None and t.dtype != dtype:
+        raise TypeError(f"{name} must be {dtype}, got {t.dtype}")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise ValueError(f"{name} must have shape {tuple(shape)}, got {tuple(t.shape)}")
+    return t
+
+
+def _ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream(dev) -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+
+_workspaces: dict = {}
+
+
+def workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
+    """A grow-only byte buffer per (device, stream): calls on one stream are ordered, so they may share it."""
+    key = (dev.index, torch.cuda.current_stream(dev).cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=dev)
+        _workspaces[key] = ws
+    return ws
+
+
+def workspace_bytes(T, H, E, k, I, dtype_code) -> int:
+    sh = L.Shape(T, H, E, k, I, dtype_code)
+    out = ctypes.c_size_t(0)
+    L.check(L.lib().bibo_moe_workspace_bytes(ctypes.byref(sh), ctypes.byref(out)), "bibo_moe_workspace_bytes")
+    return out.value
+
+
+def router_fwd(x, w_router, bias, k, norm="sum", want_logits=False, want_gap=False):
+    """x [T,H], w_router [E,H], bias fp32 [E] -> idx int32 [T,k], w fp32 [T,k], logits fp32 [T,E]|None, gap fp32 [T]|None."""
+    T, H = x.shape
+    E = w_router.shape[0]
+    dc = _dtype_code(x)
+    _chk(x, "x"); _chk(w_router, "w_router", x.dtype, (E, H)); _chk(bias, "bias", torch.float32, (E,))
+    dev = x.device
+    idx = torch.empty(T, k, dtype=torch.int32, device=dev)
+    w = torch.empty(T, k, dtype=torch.float32, device=dev)
+    logits = torch.empty(T, E, dtype=torch.float32, device=dev) if want_logits else None
+    gap = torch.empty(T, dtype=torch.float32, device=dev) if want_gap else None
+    with torch.cuda.device(dev):
+        L.check(L.lib().bibo_moe_router_fwd(_ptr(x), _ptr(w_router), _ptr(bias), T, H, E, k, dc, norm_mode(norm),
+                                            _ptr(logits), _ptr(idx), _ptr(w), _ptr(gap), _stream(dev)),
+                "bibo_moe_router_fwd")
+    return idx, w, logits, gap
+
+
+def permute(idx, E):
+    """idx int32 [T,k] -> counts [E], offsets [E+1], perm_slot [T*k], perm_token [T*k] (all int32)."""
+    T, k = idx.shape
+    _chk(idx, "idx", torch.int32)
+    dev = idx.device
+    counts = torch.empty(E, dtype=torch.int32, device=dev)
+    offsets = torch.empty(E + 1, dtype=torch.int32, device=dev)
+    perm_slot = torch.empty(T * k, dtype=torch.int32, device=dev)
+    perm_token = torch.empty(T * k, dtype=torch.int32, device=dev)
+    nb = max(1, (T + 63) // 64) * 64 * 4
+    ws = workspace(dev, nb)
+    with torch.cuda.device(dev):
+        L.check(L.lib().bibo_moe_permute(_ptr(idx), T, E, k, _ptr(counts), _ptr(offsets), _ptr(perm_slot),
+                                         _ptr(perm_token), _ptr(ws), ws.numel(), _stream(dev)), "bibo_moe_permute")
+    return counts, offsets, perm_slot, perm_token
+
+
+def gateup_fwd(x, w_gate_up, theta, offsets, perm_token, k, algo="auto"):
+    """-> hidden [T*k, I] in x.dtype, rows in permuted order."""
+    T, H = x.shape
+    E, two_i, _ = w_gate_up.shape
+    I = two_i // 2
+    dc = _dtype_code(x)
+    _chk(x, "x"); _chk(w_gate_up, "w_gate_up", x.dtype, (E, 2 * I, H)); _chk(theta, "theta", torch.float32, (E,))
+    _chk(offsets, "offsets", torch.int32, (E + 1,)); _chk(perm_token, "perm_token", torch.int32, (T * k,))
+    hidden = torch.empty(T * k, I, dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        L.check(L.lib().bibo_moe_gateup_fwd(_ptr(x), _ptr(w_gate_up), _ptr(theta), _ptr(offsets), _ptr(perm_token),
+                                            T, H, E, k, I, dc, algo_code(algo), _ptr(hidden), _stream(x.device)),
+                "bibo_moe_gateup_fwd")
+    return hidden
+
+
+def down_combine_fwd(hidden, w_down, w, offsets, perm_slot, T, algo="auto"):
+    """-> out [T,H] in hidden.dtype."""
+    E, H, I = w_down.shape
+    k = w.shape[1]
+    dc = _dtype_code(hidden)
+    _chk(hidden, "hidden", None, (T * k, I)); _chk(w_down, "w_down", hidden.dtype); _chk(w, "w", torch.float32, (T, k))
+    _chk(offsets, "offsets", torch.int32, (E + 1,)); _chk(perm_slot, "perm_slot", torch.int32, (T * k,))
+    dev = hidden.device
+    out = torch.empty(T, H, dtype=hidden.dtype, device=dev)
+    ws = workspace(dev, T * k * H * 4)
+    with torch.cuda.device(dev):
+        L.check(L.lib().bibo_moe_down_combine_fwd(_ptr(hidden), _ptr(w_down), _ptr(w), _ptr(offsets), _ptr(perm_slot),
+                                                  T, H, E, k, I, dc, algo_code(algo), _ptr(out), _ptr(ws), ws.numel(),
+                                                  _stream(dev)), "bibo_moe_down_combine_fwd")
+    return out
+
+
+def experts_fwd(x, idx, w, w_gate_up, w_down, theta, algo="auto", want_counts=False):
+    """Seam 2.  x [T,H]; idx int32 [T,k]; w fp32 [T,k] -> out [T,H] (x.dtype), counts int32 [E]|None."""
+    T, H = x.shape
+    E, two_i, _ = w_gate_up.shape
+    I = two_i // 2
+    k = idx.shape[1]
+    dc = _dtype_code(x)
+    _chk(x, "x"); _chk(idx, "idx", torch.int32, (T, k)); _chk(w, "w", torch.float32, (T, k))
+    _chk(w_gate_up, "w_gate_up", x.dtype, (E, 2 * I, H)); _chk(w_down, "w_down", x.dtype, (E, H, I))
+    _chk(theta, "theta", torch.float32, (E,))
+    dev = x.device
+    out = torch.empty(T, H, dtype=x.dtype, device=dev)
+    counts = torch.empty(E, dtype=torch.int32, device=dev) if want_counts else None
+    ws = workspace(dev, workspace_bytes(T, H, E, k, I, dc))
+    sh = L.Shape(T, H, E, k, I, dc)
+    with torch.cuda.device(dev):
+        L.check(L.lib().bibo_moe_experts_fwd(_ptr(x), _ptr(idx), _ptr(w), _ptr(w_gate_up), _ptr(w_down), _ptr(theta),
+                                             ctypes.byref(sh), algo_code(algo), _ptr(out), _ptr(counts), _ptr(ws),
+                                             ws.numel(), _stream(dev)), "bibo_moe_experts_fwd")
+    return out, counts
+
+
+def moe_forward(x, w_router, bias, w_gate_up, w_down, theta, k, norm="sum", algo="auto", want_routing=False,
+                want_counts=False, want_logits=False):
+    """Seam 1.  -> out [T,H], idx int32 [T,k]|None, w fp32 [T,k]|None, counts int32 [E]|None, logits fp32 [T,E]|None."""
+    T, H = x.shape
+    E, two_i, _ = w_gate_up.shape
+    I = two_i // 2
+    dc = _dtype_code(x)
+    _chk(x, "x"); _chk(w_router, "w_router", x.dtype, (E, H)); _chk(bias, "bias", torch.float32, (E,))
+    _chk(w_gate_up, "w_gate_up", x.dtype, (E, 2 * I, H)); _chk(w_down, "w_down", x.dtype, (E, H, I))
+    _chk(theta, "theta", torch.float32, (E,))
+    dev = x.device
+    out = torch.empty(T, H, dtype=x.dtype, device=dev)
+    idx = torch.empty(T, k, dtype=torch.int32, device=dev) if want_routing else None
+    w = torch.empty(T, k, dtype=torch.float32, device=dev) if want_routing else None
+    counts = torch.empty(E, dtype=torch.int32, device=dev) if want_counts else None
+    logits = torch.empty(T, E, dtype=torch.float32, device=dev) if want_logits else None
+    ws = workspace(dev, workspace_bytes(T, H, E, k, I, dc))
+    sh = L.Shape(T, H, E, k, I, dc)
+    with torch.cuda.device(dev):
+        L.check(L.lib().bibo_moe_forward(_ptr(x), _ptr(w_router), _ptr(bias), _ptr(w_gate_up), _ptr(w_down),
+                                         _ptr(theta), ctypes.byref(sh), norm_mode(norm), algo_code(algo), _ptr(out),
+                                         _ptr(idx), _ptr(w), _ptr(counts), _ptr(logits), _ptr(ws), ws.numel(),
+                                         _stream(dev)), "bibo_moe_forward")
+    return out, idx, w, counts, logits

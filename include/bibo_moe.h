@@ -1,0 +1,152 @@
+/*
+ * bibo_moe.h -- C ABI of the MI355X (gfx950) implementation of BiBo's sparse-MoE feed-forward block.
+ *
+ * The reference (IsNoobgrammer/BiBo) is pure Python; the interfaces below are what a binding for its
+ * three nested seams would call.  Citations are paths inside the reference repository.
+ *
+ *   seam 1  BiBoMoELayer.forward(hidden[B,S,H]) -> [B,S,H]            src/modeling/ffn/moe.py:157-183
+ *   seam 2  BiBoFusedExperts.forward(x[N,H], idx[N,k], w[N,k]) -> [N,H] src/modeling/ffn/moe.py:46-101
+ *           (the method ablate/common/patches.py:157-180 rebinds to an external fused kernel)
+ *   router  BiBoMoERouter.forward(hidden) -> (idx, w)                  src/modeling/ffn/router.py:28-51
+ *
+ * Conventions
+ *   - Every pointer is a DEVICE pointer on the current HIP device unless stated otherwise.  The caller
+ *     allocates inputs, outputs and the workspace; the library allocates nothing, keeps no pointer
+ *     after a call returns and has no mutable global state.
+ *   - All tensors are dense row-major ("contiguous"); weights are consumed as the reference stores
+ *     them: w_router [E,H], w_gate_up [E,2I,H] (rows 0..I-1 gate, I..2I-1 up), w_down [E,H,I].
+ *   - `dtype` selects the element type of hidden states and the three weight tensors
+ *     (BIBO_DTYPE_BF16 or BIBO_DTYPE_F32).  bias, theta, logits and routing weights are always fp32;
+ *     expert indices are int32.
+ *   - `stream` is a hipStream_t passed as void*; every call is stream-ordered and asynchronous and
+ *     never synchronises the host.
+ *   - Return value: 0 success; negative = argument error detected on the host before anything was
+ *     launched (see BIBO_ERR_*); positive = hipError_t reported by a launch.
+ *   - Limits: 1 <= E <= 64, 1 <= k <= min(E, 8).
+ *   - Canonical orders (the reference leaves both implementation-defined): the k experts of a token
+ *     are emitted in ascending expert index with top-k ties going to the lowest index; routed slots
+ *     are ordered by (expert, token, slot) ascending, i.e. a stable sort of slot ids by expert.
+ */
+#ifndef BIBO_MOE_H
+#define BIBO_MOE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define BIBO_MOE_ABI_VERSION 1
+#define BIBO_MOE_MAX_EXPERTS 64
+#define BIBO_MOE_MAX_TOPK 8
+
+enum bibo_dtype { BIBO_DTYPE_BF16 = 0, BIBO_DTYPE_F32 = 1 };
+
+/* norm_topk_prob of the reference router (src/modeling/ffn/router.py:42-47) */
+enum bibo_norm_mode { BIBO_NORM_NONE = 0, BIBO_NORM_SUM = 1, BIBO_NORM_SOFTMAX = 2 };
+
+/* kernel family for the expert GEMMs */
+enum bibo_algo {
+  BIBO_ALGO_AUTO = 0,    /* pick by shape */
+  BIBO_ALGO_GENERIC = 1, /* one workgroup per routed row, any H and I, bf16 or fp32 */
+  BIBO_ALGO_MFMA = 2,    /* grouped bf16 MFMA tiles; needs H % 32 == 0 and I in {128,256,384,512} */
+  BIBO_ALGO_STREAM = 3   /* weight-streaming kernels for few rows per expert (decode) */
+};
+
+enum bibo_error {
+  BIBO_OK = 0,
+  BIBO_ERR_NULL_POINTER = -1,
+  BIBO_ERR_BAD_SHAPE = -2,
+  BIBO_ERR_BAD_DTYPE = -3,
+  BIBO_ERR_WORKSPACE_TOO_SMALL = -4,
+  BIBO_ERR_MISALIGNED = -5,
+  BIBO_ERR_UNSUPPORTED = -6
+};
+
+typedef struct bibo_moe_shape {
+  int32_t T; /* tokens = B*S */
+  int32_t H; /* hidden size */
+  int32_t E; /* routed experts (all GLU) */
+  int32_t k; /* experts per token */
+  int32_t I; /* expert intermediate size */
+  int32_t dtype;
+} bibo_moe_shape;
+
+int bibo_moe_abi_version(void);
+
+/* Static, NUL-terminated description of a negative code; for positive codes the HIP error string. */
+const char* bibo_moe_strerror(int code);
+
+/* Bytes of workspace that any entry point below needs for this shape (256-byte aligned base). */
+int bibo_moe_workspace_bytes(const bibo_moe_shape* shape, size_t* bytes);
+
+/*
+ * Router: fp32 logits, sigmoid scores, selection on scores+bias, gather of the unbiased scores and
+ * normalisation.  Replaces BiBoMoERouter.forward (src/modeling/ffn/router.py:28-51) and the external
+ * fused router the reference once bound (legacy/bench/exp_kappa.py:142-155).
+ *   x [T,H], w_router [E,H], bias fp32 [E]
+ *   logits  fp32 [T,E]  optional (may be NULL)
+ *   idx     int32 [T,k] ascending expert index
+ *   w       fp32 [T,k]
+ *   gap     fp32 [T]    optional: score_k - score_{k+1} on unbiased scores (router.py:33-36)
+ */
+int bibo_moe_router_fwd(const void* x, const void* w_router, const float* bias, int T, int H, int E, int k,
+                        int dtype, int norm_mode, float* logits, int32_t* idx, float* w, float* gap,
+                        void* stream);
+
+/*
+ * Histogram, prefix sum and stable permutation of the T*k routed slots by expert.  Replaces the
+ * sort / bincount / cumsum / .tolist() prologue of BiBoFusedExperts.forward (moe.py:56-68) and the
+ * bincount of BiBoMoELayer._balance_step (moe.py:141-145).
+ *   idx int32 [T,k]; counts int32 [E]; offsets int32 [E+1]; perm_slot, perm_token int32 [T*k]
+ * Indices outside [0,E) are ignored (their slots get no row and offsets[E] < T*k).
+ */
+int bibo_moe_permute(const int32_t* idx, int T, int E, int k, int32_t* counts, int32_t* offsets,
+                     int32_t* perm_slot, int32_t* perm_token, void* workspace, size_t workspace_bytes,
+                     void* stream);
+
+/*
+ * Grouped gate/up projection with the Radial NormSiLU epilogue r^p * SiLU(g/r) * up,
+ * r = sqrt(mean_I(g^2) + 1e-6), p = sigmoid(theta[e]).  Replaces moe.py:81-90 and the
+ * `activated * up` of moe.py:92.
+ *   hidden  [T*k, I] in `dtype`, rows in permuted (sorted-by-expert) order
+ */
+int bibo_moe_gateup_fwd(const void* x, const void* w_gate_up, const float* theta, const int32_t* offsets,
+                        const int32_t* perm_token, int T, int H, int E, int k, int I, int dtype, int algo,
+                        void* hidden, void* stream);
+
+/*
+ * Grouped down projection; the epilogue scales each row by its routing weight and scatters it back to
+ * token order, where the k rows of a token are summed in fp32 and rounded once to `dtype`.
+ * Replaces the F.linear(..., down_proj) of moe.py:92, moe.py:93 and the cast of moe.py:101.
+ *   hidden [T*k, I] permuted order; w fp32 [T,k]; out [T,H] in `dtype`
+ */
+int bibo_moe_down_combine_fwd(const void* hidden, const void* w_down, const float* w, const int32_t* offsets,
+                              const int32_t* perm_slot, int T, int H, int E, int k, int I, int dtype, int algo,
+                              void* out, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Seam 2: BiBoFusedExperts.forward(x, idx, w) (moe.py:46-101; the signature of the external
+ * moe_per_expert bound at ablate/common/patches.py:165-166).  idx int32 [T,k], w fp32 [T,k], out [T,H].
+ * counts_out int32 [E] optional.
+ */
+int bibo_moe_experts_fwd(const void* x, const int32_t* idx, const float* w, const void* w_gate_up,
+                         const void* w_down, const float* theta, const bibo_moe_shape* shape, int algo,
+                         void* out, int32_t* counts_out, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Seam 1: the whole layer, router included (moe.py:157-183 in eval mode; the contract of the external
+ * megakernel_block minus the RMSNorm, ablate/common/patches.py:255-258).
+ * Optional outputs (may be NULL): idx_out int32 [T,k], w_out fp32 [T,k], counts_out int32 [E]
+ * (the per-expert token counts BiBoMoELayer._balance_step accumulates), logits_out fp32 [T,E].
+ */
+int bibo_moe_forward(const void* x, const void* w_router, const float* bias, const void* w_gate_up,
+                     const void* w_down, const float* theta, const bibo_moe_shape* shape, int norm_mode, int algo,
+                     void* out, int32_t* idx_out, float* w_out, int32_t* counts_out, float* logits_out,
+                     void* workspace, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BIBO_MOE_H */

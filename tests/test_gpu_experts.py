@@ -1,0 +1,162 @@
+"""Kernels 3 and 4 (grouped gate/up + Radial NormSiLU, grouped down + weighted combine) against the
+oracle, for the generic and the MFMA kernel families, through the C ABI.
+
+Tolerances: fp32 kernels vs the fp64 oracle 1e-5 (reference: ablate/common/test_eager_radial.py:61);
+bf16 kernels vs the fp32 oracle max|d|/max|ref| <= 2e-2 (reference: ablate/common/test_act_silu.py:65-66)."""
+import numpy as np
+import pytest
+import torch
+
+from bibo_amd import ops
+from oracle import bibo_moe_oracle as O
+from conftest import rel_err
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+BF16_TOL = 2e-2
+
+
+def _route(p):
+    idx, w, _ = O.route_from_logits(O.router_logits(p["x"], p["w_router"]), p["bias"].numpy(), p["k"])
+    return idx, w
+
+
+def _gpu_experts(p, idx, w, algo):
+    out, counts = ops.experts_fwd(p["x"].to(DEV), torch.from_numpy(idx).to(DEV), torch.from_numpy(w).to(DEV),
+                                  p["w_gate_up"].to(DEV), p["w_down"].to(DEV), p["theta"].to(DEV), algo=algo,
+                                  want_counts=True)
+    torch.cuda.synchronize()
+    return out.cpu(), counts.cpu().numpy()
+
+
+def _stages(p, idx, w, algo):
+    """The two expert kernels called separately, returning the intermediate activations too."""
+    E = p["w_gate_up"].shape[0]
+    idx_d = torch.from_numpy(idx).to(DEV)
+    counts, offsets, perm_slot, perm_token = ops.permute(idx_d, E)
+    hidden = ops.gateup_fwd(p["x"].to(DEV), p["w_gate_up"].to(DEV), p["theta"].to(DEV), offsets, perm_token,
+                            idx.shape[1], algo=algo)
+    out = ops.down_combine_fwd(hidden, p["w_down"].to(DEV), torch.from_numpy(w).to(DEV), offsets, perm_slot,
+                               idx.shape[0], algo=algo)
+    torch.cuda.synchronize()
+    return hidden.cpu(), out.cpu()
+
+
+# ------------------------------------------------------------------ fp32 generic kernels vs fp64
+def test_fp32_kernels_match_the_fp64_closed_form():
+    """theta = -2/0/1.5/3 (p = .12/.50/.82/.95), every row through one expert with weight 1
+    (tests/test_moe.py:35-50 of the reference)."""
+    g = torch.Generator().manual_seed(0)
+    E, H, I, N = 4, 64, 96, 40
+    p = dict(x=torch.randn(N, H, generator=g), w_gate_up=torch.randn(E, 2 * I, H, generator=g) * 0.1,
+             w_down=torch.randn(E, H, I, generator=g) * 0.1, theta=torch.tensor([-2.0, 0.0, 1.5, 3.0]))
+    for e in range(E):
+        idx = np.full((N, 1), e, dtype=np.int32)
+        w = np.ones((N, 1), dtype=np.float32)
+        out, counts = _gpu_experts(p, idx, w, "generic")
+        ref = O.experts_forward(p["x"], idx, w, p["w_gate_up"], p["w_down"], p["theta"], dtype=torch.float64)
+        assert rel_err(out, ref) < 1e-5
+        assert counts.tolist() == [N if j == e else 0 for j in range(E)]
+
+
+def test_fp32_kernels_at_p_zero_are_normsilu_and_theta_moves_the_output():
+    g = torch.Generator().manual_seed(1)
+    E, H, I, N = 4, 32, 64, 40                                   # ablate/common/test_eager_radial.py:34
+    x = torch.randn(N, H, generator=g)
+    wgu = torch.randn(E, 2 * I, H, generator=g) * 0.2
+    wd = torch.randn(E, H, I, generator=g) * 0.2
+    idx = np.zeros((N, 1), dtype=np.int32); w = np.ones((N, 1), dtype=np.float32)
+    p = dict(x=x, w_gate_up=wgu, w_down=wd, theta=torch.tensor([-40.0, 0, 0, 0]))
+    out, _ = _gpu_experts(p, idx, w, "generic")
+    gate, up = (x.double() @ wgu[0].double().t()).chunk(2, -1)
+    ns = torch.nn.functional.silu(gate * torch.rsqrt(gate.square().mean(-1, keepdim=True) + 1e-6)) * up
+    assert (out.double() - ns @ wd[0].double().t()).abs().max() < 1e-4
+    p2 = dict(p, theta=torch.tensor([-38.0, 0, 0, 0]))
+    assert (_gpu_experts(p2, idx, w, "generic")[0] - out).abs().max() < 1e-5      # still the p=0 floor
+    p3 = dict(p, theta=torch.tensor([2.0, 0, 0, 0]))
+    assert (_gpu_experts(p3, idx, w, "generic")[0] - out).abs().max() > 1e-4      # theta is live
+
+
+def test_fp32_combine_is_linear_and_handles_repeated_experts():
+    g = torch.Generator().manual_seed(2)
+    E, H, I, N = 6, 48, 40, 33
+    p = dict(x=torch.randn(N, H, generator=g), w_gate_up=torch.randn(E, 2 * I, H, generator=g) * 0.1,
+             w_down=torch.randn(E, H, I, generator=g) * 0.1, theta=torch.randn(E, generator=g))
+    one = lambda e: _gpu_experts(p, np.full((N, 1), e, np.int32), np.ones((N, 1), np.float32), "generic")[0]
+    idx = np.tile(np.array([[1, 4]], np.int32), (N, 1))
+    w = np.tile(np.array([[0.3, 0.7]], np.float32), (N, 1))
+    both, _ = _gpu_experts(p, idx, w, "generic")
+    assert torch.allclose(both, 0.3 * one(1) + 0.7 * one(4), atol=1e-6)
+    rep, _ = _gpu_experts(p, np.tile(np.array([[2, 2]], np.int32), (N, 1)), w, "generic")
+    assert torch.allclose(rep, one(2), atol=1e-6)                 # 0.3*E2 + 0.7*E2
+
+
+# ------------------------------------------------------------------ bf16 kernels vs fp32 oracle
+@pytest.mark.parametrize("algo", ["generic", "mfma"])
+@pytest.mark.parametrize("name", ["c1", "c3"])
+def test_bf16_experts_match_oracle_on_named_workloads(name, algo):
+    p = O.make_inputs(**O.CONFIGS[name])
+    idx, w = _route(p)
+    ref, ref_hidden = O.experts_forward(p["x"], idx, w, p["w_gate_up"], p["w_down"], p["theta"], return_hidden=True)
+    hidden, out_staged = _stages(p, idx, w, algo)
+    assert rel_err(hidden, ref_hidden) <= BF16_TOL
+    out, counts = _gpu_experts(p, idx, w, algo)
+    assert out.dtype == torch.bfloat16
+    assert rel_err(out, ref) <= BF16_TOL
+    assert torch.equal(out, out_staged), "composite and staged entry points must agree exactly"
+    assert np.array_equal(counts, O.permute(idx, 64)[0])
+
+
+@pytest.mark.parametrize("algo", ["generic", "mfma"])
+@pytest.mark.parametrize("T,H,I,bias,theta", [(1024, 768, 384, "uniform", "normal"), (1024, 768, 384, "hot4", "normal"),
+                                              (7, 1024, 512, "zero", "normal"), (333, 256, 128, "uniform", "normal"),
+                                              (130, 128, 256, "zero", "zero")])
+def test_bf16_experts_reduced_prefill_and_ragged_shapes(T, H, I, bias, theta, algo):
+    p = O.make_inputs(T=T, H=H, E=64, k=6, I=I, bias=bias, theta=theta, seed=T + H)
+    idx, w = _route(p)
+    ref = O.experts_forward(p["x"], idx, w, p["w_gate_up"], p["w_down"], p["theta"])
+    out, _ = _gpu_experts(p, idx, w, algo)
+    assert rel_err(out, ref) <= BF16_TOL
+
+
+def test_mfma_and_generic_families_agree():
+    p = O.make_inputs(T=777, H=768, E=64, k=6, I=384, bias="uniform", theta="normal", seed=5)
+    idx, w = _route(p)
+    h_g, o_g = _stages(p, idx, w, "generic")
+    h_m, o_m = _stages(p, idx, w, "mfma")
+    assert rel_err(h_m, h_g) <= 1e-2 and rel_err(o_m, o_g) <= 1e-2
+
+
+def test_mfma_with_empty_experts_and_one_hot_expert():
+    """Only experts {5, 9} get rows (everything else empty), one of them with a ragged last tile."""
+    g = torch.Generator().manual_seed(11)
+    T, H, I, E = 201, 512, 256, 64
+    p = O.make_inputs(T=T, H=H, E=E, k=2, I=I, theta="normal", seed=11)
+    idx = np.tile(np.array([[5, 9]], np.int32), (T, 1))
+    w = torch.rand(T, 2, generator=g).numpy().astype(np.float32)
+    ref = O.experts_forward(p["x"], idx, w, p["w_gate_up"], p["w_down"], p["theta"])
+    for algo in ("generic", "mfma"):
+        out, counts = _gpu_experts(p, idx, w, algo)
+        assert rel_err(out, ref) <= BF16_TOL
+        assert counts[5] == T and counts[9] == T and counts.sum() == 2 * T
+
+
+@pytest.mark.parametrize("name", ["c2", "c4"])
+def test_full_size_prefill_properties(name):
+    """Full T: (a) oracle parity on a 256-token sample (a token's output depends only on its own row and
+    routing); (b) doubling the routing weights doubles the bf16 output exactly; (c) permuting the tokens
+    permutes the output rows exactly."""
+    p = O.make_inputs(**O.CONFIGS[name])
+    T = p["x"].shape[0]
+    idx, w = _route(p)
+    out, counts = _gpu_experts(p, idx, w, "mfma")
+    assert counts.sum() == T * 6 and np.array_equal(counts, np.bincount(idx.reshape(-1), minlength=64))
+    sample = np.random.default_rng(0).choice(T, 256, replace=False)
+    ref = O.experts_forward(p["x"][sample], idx[sample], w[sample], p["w_gate_up"], p["w_down"], p["theta"])
+    assert rel_err(out[sample], ref) <= BF16_TOL
+    out2, _ = _gpu_experts(p, idx, (2 * w).astype(np.float32), "mfma")
+    assert torch.equal(out2.float(), 2 * out.float())
+    perm = torch.randperm(T, generator=torch.Generator().manual_seed(1))
+    pp = dict(p, x=p["x"][perm].contiguous())
+    outp, _ = _gpu_experts(pp, idx[perm.numpy()], w[perm.numpy()], "mfma")
+    assert torch.equal(outp, out[perm])

@@ -1,0 +1,158 @@
+"""The drop-in modules on the GPU: same behaviours the reference's tests/test_moe.py checks on
+BiBoMoELayer / BiBoMoERouter, plus parity of the whole layer with the oracle."""
+import numpy as np
+import pytest
+import torch
+
+import bibo_amd
+from oracle import bibo_moe_oracle as O
+from conftest import rel_err
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+
+
+def make_config(**kw):
+    base = dict(hidden_size=64, intermediate_size=96, moe_intermediate_size=96, num_routed_experts=8,
+                special_expert_pairs=0, num_experts_per_tok=2)
+    base.update(kw)
+    return bibo_amd.BiBoMoEConfig(**base)
+
+
+def _layer_from(p, dtype=torch.bfloat16, **cfg):
+    E, two_i, H = p["w_gate_up"].shape
+    c = bibo_amd.BiBoMoEConfig(hidden_size=H, moe_intermediate_size=two_i // 2, num_routed_experts=E,
+                               special_expert_pairs=0, num_experts_per_tok=p["k"], **cfg)
+    layer = bibo_amd.BiBoMoELayer(c)
+    sd = {"gate.gate_proj.weight": p["w_router"].float(), "gate.bias": p["bias"],
+          "experts.gate_up_proj": p["w_gate_up"].float(), "experts.down_proj": p["w_down"].float(),
+          "experts.radial_theta": p["theta"], "accumulated_tpe": torch.zeros(E)}
+    layer.load_state_dict(sd, strict=True)
+    return layer.to(DEV).to(dtype).eval()
+
+
+@pytest.mark.parametrize("name", ["c1", "c3"])
+def test_layer_matches_oracle(name):
+    cfg = O.CONFIGS[name]
+    p = O.make_inputs(**cfg)
+    layer = _layer_from(p)
+    x3 = p["x"].view(cfg["B"], -1, cfg["H"]).to(DEV)
+    with torch.no_grad():
+        out = layer(x3)
+        logits = layer.gate.router_logits(x3)
+        idx, w = layer.gate(x3)
+    assert out.shape == x3.shape and out.dtype == torch.bfloat16
+    assert idx.dtype == torch.int64 and w.dtype == torch.float32 and idx.shape == (cfg["B"], cfg["T"] // cfg["B"], 6)
+    ref, oi, ow = O.moe_forward(**p, logits=logits.cpu().numpy())
+    assert np.array_equal(idx.view(-1, 6).cpu().numpy(), oi)
+    assert np.array_equal(w.view(-1, 6).cpu().numpy(), ow)
+    assert rel_err(out.view(-1, cfg["H"]).cpu(), ref) <= 2e-2
+    # the same layer evaluated with the oracle's own logits: routing flips only at ulp-level near-ties
+    ref2, oi2, _ = O.moe_forward(**p)
+    assert (oi2 != oi).any(1).mean() < 0.01
+
+
+def test_hooked_path_equals_fused_path_and_replays_hooks():
+    p = O.make_inputs(**O.CONFIGS["c1"])
+    layer = _layer_from(p)
+    x3 = p["x"].view(1, -1, 512).to(DEV)
+    with torch.no_grad():
+        fused = layer(x3)
+    seen = {}
+    h1 = layer.experts.register_forward_pre_hook(lambda m, a: seen.__setitem__("experts", a))
+    h2 = layer.gate.register_forward_hook(lambda m, a, o: seen.__setitem__("gate", (a, o)))
+    layer.gate._probe_gap = True
+    with torch.no_grad():
+        hooked = layer(x3)
+    h1.remove(); h2.remove(); layer.gate._probe_gap = False
+    assert torch.equal(fused, hooked)
+    flat, idx, w = seen["experts"]                              # (hidden, idx.long(), w): router_trace.py of the reference
+    assert flat.shape == (512, 512) and idx.dtype == torch.int64 and idx.shape == (512, 6) and w.dtype == torch.float32
+    (gin,), (gidx, gw) = seen["gate"]
+    assert gin.shape == (1, 512, 512) and gidx.shape == (1, 512, 6) and gw.shape == (1, 512, 6)
+    gap = layer.gate.boundary_gap
+    assert gap is not None and gap.ndim == 0 and 0 < float(gap) < 1
+
+
+def test_router_module_contract():
+    """tests/test_moe.py:138-202 of the reference: fp32 positive weights with unit mass, raw scores without
+    normalisation, bias only moves selection."""
+    for norm in ("sum", "softmax"):
+        r = bibo_amd.BiBoMoERouter(make_config(norm_topk_prob=norm)).to(DEV)
+        with torch.no_grad():
+            idx, w = r(torch.randn(2, 5, 64, device=DEV) * 3)
+        assert w.dtype == torch.float32 and (w > 0).all() and idx.min() >= 0 and idx.max() < 8
+        assert torch.allclose(w.sum(-1), torch.ones(2, 5, device=DEV), atol=1e-6)
+    r = bibo_amd.BiBoMoERouter(make_config(norm_topk_prob=False)).to(DEV)
+    x = torch.randn(2, 5, 64, device=DEV) * 3
+    with torch.no_grad():
+        _, w = r(x)
+        scores = torch.sigmoid(r.router_logits(x))
+    assert not torch.allclose(w.sum(-1), torch.ones(2, 5, device=DEV), atol=1e-3)
+    assert torch.allclose(w.flatten().sort().values, scores.topk(2, -1).values.flatten().sort().values, atol=1e-6)
+    with torch.no_grad():
+        r.bias[0] = 5.0
+        idx, w = r(x)
+    assert (idx == 0).any(-1).all() and w.max() <= 1.0 + 1e-6
+
+
+def test_dtype_regimes():
+    """fp32 module: fp32 kernels, tight tolerance; .to(bfloat16) module keeps routing fp32 and returns bf16
+    (tests/test_moe.py:252-259); bf16 autocast over fp32 masters runs the bf16 kernels and returns fp32."""
+    p = O.make_inputs(T=40, H=64, E=8, k=2, I=96, bias="uniform", theta="normal", seed=4, dtype=torch.float32)
+    layer = _layer_from(p, dtype=torch.float32)
+    x3 = p["x"].view(2, 20, 64).to(DEV)
+    with torch.no_grad():
+        out = layer(x3)
+        logits = layer.gate.router_logits(x3)
+    idx, w, _ = O.route_from_logits(logits.cpu().numpy(), p["bias"].numpy(), 2)
+    ref = O.experts_forward(p["x"], idx, w, p["w_gate_up"], p["w_down"], p["theta"], dtype=torch.float64)
+    assert out.dtype == torch.float32 and rel_err(out.view(-1, 64).cpu(), ref) < 1e-5
+    half = _layer_from(p, dtype=torch.bfloat16)
+    with torch.no_grad():
+        _, wh = half.gate(x3.bfloat16())
+        oh = half(x3.bfloat16())
+    assert wh.dtype == torch.float32 and oh.dtype == torch.bfloat16
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        oa = layer(x3)
+        la = layer.gate.router_logits(x3)
+    pb = {k_: (v.bfloat16() if k_ in ("x", "w_router", "w_gate_up", "w_down") else v) for k_, v in p.items()}
+    ref_a, _, _ = O.moe_forward(**pb, logits=la.cpu().numpy())
+    assert oa.dtype == torch.float32 and rel_err(oa.view(-1, 64).cpu(), ref_a) <= 2e-2
+
+
+def test_training_mode_balances_once_per_forward_and_eval_never():
+    p = O.make_inputs(T=64, H=64, E=8, k=2, I=96, seed=6)
+    layer = _layer_from(p, bias_update_factor=0.4, bias_update_threshold=64 * 2)
+    x3 = p["x"].view(2, 32, 64).to(DEV)
+    with torch.no_grad():
+        layer(x3)
+    assert layer._fwd_step == 0 and float(layer.accumulated_tpe.sum()) == 0         # eval: never
+    layer.train()
+    with torch.no_grad():
+        layer(x3)
+    assert layer._fwd_step == 1 and float(layer.accumulated_tpe.sum()) == 64 * 2    # T*k slots counted once
+    idx, _, _ = O.route_from_logits(layer.gate.router_logits(x3).cpu().numpy(), p["bias"].numpy(), 2)
+    assert np.array_equal(layer.accumulated_tpe.float().cpu().numpy(), np.bincount(idx.reshape(-1), minlength=8))
+    bias_before = layer.gate.bias.clone()
+    with torch.no_grad():
+        layer(x3)                                                                    # second forward fires
+    assert layer._fwd_step == 2 and float(layer.accumulated_tpe.sum()) == 0
+    assert not torch.equal(bias_before, layer.gate.bias) and abs(float(layer.gate.bias.float().mean())) < 1e-3
+    # hooked path takes the same counts
+    layer2 = _layer_from(p, bias_update_factor=0.4, bias_update_threshold=64 * 2).train()
+    h = layer2.experts.register_forward_pre_hook(lambda m, a: None)
+    with torch.no_grad():
+        layer2(x3)
+    h.remove()
+    assert np.array_equal(layer2.accumulated_tpe.float().cpu().numpy(), np.bincount(idx.reshape(-1), minlength=8))
+
+
+def test_experts_module_seam_takes_int64_indices():
+    p = O.make_inputs(T=50, H=64, E=8, k=2, I=96, theta="normal", seed=8)
+    layer = _layer_from(p)
+    idx, w, _ = O.route_from_logits(O.router_logits(p["x"], p["w_router"]), p["bias"].numpy(), 2)
+    with torch.no_grad():
+        out = layer.experts(p["x"].to(DEV), torch.from_numpy(idx).long().to(DEV), torch.from_numpy(w).to(DEV))
+    ref = O.experts_forward(p["x"], idx, w, p["w_gate_up"], p["w_down"], p["theta"])
+    assert out.dtype == torch.bfloat16 and rel_err(out.cpu(), ref) <= 2e-2

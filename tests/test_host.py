@@ -1,0 +1,143 @@
+"""CPU-side checks: the C-ABI library loads and exports what the header declares, argument errors are
+reported before anything is launched, and the host mirror keeps the reference's module contract
+(tests/test_moe.py:14-24,198-310 of the reference for layout and balancing closed forms)."""
+import ctypes
+import pathlib
+import re
+
+import pytest
+import torch
+
+import bibo_amd
+from bibo_amd import _lib as L
+from bibo_amd import ops
+
+ROOT = pathlib.Path(__file__).resolve().parents[1]
+
+
+def make_config(**kw):
+    base = dict(hidden_size=64, intermediate_size=96, moe_intermediate_size=96, num_routed_experts=8,
+                special_expert_pairs=0, num_experts_per_tok=2)
+    base.update(kw)
+    return bibo_amd.BiBoMoEConfig(**base)
+
+
+# ------------------------------------------------------------------ C ABI
+def test_library_exports_every_declared_symbol():
+    header = (ROOT / "include" / "bibo_moe.h").read_text()
+    declared = set(re.findall(r"^(?:int|const char\*)\s+(bibo_moe_\w+)\s*\(", header, re.M))
+    assert declared == set(L.SYMBOLS), "binding and header disagree"
+    lib = L.lib()
+    for name in declared:
+        assert hasattr(lib, name)
+    assert lib.bibo_moe_abi_version() == 1
+
+
+def test_argument_errors_are_reported_without_a_gpu():
+    lib = L.lib()
+    out = ctypes.c_size_t(0)
+    ok = L.Shape(8192, 768, 64, 6, 384, L.DTYPE_BF16)
+    assert lib.bibo_moe_workspace_bytes(ctypes.byref(ok), ctypes.byref(out)) == 0 and out.value > 0
+    for bad in (L.Shape(8, 64, 65, 2, 32, 0), L.Shape(8, 64, 8, 9, 32, 0), L.Shape(8, 64, 4, 5, 32, 0),
+                L.Shape(-1, 64, 8, 2, 32, 0), L.Shape(8, 0, 8, 2, 32, 0)):
+        assert lib.bibo_moe_workspace_bytes(ctypes.byref(bad), ctypes.byref(out)) == -2
+    assert lib.bibo_moe_workspace_bytes(ctypes.byref(L.Shape(8, 64, 8, 2, 32, 7)), ctypes.byref(out)) == -3
+    assert lib.bibo_moe_workspace_bytes(None, ctypes.byref(out)) == -1
+    # stage entry points validate before launching
+    assert lib.bibo_moe_router_fwd(None, None, None, 4, 64, 8, 2, 0, 1, None, None, None, None, None) == -1
+    assert lib.bibo_moe_router_fwd(None, None, None, 4, 64, 8, 9, 0, 1, None, None, None, None, None) == -2
+    assert lib.bibo_moe_gateup_fwd(None, None, None, None, None, 4, 64, 8, 2, 96, 0, L.ALGO_MFMA, None, None) == -6
+    assert lib.bibo_moe_permute(None, 4, 8, 2, None, None, None, None, None, 0, None) == -1
+    assert b"workspace" in lib.bibo_moe_strerror(-4)
+    with pytest.raises(RuntimeError, match="workspace"):
+        L.check(-4, "x")
+
+
+def test_cpu_tensors_are_refused_loudly():
+    x = torch.zeros(4, 64, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="GPU"):
+        ops.router_fwd(x, torch.zeros(8, 64, dtype=torch.bfloat16), torch.zeros(8), 2)
+    layer = bibo_amd.BiBoMoELayer(make_config())
+    with torch.no_grad(), pytest.raises(RuntimeError, match="GPU"):
+        layer(torch.zeros(1, 4, 64))
+
+
+# ------------------------------------------------------------------ config + module contract
+def test_config_derivations_follow_the_reference():
+    c = bibo_amd.BiBoMoEConfig(intermediate_size=2304, num_experts_per_tok=6, num_routed_experts=64,
+                               special_expert_pairs=0, norm_topk_prob=True)
+    assert c.moe_intermediate_size == 384 and c.norm_topk_prob == "sum"
+    assert c.bias_update_factor == 0.4 and c.bias_update_threshold == 8000 and c.num_glu_experts == 64
+    c = bibo_amd.BiBoMoEConfig(num_routed_experts=8, special_expert_pairs=1, num_experts_per_tok=2)
+    assert c.num_glu_experts == 6 and c.num_pos_identity_experts == 1
+    with pytest.raises(ValueError):
+        bibo_amd.BiBoMoEConfig(num_routed_experts=4, num_experts_per_tok=5, special_expert_pairs=0)
+    with pytest.raises(ValueError):
+        bibo_amd.BiBoMoEConfig(num_routed_experts=2, special_expert_pairs=1, num_experts_per_tok=1)
+    with pytest.raises(ValueError):
+        bibo_amd.BiBoMoEConfig(norm_topk_prob="max", special_expert_pairs=0)
+
+
+def test_state_dict_layout_matches_the_reference_layer():
+    c = make_config()
+    layer = bibo_amd.BiBoMoELayer(c)
+    sd = layer.state_dict()
+    assert {k: tuple(v.shape) for k, v in sd.items()} == {
+        "accumulated_tpe": (8,), "gate.bias": (8,), "gate.gate_proj.weight": (8, 64),
+        "experts.gate_up_proj": (8, 192, 64), "experts.down_proj": (8, 64, 96), "experts.radial_theta": (8,)}
+    assert layer.gate.bias.requires_grad is False and layer.experts.radial_theta.requires_grad
+    assert float(layer.experts.radial_theta.abs().max()) == 0.0
+    e = layer.experts
+    assert (e.pos_start, e.pos_end, e.neg_start, e.neg_end) == (8, 8, 8, 8)
+    assert layer.gate.top_k == 2 and layer.gate.norm_topk_prob == "sum" and layer.gate._probe_gap is False
+    assert not hasattr(layer.gate, "gate_conv")
+
+
+def test_unsupported_configurations_raise():
+    with pytest.raises(NotImplementedError, match="Identity"):
+        bibo_amd.BiBoMoELayer(make_config(special_expert_pairs=1))
+    with pytest.raises(NotImplementedError, match="shared"):
+        bibo_amd.BiBoMoELayer(make_config(use_shared_expert=True))
+
+
+def test_forward_refuses_to_drop_gradients():
+    layer = bibo_amd.BiBoMoELayer(make_config())
+    with pytest.raises(RuntimeError, match="forward pass only"):
+        layer(torch.zeros(1, 4, 64))
+
+
+# ------------------------------------------------------------------ balancing closed forms
+def test_bias_update_moves_toward_balance_and_keeps_the_mean():
+    layer = bibo_amd.BiBoMoELayer(make_config(bias_update_factor=0.4))
+    tpe = torch.full((8,), 10.0); tpe[0] = 100.0
+    layer.update_bias(tpe)
+    b = layer.gate.bias
+    assert b[0] < 0 and (b[1:] > 0).all() and abs(float(b.mean())) < 1e-6
+    share = tpe / tpe.sum()
+    assert torch.allclose(b, 0.4 * (share.mean() - share), atol=1e-7)
+
+
+def test_balanced_load_gives_no_update_and_zero_factor_disables():
+    layer = bibo_amd.BiBoMoELayer(make_config(bias_update_factor=1.0))
+    layer.update_bias(torch.full((8,), 100.0))
+    assert float(layer.gate.bias.abs().max()) < 1e-6
+    off = bibo_amd.BiBoMoELayer(make_config(bias_update_factor=0.0))
+    off.update_bias(torch.tensor([1000.0] + [10.0] * 7))
+    assert float(off.gate.bias.abs().max()) == 0.0
+    empty = bibo_amd.BiBoMoELayer(make_config(bias_update_factor=0.4))
+    empty.update_bias(torch.zeros(8))                       # nothing routed: clamp avoids 0/0
+    assert torch.isfinite(empty.gate.bias).all()
+
+
+def test_balance_step_fires_on_the_forward_step_interval():
+    tokens = 16
+    layer = bibo_amd.BiBoMoELayer(make_config(bias_update_threshold=tokens * 3)).train()
+    idx = torch.zeros(2, 8, 2, dtype=torch.long)
+    fired = [layer._balance_step(idx, tokens) is not None for _ in range(7)]
+    assert layer._update_every == 3 and fired == [False, False, True, False, False, True, False]
+    # counts accumulate between firings and reset after
+    layer = bibo_amd.BiBoMoELayer(make_config(bias_update_threshold=tokens * 2)).train()
+    assert layer._balance_step(idx, tokens) is None
+    tpe = layer._balance_step(None, tokens, counts=torch.tensor([1, 2, 3, 4, 5, 6, 7, 4], dtype=torch.int32))
+    assert tpe.tolist() == [33.0, 2.0, 3.0, 4.0, 5.0, 6.0, 7.0, 4.0]
+    assert float(layer.accumulated_tpe.abs().max()) == 0.0
