@@ -142,7 +142,7 @@ class Layer:
         return ((got - ref.double()).abs().max() / ref.double().abs().max()).item(), int((self.counts > 0).sum())
 
 
-def cpu_baseline(name, budget_s=20.0, sample_tokens=2048):
+def cpu_baseline(name, budget_s=20.0, sample_tokens=8192):
     """The reference's eager CPU path (oracle restatement) timed on this box's host cores."""
     import torch
     from oracle import bibo_moe_oracle as O
@@ -156,7 +156,7 @@ def cpu_baseline(name, budget_s=20.0, sample_tokens=2048):
         O.eager_loop_forward(**q)                       # warm-up
         t0 = time.perf_counter()
         reps = 0
-        while reps < 5 and (time.perf_counter() - t0) < budget_s / 2:
+        while reps < 3 or (time.perf_counter() - t0) < budget_s / 2:
             O.eager_loop_forward(**q)
             reps += 1
         dt = (time.perf_counter() - t0) / max(reps, 1)
