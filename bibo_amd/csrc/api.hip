@@ -18,13 +18,29 @@ int check_dims(int T, int H, int E, int k, int I, int dtype) {
   return BIBO_OK;
 }
 
-int resolve_algo(int algo, int H, int I, int dtype, int* out) {
+// rows per expert at or below which the weight-streaming kernels are preferred
+constexpr long long kStreamRowsPerExpert = 32;
+
+inline bool stream_eligible(int T, int H, int E, int k, int I, int dtype) {
+  return stream_supported(H, I, dtype) && (long long)T * k <= kStreamRowsPerExpert * E;
+}
+
+// `composite`: the caller is bibo_moe_experts_fwd / bibo_moe_forward, the only entry points that can run
+// the streaming kernels (they hand fp32 pre-activations, not `hidden`, from one kernel to the next).
+int resolve_algo(int algo, int T, int H, int E, int k, int I, int dtype, bool composite, int* out) {
   switch (algo) {
-    case BIBO_ALGO_AUTO: *out = mfma_supported(H, I, dtype) ? BIBO_ALGO_MFMA : BIBO_ALGO_GENERIC; break;
+    case BIBO_ALGO_AUTO:
+      if (composite && stream_eligible(T, H, E, k, I, dtype)) *out = BIBO_ALGO_STREAM;
+      else *out = mfma_supported(H, I, dtype) ? BIBO_ALGO_MFMA : BIBO_ALGO_GENERIC;
+      break;
     case BIBO_ALGO_GENERIC: *out = BIBO_ALGO_GENERIC; break;
     case BIBO_ALGO_MFMA:
       if (!mfma_supported(H, I, dtype)) return BIBO_ERR_UNSUPPORTED;
       *out = BIBO_ALGO_MFMA;
+      break;
+    case BIBO_ALGO_STREAM:
+      if (!composite || !stream_supported(H, I, dtype)) return BIBO_ERR_UNSUPPORTED;
+      *out = BIBO_ALGO_STREAM;
       break;
     default: return BIBO_ERR_UNSUPPORTED;
   }
@@ -49,7 +65,10 @@ Workspace carve(int T, int H, int E, int k, int I, int dtype) {
   ws.offsets = o;    o += align_up((kMaxE + 1) * sizeof(int32_t));
   ws.perm_slot = o;  o += align_up(S * sizeof(int32_t));
   ws.perm_token = o; o += align_up(S * sizeof(int32_t));
-  ws.hidden = o;     o += align_up(S * (size_t)I * elt_size(dtype));
+  // `hidden` (permuted activations) and, for the streaming kernels, fp32 gate/up pre-activations share a segment
+  const size_t hidden_bytes = S * (size_t)I * elt_size(dtype);
+  const size_t gu_bytes = stream_supported(H, I, dtype) ? S * (size_t)2 * I * sizeof(float) : 0;
+  ws.hidden = o;     o += align_up(hidden_bytes > gu_bytes ? hidden_bytes : gu_bytes);
   ws.yw = o;         o += align_up(S * (size_t)H * sizeof(float));
   ws.total = o;
   return ws;
@@ -72,12 +91,34 @@ int down_dispatch(const void* hidden, const void* wd, const float* w, const int3
   hipError_t e;
   if (algo == BIBO_ALGO_MFMA) {
     if (!aligned16(hidden) || !aligned16(wd)) return BIBO_ERR_MISALIGNED;
-    e = launch_down_mfma(hidden, wd, w, offsets, perm_slot, T, H, E, k, I, yw, /*yw_is_bf16=*/0, s);
-  } else {
-    e = launch_down_generic(hidden, wd, w, offsets, perm_slot, T, H, E, k, I, dtype, yw, s);
+    // weighted expert outputs travel to the combine in bf16 (the reference's bf16 eager path rounds each
+    // expert output to bf16 as well, moe.py:92)
+    e = launch_down_mfma(hidden, wd, w, offsets, perm_slot, T, H, E, k, I, yw, /*yw_is_bf16=*/1, s);
+    if (e != hipSuccess) return (int)e;
+    return hip_rc(launch_combine(yw, 1, T, H, k, dtype, out, s));
   }
+  e = launch_down_generic(hidden, wd, w, offsets, perm_slot, T, H, E, k, I, dtype, yw, s);
   if (e != hipSuccess) return (int)e;
   return hip_rc(launch_combine(yw, 0, T, H, k, dtype, out, s));
+}
+
+// kernels 3 and 4 (+ combine) after the permutation, for the composite entry points
+int experts_dispatch(const void* x, const void* wgu, const void* wd, const float* theta, const float* w,
+                     const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token, int T, int H, int E,
+                     int k, int I, int dtype, int algo, void* out, char* base, const Workspace& ws, hipStream_t s) {
+  float* yw = reinterpret_cast<float*>(base + ws.yw);
+  if (algo == BIBO_ALGO_STREAM) {
+    if (!aligned16(x) || !aligned16(wgu) || !aligned16(wd)) return BIBO_ERR_MISALIGNED;
+    float* gu = reinterpret_cast<float*>(base + ws.hidden);
+    hipError_t e = launch_gateup_stream(x, wgu, offsets, perm_token, T, H, E, k, I, gu, s);
+    if (e != hipSuccess) return (int)e;
+    e = launch_down_stream(gu, wd, theta, w, offsets, perm_slot, T, H, E, k, I, yw, s);
+    if (e != hipSuccess) return (int)e;
+    return hip_rc(launch_combine(yw, 0, T, H, k, dtype, out, s));
+  }
+  const int rc = gateup_dispatch(x, wgu, theta, offsets, perm_token, T, H, E, k, I, dtype, algo, base + ws.hidden, s);
+  if (rc != BIBO_OK) return rc;
+  return down_dispatch(base + ws.hidden, wd, w, offsets, perm_slot, T, H, E, k, I, dtype, algo, out, yw, s);
 }
 
 }  // namespace
@@ -137,7 +178,7 @@ int bibo_moe_gateup_fwd(const void* x, const void* w_gate_up, const float* theta
   int rc = check_dims(T, H, E, k, I, dtype);
   if (rc != BIBO_OK) return rc;
   int a;
-  if ((rc = resolve_algo(algo, H, I, dtype, &a)) != BIBO_OK) return rc;
+  if ((rc = resolve_algo(algo, T, H, E, k, I, dtype, false, &a)) != BIBO_OK) return rc;
   if (T == 0) return BIBO_OK;
   if (!x || !w_gate_up || !theta || !offsets || !perm_token || !hidden) return BIBO_ERR_NULL_POINTER;
   return gateup_dispatch(x, w_gate_up, theta, offsets, perm_token, T, H, E, k, I, dtype, a, hidden,
@@ -150,7 +191,7 @@ int bibo_moe_down_combine_fwd(const void* hidden, const void* w_down, const floa
   int rc = check_dims(T, H, E, k, I, dtype);
   if (rc != BIBO_OK) return rc;
   int a;
-  if ((rc = resolve_algo(algo, H, I, dtype, &a)) != BIBO_OK) return rc;
+  if ((rc = resolve_algo(algo, T, H, E, k, I, dtype, false, &a)) != BIBO_OK) return rc;
   if (T == 0) return BIBO_OK;
   if (!hidden || !w_down || !w || !offsets || !perm_slot || !out || !workspace) return BIBO_ERR_NULL_POINTER;
   if (workspace_bytes < (size_t)T * k * H * sizeof(float)) return BIBO_ERR_WORKSPACE_TOO_SMALL;
@@ -166,7 +207,7 @@ int bibo_moe_experts_fwd(const void* x, const int32_t* idx, const float* w, cons
   int rc = check_dims(T, H, E, k, I, dtype);
   if (rc != BIBO_OK) return rc;
   int a;
-  if ((rc = resolve_algo(algo, H, I, dtype, &a)) != BIBO_OK) return rc;
+  if ((rc = resolve_algo(algo, T, H, E, k, I, dtype, true, &a)) != BIBO_OK) return rc;
   if (!workspace) return BIBO_ERR_NULL_POINTER;
   if (T > 0 && (!x || !idx || !w || !w_gate_up || !w_down || !theta || !out)) return BIBO_ERR_NULL_POINTER;
   const Workspace ws = carve(T, H, E, k, I, dtype);
@@ -180,11 +221,8 @@ int bibo_moe_experts_fwd(const void* x, const int32_t* idx, const float* w, cons
   if ((rc = hip_rc(launch_permute(idx, T, E, k, counts, offsets, perm_slot, perm_token, base + ws.hist, s))) != BIBO_OK)
     return rc;
   if (T == 0) return BIBO_OK;
-  if ((rc = gateup_dispatch(x, w_gate_up, theta, offsets, perm_token, T, H, E, k, I, dtype, a, base + ws.hidden, s)) !=
-      BIBO_OK)
-    return rc;
-  return down_dispatch(base + ws.hidden, w_down, w, offsets, perm_slot, T, H, E, k, I, dtype, a, out,
-                       reinterpret_cast<float*>(base + ws.yw), s);
+  return experts_dispatch(x, w_gate_up, w_down, theta, w, offsets, perm_slot, perm_token, T, H, E, k, I, dtype, a, out,
+                          base, ws, s);
 }
 
 int bibo_moe_forward(const void* x, const void* w_router, const float* bias, const void* w_gate_up, const void* w_down,
@@ -197,7 +235,7 @@ int bibo_moe_forward(const void* x, const void* w_router, const float* bias, con
   if (rc != BIBO_OK) return rc;
   if (norm_mode < BIBO_NORM_NONE || norm_mode > BIBO_NORM_SOFTMAX) return BIBO_ERR_UNSUPPORTED;
   int a;
-  if ((rc = resolve_algo(algo, H, I, dtype, &a)) != BIBO_OK) return rc;
+  if ((rc = resolve_algo(algo, T, H, E, k, I, dtype, true, &a)) != BIBO_OK) return rc;
   if (!workspace) return BIBO_ERR_NULL_POINTER;
   if (T > 0 && (!x || !w_router || !bias || !w_gate_up || !w_down || !theta || !out)) return BIBO_ERR_NULL_POINTER;
   const Workspace ws = carve(T, H, E, k, I, dtype);
@@ -217,11 +255,8 @@ int bibo_moe_forward(const void* x, const void* w_router, const float* bias, con
   if ((rc = hip_rc(launch_permute(idx, T, E, k, counts, offsets, perm_slot, perm_token, base + ws.hist, s))) != BIBO_OK)
     return rc;
   if (T == 0) return BIBO_OK;
-  if ((rc = gateup_dispatch(x, w_gate_up, theta, offsets, perm_token, T, H, E, k, I, dtype, a, base + ws.hidden, s)) !=
-      BIBO_OK)
-    return rc;
-  return down_dispatch(base + ws.hidden, w_down, w, offsets, perm_slot, T, H, E, k, I, dtype, a, out,
-                       reinterpret_cast<float*>(base + ws.yw), s);
+  return experts_dispatch(x, w_gate_up, w_down, theta, w, offsets, perm_slot, perm_token, T, H, E, k, I, dtype, a, out,
+                          base, ws, s);
 }
 
 }  // extern "C"

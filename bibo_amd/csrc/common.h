@@ -15,7 +15,7 @@ constexpr float kNormSiluEps = 1e-6f;   // src/modeling/ffn/moe.py:16
 constexpr float kSumNormEps = 1e-20f;   // src/modeling/ffn/router.py:45
 
 // tokens handled by one workgroup of the histogram / permutation kernels
-constexpr int kPermTokens = 64;
+constexpr int kPermTokens = 256;
 
 typedef __bf16 bf16_t;
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -110,5 +110,12 @@ hipError_t launch_gateup_mfma(const void* x, const void* wgu, const float* theta
 hipError_t launch_down_mfma(const void* hidden, const void* wd, const float* w, const int32_t* offsets,
                             const int32_t* perm_slot, int T, int H, int E, int k, int I, void* yw, int yw_is_bf16,
                             hipStream_t s);
+
+bool stream_supported(int H, int I, int dtype);
+hipError_t launch_gateup_stream(const void* x, const void* wgu, const int32_t* offsets, const int32_t* perm_token,
+                                int T, int H, int E, int k, int I, float* gu, hipStream_t s);
+hipError_t launch_down_stream(const float* gu, const void* wd, const float* theta, const float* w,
+                              const int32_t* offsets, const int32_t* perm_slot, int T, int H, int E, int k, int I,
+                              float* yw, hipStream_t s);
 
 }  // namespace bibo

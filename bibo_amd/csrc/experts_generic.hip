@@ -100,6 +100,28 @@ __global__ __launch_bounds__(256) void combine_kernel(const TY* __restrict__ yw,
   }
 }
 
+// bf16 slot rows -> bf16 output, 8 columns (16 bytes) per thread, fp32 sum in ascending j   (moe.py:93,101)
+__global__ __launch_bounds__(256) void combine_bf16x8_kernel(const bf16_t* __restrict__ yw, int T, int H8, int k,
+                                                             bf16_t* __restrict__ out) {
+  const size_t n = (size_t)T * H8;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
+    const size_t t = i / H8, c = i - t * H8;
+    float acc[8];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) acc[q] = 0.f;
+    const bf16x8* src = reinterpret_cast<const bf16x8*>(yw) + (t * k) * H8 + c;
+    for (int j = 0; j < k; ++j) {
+      const bf16x8 v = src[(size_t)j * H8];
+#pragma unroll
+      for (int q = 0; q < 8; ++q) acc[q] += (float)v[q];
+    }
+    bf16x8 o;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) o[q] = (bf16_t)acc[q];
+    reinterpret_cast<bf16x8*>(out)[i] = o;
+  }
+}
+
 }  // namespace
 
 hipError_t launch_gateup_generic(const void* x, const void* wgu, const float* theta, const int32_t* offsets,
@@ -140,8 +162,14 @@ hipError_t launch_combine(const void* yw, int yw_is_bf16, int T, int H, int k, i
   const int grid = (int)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
   if (yw_is_bf16) {
     if (dtype != BIBO_DTYPE_BF16) return hipErrorInvalidValue;
-    hipLaunchKernelGGL((combine_kernel<bf16_t, bf16_t>), dim3(grid), dim3(256), 0, s,
-                       static_cast<const bf16_t*>(yw), T, H, k, static_cast<bf16_t*>(out));
+    if ((H % 8) == 0 && ((reinterpret_cast<uintptr_t>(yw) | reinterpret_cast<uintptr_t>(out)) & 15) == 0) {
+      const size_t n8 = n / 8;
+      const int g8 = (int)((n8 + 255) / 256 < 65536 ? (n8 + 255) / 256 : 65536);
+      hipLaunchKernelGGL(combine_bf16x8_kernel, dim3(g8), dim3(256), 0, s, static_cast<const bf16_t*>(yw), T, H / 8, k,
+                         static_cast<bf16_t*>(out));
+    } else
+      hipLaunchKernelGGL((combine_kernel<bf16_t, bf16_t>), dim3(grid), dim3(256), 0, s,
+                         static_cast<const bf16_t*>(yw), T, H, k, static_cast<bf16_t*>(out));
   } else if (dtype == BIBO_DTYPE_BF16) {
     hipLaunchKernelGGL((combine_kernel<float, bf16_t>), dim3(grid), dim3(256), 0, s, static_cast<const float*>(yw), T,
                        H, k, static_cast<bf16_t*>(out));

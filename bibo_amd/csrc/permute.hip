@@ -7,65 +7,96 @@
 namespace bibo {
 namespace {
 
-// One wave per 64 tokens: LDS histogram of the chunk's slots.
-__global__ __launch_bounds__(64) void hist_kernel(const int32_t* __restrict__ idx, int S, int E, int k,
-                                                  int32_t* __restrict__ block_hist) {
+// Histogram of one chunk of kPermTokens tokens (LDS atomics; only the totals matter here).
+__global__ __launch_bounds__(256) void hist_kernel(const int32_t* __restrict__ idx, int S, int E, int k,
+                                                   int32_t* __restrict__ block_hist) {
   __shared__ int h[kMaxE];
-  const int lane = threadIdx.x;
-  h[lane] = 0;
+  const int tid = threadIdx.x;
+  if (tid < kMaxE) h[tid] = 0;
   __syncthreads();
   const int s0 = blockIdx.x * kPermTokens * k;
   const int s1 = min(S, s0 + kPermTokens * k);
-  for (int s = s0 + lane; s < s1; s += kWave) {
+  for (int s = s0 + tid; s < s1; s += 256) {
     const unsigned e = (unsigned)idx[s];
     if (e < (unsigned)E) atomicAdd(&h[e], 1);
   }
   __syncthreads();
-  block_hist[blockIdx.x * kMaxE + lane] = h[lane];
+  if (tid < kMaxE) block_hist[blockIdx.x * kMaxE + tid] = h[tid];
 }
 
-// One wave per 64 tokens, lane = expert for the bookkeeping.  Each wave sums the chunk histograms
-// (all of them for the totals, the earlier ones for its own base), scans over experts, then ranks
-// its slots 64 at a time with ballots: slots of one expert keep ascending slot order.
-__global__ __launch_bounds__(64) void scatter_kernel(const int32_t* __restrict__ idx, int S, int E, int k,
-                                                     const int32_t* __restrict__ block_hist,
-                                                     int32_t* __restrict__ counts, int32_t* __restrict__ offsets,
-                                                     int32_t* __restrict__ perm_slot, int32_t* __restrict__ perm_token) {
-  const int lane = threadIdx.x;
-  const int b = blockIdx.x, nblk = gridDim.x;
-  int total = 0, before = 0;
-  for (int bb = 0; bb < nblk; ++bb) {
-    const int v = block_hist[bb * kMaxE + lane];
-    total += v;
-    before += (bb < b) ? v : 0;
+// Ballot ranking of 64 consecutive slots.  `peers` = lanes whose slot has my expert, `mine` = lanes whose
+// slot has the expert whose id is my lane id.
+__device__ __forceinline__ void match64(int e, bool valid, int lane, unsigned long long& peers,
+                                        unsigned long long& mine) {
+  const unsigned long long vmask = __ballot(valid);
+  peers = vmask;
+  mine = vmask;
+#pragma unroll
+  for (int bit = 0; bit < 6; ++bit) {
+    const unsigned long long bb = __ballot(valid && ((e >> bit) & 1));
+    peers &= ((e >> bit) & 1) ? bb : ~bb;
+    mine &= ((lane >> bit) & 1) ? bb : ~bb;
   }
-  const int incl = wave_inclusive_scan(total);
-  const int excl = incl - total;
-  if (b == 0) {
-    if (lane < E) { counts[lane] = total; offsets[lane] = excl; }
-    if (lane == E - 1) offsets[E] = incl;
-  }
-  int cnt = excl + before;                       // next free row of expert `lane`
-  const int s0 = b * kPermTokens * k;
-  const int s1 = min(S, s0 + kPermTokens * k);
+}
+
+// One workgroup per chunk of kPermTokens tokens, four waves of 64 tokens each, lane = expert for the
+// bookkeeping.  (1) every wave counts its own slots per expert; (2) the chunk histograms are summed
+// (all chunks for the totals, earlier chunks for this chunk's base) with the loads spread over the
+// 256 threads; (3) exclusive scan over experts; (4) every wave ranks its slots 64 at a time, slots of
+// one expert keeping ascending slot order.
+__global__ __launch_bounds__(256) void scatter_kernel(const int32_t* __restrict__ idx, int S, int E, int k,
+                                                      const int32_t* __restrict__ block_hist, int nblk,
+                                                      int32_t* __restrict__ counts, int32_t* __restrict__ offsets,
+                                                      int32_t* __restrict__ perm_slot, int32_t* __restrict__ perm_token) {
+  __shared__ int part_tot[4][kMaxE], part_bef[4][kMaxE], wave_cnt[4][kMaxE];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int b = blockIdx.x;
+  const int s0 = (b * kPermTokens + wave * 64) * k;
+  const int s1 = min(S, s0 + 64 * k);
   const unsigned long long lt = (1ull << lane) - 1ull;
+
+  int mycnt = 0;                                  // slots of expert `lane` among this wave's tokens
   for (int base = s0; base < s1; base += kWave) {
     const int s = base + lane;
     int e = 0;
     bool valid = s < s1;
     if (valid) { e = idx[s]; valid = (unsigned)e < (unsigned)E; }
     if (!valid) e = 0;
-    const unsigned long long vmask = __ballot(valid);
-    unsigned long long peers = vmask;            // lanes whose slot has my expert
-    unsigned long long mine = vmask;             // lanes whose slot has expert == my lane id
-#pragma unroll
-    for (int bit = 0; bit < 6; ++bit) {
-      const unsigned long long bb = __ballot(valid && ((e >> bit) & 1));
-      peers &= ((e >> bit) & 1) ? bb : ~bb;
-      mine &= ((lane >> bit) & 1) ? bb : ~bb;
-    }
-    const int rank = __popcll(peers & lt);
-    const int pos = __shfl(cnt, e, kWave) + rank;
+    unsigned long long peers, mine;
+    match64(e, valid, lane, peers, mine);
+    mycnt += __popcll(mine);
+  }
+  wave_cnt[wave][lane] = mycnt;
+
+  int tot = 0, bef = 0;
+  for (int bb = wave; bb < nblk; bb += 4) {
+    const int v = block_hist[bb * kMaxE + lane];
+    tot += v;
+    bef += (bb < b) ? v : 0;
+  }
+  part_tot[wave][lane] = tot;
+  part_bef[wave][lane] = bef;
+  __syncthreads();
+  const int total = (part_tot[0][lane] + part_tot[1][lane]) + (part_tot[2][lane] + part_tot[3][lane]);
+  const int before = (part_bef[0][lane] + part_bef[1][lane]) + (part_bef[2][lane] + part_bef[3][lane]);
+  const int incl = wave_inclusive_scan(total);
+  const int excl = incl - total;
+  if (b == 0 && wave == 0) {
+    if (lane < E) { counts[lane] = total; offsets[lane] = excl; }
+    if (lane == E - 1) offsets[E] = incl;
+  }
+  int cnt = excl + before;                        // next free row of expert `lane` for this wave
+  for (int ww = 0; ww < wave; ++ww) cnt += wave_cnt[ww][lane];
+
+  for (int base = s0; base < s1; base += kWave) {
+    const int s = base + lane;
+    int e = 0;
+    bool valid = s < s1;
+    if (valid) { e = idx[s]; valid = (unsigned)e < (unsigned)E; }
+    if (!valid) e = 0;
+    unsigned long long peers, mine;
+    match64(e, valid, lane, peers, mine);
+    const int pos = __shfl(cnt, e, kWave) + __popcll(peers & lt);
     if (valid) { perm_slot[pos] = s; perm_token[pos] = s / k; }
     cnt += __popcll(mine);
   }
@@ -85,8 +116,8 @@ hipError_t launch_permute(const int32_t* idx, int T, int E, int k, int32_t* coun
   const int S = T * k;
   // T == 0 still has to produce counts = 0 and offsets = 0: one chunk with no slots does that.
   const int grid = nblk > 0 ? nblk : 1;
-  hipLaunchKernelGGL(hist_kernel, dim3(grid), dim3(64), 0, s, idx, S, E, k, block_hist);
-  hipLaunchKernelGGL(scatter_kernel, dim3(grid), dim3(64), 0, s, idx, S, E, k, block_hist, counts, offsets,
+  hipLaunchKernelGGL(hist_kernel, dim3(grid), dim3(256), 0, s, idx, S, E, k, block_hist);
+  hipLaunchKernelGGL(scatter_kernel, dim3(grid), dim3(256), 0, s, idx, S, E, k, block_hist, grid, counts, offsets,
                      perm_slot, perm_token);
   return hipGetLastError();
 }

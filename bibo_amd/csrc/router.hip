@@ -137,6 +137,91 @@ __global__ __launch_bounds__(256) void router_generic_kernel(const TIn* __restri
   }
 }
 
+// Cooperative selection: 16 lanes per token, lane `seg` owns experts 4*seg .. 4*seg+3.  k rounds of
+// "best remaining candidate": local scan in ascending expert order, then a 16-lane butterfly on
+// (value, expert) where the larger value wins and equal values go to the lower expert.  All 16 lanes
+// end every round with the same winner.  Returns the bit mask of the chosen experts.
+__device__ __forceinline__ unsigned long long select_mask16(const float (&v)[4], int seg, int rounds, float* kth,
+                                                            float* kth1) {
+  unsigned taken = 0;
+  unsigned long long mask = 0;
+  for (int r = 0; r < rounds; ++r) {
+    float bv = -INFINITY;
+    int be = kMaxE;
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      if (!((taken >> q) & 1) && (v[q] > bv || be == kMaxE)) { bv = v[q]; be = seg * 4 + q; }
+    if (taken == 0xf) { bv = -INFINITY; be = kMaxE; }
+#pragma unroll
+    for (int o = 1; o < 16; o <<= 1) {
+      const float ov = __shfl_xor(bv, o, kWave);
+      const int oe = __shfl_xor(be, o, kWave);
+      if (ov > bv || (ov == bv && oe < be)) { bv = ov; be = oe; }
+    }
+    be &= kMaxE - 1;
+    if ((be >> 2) == seg) taken |= 1u << (be & 3);
+    mask |= 1ull << be;
+    if (kth != nullptr) { if (r == rounds - 2) *kth = bv; if (r == rounds - 1) *kth1 = bv; }
+  }
+  return mask;
+}
+
+// Selection for the tokens of one workgroup whose scores sit in LDS rows `sc` (stride kRowPad):
+// thread = (token tid>>4, segment tid&15); needs blockDim.x >= 16 * ntok_max.
+__device__ __forceinline__ void select_tokens16(const float* __restrict__ sc, const float* __restrict__ bias_s, int E,
+                                                int k, int norm_mode, int t0, int ntok, int32_t* __restrict__ idx,
+                                                float* __restrict__ w, float* __restrict__ gap) {
+  const int tid = threadIdx.x;
+  const int tl = tid >> 4, seg = tid & 15;
+  const bool live = tl < ntok;                       // whole 16-lane groups are live or not
+  const float* row = sc + (live ? tl : 0) * kRowPad;
+  float v[4], u[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int e = seg * 4 + q;
+    u[q] = (e < E) ? row[e] : -INFINITY;
+    v[q] = (e < E) ? row[e] + bias_s[e] : -INFINITY;                      // router.py:38
+  }
+  const unsigned long long mask = select_mask16(v, seg, k, nullptr, nullptr);
+  float g_hi = 0.f, g_lo = 0.f;
+  if (gap != nullptr && k < E) select_mask16(u, seg, k + 1, &g_hi, &g_lo);   // router.py:33-36, unbiased scores
+  if (live && seg == 0) {
+    const int t = t0 + tl;
+    float raw[kMaxK];
+    float sum = 0.f, mx = -INFINITY;
+    unsigned long long m = mask;
+#pragma unroll
+    for (int j = 0; j < kMaxK; ++j) {
+      raw[j] = 0.f;
+      if (j < k) {
+        const int e = __ffsll((long long)m) - 1;                          // ascending expert order
+        m &= m - 1;
+        idx[(size_t)t * k + j] = e;
+        raw[j] = row[e];                                                  // UNBIASED score, router.py:41
+        sum += raw[j];
+        mx = fmaxf(mx, raw[j]);
+      }
+    }
+    float* wo = w + (size_t)t * k;
+    if (k > 1 && norm_mode == BIBO_NORM_SOFTMAX) {                        // router.py:42-43
+      float ex[kMaxK];
+      float es = 0.f;
+#pragma unroll
+      for (int j = 0; j < kMaxK; ++j) { ex[j] = (j < k) ? expf(raw[j] - mx) : 0.f; es += ex[j]; }
+#pragma unroll
+      for (int j = 0; j < kMaxK; ++j) if (j < k) wo[j] = ex[j] / es;
+    } else if (k > 1 && norm_mode == BIBO_NORM_SUM) {                     // router.py:44-45
+      const float den = sum + kSumNormEps;
+#pragma unroll
+      for (int j = 0; j < kMaxK; ++j) if (j < k) wo[j] = raw[j] / den;
+    } else {                                                              // router.py:46-47
+#pragma unroll
+      for (int j = 0; j < kMaxK; ++j) if (j < k) wo[j] = raw[j];
+    }
+    if (gap != nullptr) gap[t] = (k < E) ? (g_hi - g_lo) : 0.f;
+  }
+}
+
 // ---- MFMA router: bf16, H % 32 == 0 -------------------------------------------------------------
 // One workgroup = 16 tokens, 4 waves.  The waves split K (32-wide steps round-robin); each keeps
 // four 16x16 fp32 accumulators (64 experts), partials are summed through LDS in wave order.
@@ -164,14 +249,24 @@ __global__ __launch_bounds__(256) void router_mfma_kernel(const bf16_t* __restri
 #pragma unroll
   for (int nt = 0; nt < 4; ++nt) acc[nt] = floatx4{0.f, 0.f, 0.f, 0.f};
   const int nsteps = H / 32;
-  for (int s = wave; s < nsteps; s += 4) {
-    const int k0 = s * 32;
-    const bf16x8 a = *reinterpret_cast<const bf16x8*>(xa + k0);
+  constexpr int kU = 3;                                      // K steps whose loads are issued together
+  for (int s0 = wave; s0 < nsteps; s0 += 4 * kU) {
+    bf16x8 a[kU], b[kU][4];
 #pragma unroll
-    for (int nt = 0; nt < 4; ++nt) {
-      const bf16x8 b = *reinterpret_cast<const bf16x8*>(wb[nt] + k0);
-      acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[nt], 0, 0, 0);
+    for (int u = 0; u < kU; ++u) {
+      const int s = s0 + 4 * u;
+      if (s < nsteps) {
+        a[u] = *reinterpret_cast<const bf16x8*>(xa + s * 32);
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) b[u][nt] = *reinterpret_cast<const bf16x8*>(wb[nt] + s * 32);
+      }
     }
+#pragma unroll
+    for (int u = 0; u < kU; ++u)
+      if (s0 + 4 * u < nsteps) {
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b[u][nt], acc[nt], 0, 0, 0);
+      }
   }
   // D layout of the 16x16 tile: lane holds column (expert) lane%16, rows (tokens) 4*(lane/16)+i
 #pragma unroll
@@ -192,11 +287,7 @@ __global__ __launch_bounds__(256) void router_mfma_kernel(const bf16_t* __restri
     }
   }
   __syncthreads();
-  if (tid < ntok) {
-    const int t = t0 + tid;
-    select_row(sc + tid * kRowPad, bias_s, E, k, norm_mode, idx + (size_t)t * k, w + (size_t)t * k,
-               gap ? gap + t : nullptr);
-  }
+  select_tokens16(sc, bias_s, E, k, norm_mode, t0, ntok, idx, w, gap);
 }
 
 }  // namespace

@@ -119,6 +119,31 @@ def test_bf16_experts_reduced_prefill_and_ragged_shapes(T, H, I, bias, theta, al
     assert rel_err(out, ref) <= BF16_TOL
 
 
+@pytest.mark.parametrize("T,H,I,k,theta", [(64, 1024, 512, 6, "zero"), (7, 1024, 512, 6, "normal"), (1, 768, 384, 6, "normal"),
+                                           (200, 256, 128, 6, "normal"), (130, 128, 256, 2, "normal"),
+                                           (40, 64, 64, 1, "normal")])
+def test_streaming_kernels_match_oracle(T, H, I, k, theta):
+    """Weight-streaming (decode) kernels: few rows per expert, several 16-row passes, idle experts."""
+    p = O.make_inputs(T=T, H=H, E=64, k=k, I=I, bias="uniform", theta=theta, seed=T + I)
+    idx, w = _route(p)
+    ref = O.experts_forward(p["x"], idx, w, p["w_gate_up"], p["w_down"], p["theta"])
+    out, counts = _gpu_experts(p, idx, w, "stream")
+    assert rel_err(out, ref) <= BF16_TOL
+    assert np.array_equal(counts, O.permute(idx, 64)[0])
+    gen, _ = _gpu_experts(p, idx, w, "generic")
+    assert rel_err(out, gen) <= 1e-2
+
+
+def test_streaming_kernels_with_a_crowded_expert():
+    """Every row on two experts (far more than 16 rows each): the pass loop re-streams the weights."""
+    p = O.make_inputs(T=90, H=512, E=64, k=2, I=256, theta="normal", seed=21)
+    idx = np.tile(np.array([[3, 60]], np.int32), (90, 1))
+    w = np.random.default_rng(2).random((90, 2)).astype(np.float32)
+    ref = O.experts_forward(p["x"], idx, w, p["w_gate_up"], p["w_down"], p["theta"])
+    out, _ = _gpu_experts(p, idx, w, "stream")
+    assert rel_err(out, ref) <= BF16_TOL
+
+
 def test_mfma_and_generic_families_agree():
     p = O.make_inputs(T=777, H=768, E=64, k=6, I=384, bias="uniform", theta="normal", seed=5)
     idx, w = _route(p)

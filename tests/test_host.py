@@ -47,6 +47,8 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert lib.bibo_moe_router_fwd(None, None, None, 4, 64, 8, 2, 0, 1, None, None, None, None, None) == -1
     assert lib.bibo_moe_router_fwd(None, None, None, 4, 64, 8, 9, 0, 1, None, None, None, None, None) == -2
     assert lib.bibo_moe_gateup_fwd(None, None, None, None, None, 4, 64, 8, 2, 96, 0, L.ALGO_MFMA, None, None) == -6
+    # the streaming kernels exist only behind the composite entry points
+    assert lib.bibo_moe_gateup_fwd(None, None, None, None, None, 4, 1024, 64, 6, 512, 0, L.ALGO_STREAM, None, None) == -6
     assert lib.bibo_moe_permute(None, 4, 8, 2, None, None, None, None, None, 0, None) == -1
     assert b"workspace" in lib.bibo_moe_strerror(-4)
     with pytest.raises(RuntimeError, match="workspace"):
