@@ -50,11 +50,10 @@ int resolve_algo(int algo, int T, int H, int E, int k, int I, int dtype, bool co
 }
 
 struct Workspace {
-  size_t hist, idx, w, counts, offsets, perm_slot, perm_token, hidden, yw, total;
+  size_t hist, idx, w, counts, offsets, perm_slot, perm_token, hidden, gu, yw, total;
 };
 
 Workspace carve(int T, int H, int E, int k, int I, int dtype) {
-  (void)E;
   const size_t S = (size_t)T * k;
   Workspace ws;
   size_t o = 0;
@@ -65,10 +64,9 @@ Workspace carve(int T, int H, int E, int k, int I, int dtype) {
   ws.offsets = o;    o += align_up((kMaxE + 1) * sizeof(int32_t));
   ws.perm_slot = o;  o += align_up(S * sizeof(int32_t));
   ws.perm_token = o; o += align_up(S * sizeof(int32_t));
-  // `hidden` (permuted activations) and, for the streaming kernels, fp32 gate/up pre-activations share a segment
-  const size_t hidden_bytes = S * (size_t)I * elt_size(dtype);
-  const size_t gu_bytes = stream_supported(H, I, dtype) ? S * (size_t)2 * I * sizeof(float) : 0;
-  ws.hidden = o;     o += align_up(hidden_bytes > gu_bytes ? hidden_bytes : gu_bytes);
+  ws.hidden = o;     o += align_up(S * (size_t)I * elt_size(dtype));
+  // fp32 gate/up pre-activations, only ever used when the streaming kernels are eligible
+  ws.gu = o;         o += align_up(stream_eligible(T, H, E, k, I, dtype) ? S * (size_t)2 * I * sizeof(float) : 0);
   ws.yw = o;         o += align_up(S * (size_t)H * sizeof(float));
   ws.total = o;
   return ws;
@@ -109,10 +107,11 @@ int experts_dispatch(const void* x, const void* wgu, const void* wd, const float
   float* yw = reinterpret_cast<float*>(base + ws.yw);
   if (algo == BIBO_ALGO_STREAM) {
     if (!aligned16(x) || !aligned16(wgu) || !aligned16(wd)) return BIBO_ERR_MISALIGNED;
-    float* gu = reinterpret_cast<float*>(base + ws.hidden);
+    if (!stream_eligible(T, H, E, k, I, dtype)) return BIBO_ERR_UNSUPPORTED;     // no pre-activation segment carved
+    float* gu = reinterpret_cast<float*>(base + ws.gu);
     hipError_t e = launch_gateup_stream(x, wgu, offsets, perm_token, T, H, E, k, I, gu, s);
     if (e != hipSuccess) return (int)e;
-    e = launch_down_stream(gu, wd, theta, w, offsets, perm_slot, T, H, E, k, I, yw, s);
+    e = launch_down_stream(gu, wd, theta, w, offsets, perm_slot, T, H, E, k, I, base + ws.hidden, yw, s);
     if (e != hipSuccess) return (int)e;
     return hip_rc(launch_combine(yw, 0, T, H, k, dtype, out, s));
   }
@@ -244,14 +243,14 @@ int bibo_moe_forward(const void* x, const void* w_router, const float* bias, con
   hipStream_t s = static_cast<hipStream_t>(stream);
   int32_t* idx = idx_out ? idx_out : reinterpret_cast<int32_t*>(base + ws.idx);
   float* w = w_out ? w_out : reinterpret_cast<float*>(base + ws.w);
-  if (T > 0 &&
-      (rc = hip_rc(launch_router(x, w_router, bias, T, H, E, k, dtype, norm_mode, logits_out, idx, w, nullptr, s))) !=
-          BIBO_OK)
-    return rc;
   int32_t* counts = counts_out ? counts_out : reinterpret_cast<int32_t*>(base + ws.counts);
   int32_t* offsets = reinterpret_cast<int32_t*>(base + ws.offsets);
   int32_t* perm_slot = reinterpret_cast<int32_t*>(base + ws.perm_slot);
   int32_t* perm_token = reinterpret_cast<int32_t*>(base + ws.perm_token);
+  if (T > 0 &&
+      (rc = hip_rc(launch_router(x, w_router, bias, T, H, E, k, dtype, norm_mode, logits_out, idx, w, nullptr, s))) !=
+          BIBO_OK)
+    return rc;
   if ((rc = hip_rc(launch_permute(idx, T, E, k, counts, offsets, perm_slot, perm_token, base + ws.hist, s))) != BIBO_OK)
     return rc;
   if (T == 0) return BIBO_OK;

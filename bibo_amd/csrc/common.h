@@ -82,6 +82,21 @@ __device__ __forceinline__ float sigmoid32_canonical(float x) {
   return (float)(1.0 / d);
 }
 
+// Ballot ranking of 64 consecutive slots.  `peers` = lanes whose slot has my expert, `mine` = lanes whose
+// slot has the expert whose id is my lane id.
+__device__ __forceinline__ void match64(int e, bool valid, int lane, unsigned long long& peers,
+                                        unsigned long long& mine) {
+  const unsigned long long vmask = __ballot(valid);
+  peers = vmask;
+  mine = vmask;
+#pragma unroll
+  for (int bit = 0; bit < 6; ++bit) {
+    const unsigned long long bb = __ballot(valid && ((e >> bit) & 1));
+    peers &= ((e >> bit) & 1) ? bb : ~bb;
+    mine &= ((lane >> bit) & 1) ? bb : ~bb;
+  }
+}
+
 // Map a workgroup id to a tile so that the workgroups of one XCD (ids congruent mod 8 are dispatched
 // to the same XCD) walk a contiguous range of tiles: tiles of one expert then share that XCD's L2.
 __device__ __forceinline__ int xcd_tile(int bid, int total) {
@@ -116,6 +131,6 @@ hipError_t launch_gateup_stream(const void* x, const void* wgu, const int32_t* o
                                 int T, int H, int E, int k, int I, float* gu, hipStream_t s);
 hipError_t launch_down_stream(const float* gu, const void* wd, const float* theta, const float* w,
                               const int32_t* offsets, const int32_t* perm_slot, int T, int H, int E, int k, int I,
-                              float* yw, hipStream_t s);
+                              void* hidden, float* yw, hipStream_t s);
 
 }  // namespace bibo

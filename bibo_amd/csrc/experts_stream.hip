@@ -9,9 +9,9 @@
 // whole line; the token operand, staged in LDS, is read with the same K permutation.
 //
 //   gateup_stream_kernel : raw gate/up pre-activations  gu[row, 0..2I) fp32   (src/modeling/ffn/moe.py:84)
-//   down_stream_kernel   : prologue turns a row's gate/up into r^p SiLU(g/r) up (moe.py:87-92, needs the
-//                          whole gate row, which no single gate/up workgroup has), then streams w_down and
-//                          writes routing-weighted rows in slot order        (moe.py:92-93)
+//   activate_rows_kernel : hidden[row] = r^p SiLU(g/r) up; needs the whole gate row, which no single
+//                          gate/up workgroup has, hence its own tiny launch    (moe.py:87-92)
+//   down_stream_kernel   : streams w_down and writes routing-weighted rows in slot order (moe.py:92-93)
 #include "common.h"
 
 namespace bibo {
@@ -22,38 +22,44 @@ constexpr int kRowsPerWg = 64;     // weight rows per workgroup
 constexpr int kTok = 16;           // routed rows multiplied per pass
 constexpr int kLine = 64;          // bf16 elements per 128-byte line
 
-// Stream `kRowsPerWave` weight rows (row stride K elements) against 16 token rows held in LDS `xs`
-// (row stride K + 8 elements so the 16 lanes of a fragment read hit distinct banks).
-template <int UNROLL>
-__device__ __forceinline__ floatx4 stream_rows(const bf16_t* __restrict__ wrow, const bf16_t* xs, int K, int lane) {
+constexpr int kChunk = 4;          // 128-byte lines per register chunk (two chunks are alive: 64 VGPRs)
+
+struct WChunk {
+  bf16x8 w0[kChunk], w1[kChunk];
+};
+
+// this lane's 32 bytes of lines l .. l+kChunk-1 of its weight row (lines past nlines are skipped)
+__device__ __forceinline__ void load_chunk(WChunk& c, const bf16_t* __restrict__ wp, int l, int nlines) {
+#pragma unroll
+  for (int u = 0; u < kChunk; ++u)
+    if (l + u < nlines) {
+      c.w0[u] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(wp + (l + u) * kLine));
+      c.w1[u] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(wp + (l + u) * kLine + 8));
+    }
+}
+
+// Stream kRowsPerWave weight rows (row stride K) against 16 token rows held in LDS `xs` (row stride K + 8
+// elements, so the 16 lanes of a fragment read hit distinct banks).  `first` already holds lines 0..kChunk-1
+// (loaded before the token rows were staged); each further chunk is requested one chunk ahead of its use.
+__device__ __forceinline__ floatx4 stream_rows(const bf16_t* __restrict__ wrow, const bf16_t* xs, int K, int lane,
+                                               const WChunk& first) {
   const int g = lane >> 4;
   const bf16_t* wp = wrow + g * 16;                            // this lane's 32 bytes of every line
   const bf16_t* xp = xs + (lane & 15) * (K + 8) + g * 16;
   floatx4 acc = {0.f, 0.f, 0.f, 0.f};
   const int nlines = K / kLine;
-  int l = 0;
-  for (; l + UNROLL <= nlines; l += UNROLL) {
-    bf16x8 w0[UNROLL], w1[UNROLL];
+  WChunk cur = first, nxt;
+  for (int l = 0; l < nlines; l += kChunk) {
+    if (l + kChunk < nlines) load_chunk(nxt, wp, l + kChunk, nlines);
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      w0[u] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(wp + (l + u) * kLine));
-      w1[u] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(wp + (l + u) * kLine + 8));
-    }
-#pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      const bf16x8 x0 = *reinterpret_cast<const bf16x8*>(xp + (l + u) * kLine);
-      const bf16x8 x1 = *reinterpret_cast<const bf16x8*>(xp + (l + u) * kLine + 8);
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0[u], x0, acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1[u], x1, acc, 0, 0, 0);
-    }
-  }
-  for (; l < nlines; ++l) {
-    const bf16x8 w0 = *reinterpret_cast<const bf16x8*>(wp + l * kLine);
-    const bf16x8 w1 = *reinterpret_cast<const bf16x8*>(wp + l * kLine + 8);
-    const bf16x8 x0 = *reinterpret_cast<const bf16x8*>(xp + l * kLine);
-    const bf16x8 x1 = *reinterpret_cast<const bf16x8*>(xp + l * kLine + 8);
-    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0, x0, acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1, x1, acc, 0, 0, 0);
+    for (int u = 0; u < kChunk; ++u)
+      if (l + u < nlines) {
+        const bf16x8 x0 = *reinterpret_cast<const bf16x8*>(xp + (l + u) * kLine);
+        const bf16x8 x1 = *reinterpret_cast<const bf16x8*>(xp + (l + u) * kLine + 8);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.w0[u], x0, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.w1[u], x1, acc, 0, 0, 0);
+      }
+    cur = nxt;
   }
   return acc;
 }
@@ -66,11 +72,13 @@ __global__ __launch_bounds__(256) void gateup_stream_kernel(const bf16_t* __rest
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   bf16_t* xs = reinterpret_cast<bf16_t*>(smem_raw);            // [kTok][H + 8]
   const int e = blockIdx.y;
-  const int lo = offsets[e], hi = offsets[e + 1];
-  if (lo == hi) return;                                        // idle expert: its weights are never read
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int c0 = blockIdx.x * kRowsPerWg + wave * kRowsPerWave;  // first weight row of this wave
   const bf16_t* wrow = wgu + ((size_t)e * 2 * I + c0 + (lane & 15)) * H;
+  WChunk first;
+  load_chunk(first, wrow + (lane >> 4) * 16, 0, H / kLine);    // in flight while the token rows are staged
+  const int lo = offsets[e], hi = offsets[e + 1];
+  if (lo == hi) return;                                        // idle expert
   const int gran_per_row = H / 8;
   for (int r0 = lo; r0 < hi; r0 += kTok) {
     const int nrow = min(kTok, hi - r0);
@@ -82,7 +90,7 @@ __global__ __launch_bounds__(256) void gateup_stream_kernel(const bf16_t* __rest
       *reinterpret_cast<u32x4*>(xs + t * (H + 8) + c * 8) = v;
     }
     __syncthreads();
-    const floatx4 acc = stream_rows<4>(wrow, xs, H, lane);
+    const floatx4 acc = stream_rows(wrow, xs, H, lane, first);
     // accumulator: lane holds token lane%16, weight rows 4*(lane/16) + i
     const int t = lane & 15;
     if (t < nrow)
@@ -90,52 +98,59 @@ __global__ __launch_bounds__(256) void gateup_stream_kernel(const bf16_t* __rest
   }
 }
 
-// grid = (H / 64, E).  yw[slot(row), c] = w[slot] * (act(row) . w_down[e, c, :])
-__global__ __launch_bounds__(256) void down_stream_kernel(const float* __restrict__ gu, const bf16_t* __restrict__ wd,
-                                                          const float* __restrict__ theta, const float* __restrict__ w,
+// One workgroup per routed row: hidden[row] = r^p SiLU(g/r) up from the fp32 pre-activations (moe.py:87-92).
+__global__ __launch_bounds__(256) void activate_rows_kernel(const float* __restrict__ gu, const float* __restrict__ theta,
+                                                            const int32_t* __restrict__ offsets, int E, int I,
+                                                            bf16_t* __restrict__ hidden) {
+  __shared__ float red[4];
+  __shared__ int sh_e;
+  const int row = blockIdx.x;
+  if (row >= offsets[E]) return;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  if (tid < E && offsets[tid] <= row && row < offsets[tid + 1]) sh_e = tid;
+  const float* grow = gu + (size_t)row * 2 * I;
+  float ss = 0.f;
+  for (int i = tid; i < I; i += 256) ss = fmaf(grow[i], grow[i], ss);
+  ss = wave_sum(ss);
+  if (lane == 0) red[wave] = ss;
+  __syncthreads();
+  const float r2 = (((red[0] + red[1]) + red[2]) + red[3]) / (float)I + kNormSiluEps;    // moe.py:88
+  const float p = 1.f / (1.f + __expf(-theta[sh_e]));                                      // moe.py:89
+  const float rinv = rsqrtf(r2), gain = __expf(0.5f * p * __logf(r2));                     // 1/r, r^p
+  for (int i = tid; i < I; i += 256) {
+    const float z = grow[i] * rinv;
+    hidden[(size_t)row * I + i] = (bf16_t)(z / (1.f + __expf(-z)) * gain * grow[I + i]);
+  }
+}
+
+// grid = (H / 64, E).  yw[slot(row), c] = w[slot] * (hidden[row] . w_down[e, c, :])
+__global__ __launch_bounds__(256) void down_stream_kernel(const bf16_t* __restrict__ hidden, const bf16_t* __restrict__ wd,
+                                                          const float* __restrict__ w,
                                                           const int32_t* __restrict__ offsets,
                                                           const int32_t* __restrict__ perm_slot, int H, int I,
                                                           float* __restrict__ yw) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   bf16_t* hs = reinterpret_cast<bf16_t*>(smem_raw);            // [kTok][I + 8] activations of this pass
-  __shared__ float rinv_s[kTok], gain_s[kTok];
   const int e = blockIdx.y;
-  const int lo = offsets[e], hi = offsets[e + 1];
-  if (lo == hi) return;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int c0 = blockIdx.x * kRowsPerWg + wave * kRowsPerWave;
   const bf16_t* wrow = wd + ((size_t)e * H + c0 + (lane & 15)) * I;
-  const float p = 1.f / (1.f + __expf(-theta[e]));             // moe.py:89
+  WChunk first;
+  load_chunk(first, wrow + (lane >> 4) * 16, 0, I / kLine);
+  const int lo = offsets[e], hi = offsets[e + 1];
+  if (lo == hi) return;
+  const int gran_per_row = I / 8;
   for (int r0 = lo; r0 < hi; r0 += kTok) {
     const int nrow = min(kTok, hi - r0);
     __syncthreads();
-    // r = sqrt(mean(g^2) + eps) per row: one wave per 4 rows, lanes stride the I gate values (moe.py:88)
-    for (int t = wave; t < kTok; t += 4) {
-      float ss = 0.f;
-      if (t < nrow) {
-        const float* grow = gu + (size_t)(r0 + t) * 2 * I;
-        for (int i = lane; i < I; i += kWave) ss = fmaf(grow[i], grow[i], ss);
-      }
-      ss = wave_sum(ss);
-      if (lane == 0) {
-        const float r2 = ss / (float)I + kNormSiluEps;
-        rinv_s[t] = rsqrtf(r2);
-        gain_s[t] = __expf(0.5f * p * __logf(r2));             // r^p
-      }
+    for (int i = tid; i < kTok * gran_per_row; i += 256) {
+      const int t = i / gran_per_row, c = i - t * gran_per_row;
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (t < nrow) v = *reinterpret_cast<const u32x4*>(hidden + (size_t)(r0 + t) * I + c * 8);
+      *reinterpret_cast<u32x4*>(hs + t * (I + 8) + c * 8) = v;
     }
     __syncthreads();
-    for (int i = tid; i < kTok * I; i += 256) {
-      const int t = i / I, c = i - t * I;
-      float hval = 0.f;
-      if (t < nrow) {
-        const float* grow = gu + (size_t)(r0 + t) * 2 * I;
-        const float z = grow[c] * rinv_s[t];
-        hval = z / (1.f + __expf(-z)) * gain_s[t] * grow[I + c];   // SiLU(g/r) r^p up, moe.py:89-92
-      }
-      hs[t * (I + 8) + c] = (bf16_t)hval;
-    }
-    __syncthreads();
-    const floatx4 acc = stream_rows<4>(wrow, hs, I, lane);
+    const floatx4 acc = stream_rows(wrow, hs, I, lane, first);
     const int t = lane & 15;
     if (t < nrow) {
       const int slot = perm_slot[r0 + t];
@@ -166,11 +181,13 @@ hipError_t launch_gateup_stream(const void* x, const void* wgu, const int32_t* o
 
 hipError_t launch_down_stream(const float* gu, const void* wd, const float* theta, const float* w,
                               const int32_t* offsets, const int32_t* perm_slot, int T, int H, int E, int k, int I,
-                              float* yw, hipStream_t s) {
+                              void* hidden, float* yw, hipStream_t s) {
   if (T * k == 0) return hipSuccess;
+  bf16_t* hp = static_cast<bf16_t*>(hidden);
+  hipLaunchKernelGGL(activate_rows_kernel, dim3(T * k), dim3(256), 0, s, gu, theta, offsets, E, I, hp);
   const size_t shm = (size_t)kTok * (I + 8) * sizeof(bf16_t);
-  hipLaunchKernelGGL(down_stream_kernel, dim3(H / kRowsPerWg, E), dim3(256), shm, s, gu,
-                     static_cast<const bf16_t*>(wd), theta, w, offsets, perm_slot, H, I, yw);
+  hipLaunchKernelGGL(down_stream_kernel, dim3(H / kRowsPerWg, E), dim3(256), shm, s, hp,
+                     static_cast<const bf16_t*>(wd), w, offsets, perm_slot, H, I, yw);
   return hipGetLastError();
 }
 

@@ -24,21 +24,6 @@ __global__ __launch_bounds__(256) void hist_kernel(const int32_t* __restrict__ i
   if (tid < kMaxE) block_hist[blockIdx.x * kMaxE + tid] = h[tid];
 }
 
-// Ballot ranking of 64 consecutive slots.  `peers` = lanes whose slot has my expert, `mine` = lanes whose
-// slot has the expert whose id is my lane id.
-__device__ __forceinline__ void match64(int e, bool valid, int lane, unsigned long long& peers,
-                                        unsigned long long& mine) {
-  const unsigned long long vmask = __ballot(valid);
-  peers = vmask;
-  mine = vmask;
-#pragma unroll
-  for (int bit = 0; bit < 6; ++bit) {
-    const unsigned long long bb = __ballot(valid && ((e >> bit) & 1));
-    peers &= ((e >> bit) & 1) ? bb : ~bb;
-    mine &= ((lane >> bit) & 1) ? bb : ~bb;
-  }
-}
-
 // One workgroup per chunk of kPermTokens tokens, four waves of 64 tokens each, lane = expert for the
 // bookkeeping.  (1) every wave counts its own slots per expert; (2) the chunk histograms are summed
 // (all chunks for the totals, earlier chunks for this chunk's base) with the loads spread over the
@@ -102,6 +87,45 @@ __global__ __launch_bounds__(256) void scatter_kernel(const int32_t* __restrict_
   }
 }
 
+// Small inputs (T*k <= kSmallSlots): histogram, scan and scatter by ONE wave in one launch; the two
+// passes over the slots cost less than a second kernel launch.
+constexpr int kSmallSlots = 2048;
+
+__global__ __launch_bounds__(64) void permute_small_kernel(const int32_t* __restrict__ idx, int S, int E, int k,
+                                                           int32_t* __restrict__ counts, int32_t* __restrict__ offsets,
+                                                           int32_t* __restrict__ perm_slot,
+                                                           int32_t* __restrict__ perm_token) {
+  const int lane = threadIdx.x;
+  const unsigned long long lt = (1ull << lane) - 1ull;
+  int total = 0;
+  for (int base = 0; base < S; base += kWave) {
+    const int s = base + lane;
+    int e = 0;
+    bool valid = s < S;
+    if (valid) { e = idx[s]; valid = (unsigned)e < (unsigned)E; }
+    if (!valid) e = 0;
+    unsigned long long peers, mine;
+    match64(e, valid, lane, peers, mine);
+    total += __popcll(mine);
+  }
+  const int incl = wave_inclusive_scan(total);
+  int cnt = incl - total;
+  if (lane < E) { counts[lane] = total; offsets[lane] = cnt; }
+  if (lane == E - 1) offsets[E] = incl;
+  for (int base = 0; base < S; base += kWave) {
+    const int s = base + lane;
+    int e = 0;
+    bool valid = s < S;
+    if (valid) { e = idx[s]; valid = (unsigned)e < (unsigned)E; }
+    if (!valid) e = 0;
+    unsigned long long peers, mine;
+    match64(e, valid, lane, peers, mine);
+    const int pos = __shfl(cnt, e, kWave) + __popcll(peers & lt);
+    if (valid) { perm_slot[pos] = s; perm_token[pos] = s / k; }
+    cnt += __popcll(mine);
+  }
+}
+
 }  // namespace
 
 size_t permute_workspace_bytes(int T) {
@@ -114,8 +138,12 @@ hipError_t launch_permute(const int32_t* idx, int T, int E, int k, int32_t* coun
   const int nblk = (T + kPermTokens - 1) / kPermTokens;
   int32_t* block_hist = static_cast<int32_t*>(ws);
   const int S = T * k;
-  // T == 0 still has to produce counts = 0 and offsets = 0: one chunk with no slots does that.
-  const int grid = nblk > 0 ? nblk : 1;
+  if (S <= kSmallSlots) {          // also covers T == 0: counts and offsets come out all zero
+    hipLaunchKernelGGL(permute_small_kernel, dim3(1), dim3(64), 0, s, idx, S, E, k, counts, offsets, perm_slot,
+                       perm_token);
+    return hipGetLastError();
+  }
+  const int grid = nblk;
   hipLaunchKernelGGL(hist_kernel, dim3(grid), dim3(256), 0, s, idx, S, E, k, block_hist);
   hipLaunchKernelGGL(scatter_kernel, dim3(grid), dim3(256), 0, s, idx, S, E, k, block_hist, grid, counts, offsets,
                      perm_slot, perm_token);

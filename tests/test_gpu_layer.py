@@ -156,3 +156,22 @@ def test_experts_module_seam_takes_int64_indices():
         out = layer.experts(p["x"].to(DEV), torch.from_numpy(idx).long().to(DEV), torch.from_numpy(w).to(DEV))
     ref = O.experts_forward(p["x"], idx, w, p["w_gate_up"], p["w_down"], p["theta"])
     assert out.dtype == torch.bfloat16 and rel_err(out.cpu(), ref) <= 2e-2
+
+
+@pytest.mark.parametrize("T", [1, 17, 64, 65, 200])
+def test_fused_forward_routing_equals_standalone_router(T):
+    """bibo_moe_forward takes a one-launch router+permutation path for T <= 64; its routing, logits and
+    counts must equal the standalone router's bit for bit, and the output must match the oracle."""
+    from bibo_amd import ops
+    p = O.make_inputs(T=T, H=1024, E=64, k=6, I=512, bias="uniform", theta="normal", seed=100 + T)
+    d = {k_: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k_, v in p.items()}
+    out, idx, w, counts, logits = ops.moe_forward(d["x"], d["w_router"], d["bias"], d["w_gate_up"], d["w_down"],
+                                                  d["theta"], 6, want_routing=True, want_counts=True, want_logits=True)
+    idx2, w2, logits2, _ = ops.router_fwd(d["x"], d["w_router"], d["bias"], 6, want_logits=True)
+    torch.cuda.synchronize()
+    assert torch.equal(logits, logits2) and torch.equal(idx, idx2) and torch.equal(w, w2)
+    oi, ow, _ = O.route_from_logits(logits.cpu().numpy(), p["bias"].numpy(), 6)
+    assert np.array_equal(idx.cpu().numpy(), oi) and np.array_equal(w.cpu().numpy(), ow)
+    assert np.array_equal(counts.cpu().numpy(), O.permute(oi, 64)[0])
+    ref = O.experts_forward(p["x"], oi, ow, p["w_gate_up"], p["w_down"], p["theta"])
+    assert rel_err(out.cpu(), ref) <= 2e-2
