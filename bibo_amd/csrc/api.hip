@@ -91,7 +91,7 @@ int down_dispatch(const void* hidden, const void* wd, const float* w, const int3
     if (!aligned16(hidden) || !aligned16(wd)) return BIBO_ERR_MISALIGNED;
     // weighted expert outputs travel to the combine in bf16 (the reference's bf16 eager path rounds each
     // expert output to bf16 as well, moe.py:92)
-    e = launch_down_mfma(hidden, wd, w, offsets, perm_slot, T, H, E, k, I, yw, /*yw_is_bf16=*/1, s);
+    e = launch_down_mfma(hidden, wd, w, offsets, perm_slot, T, H, E, k, I, yw, s);
     if (e != hipSuccess) return (int)e;
     return hip_rc(launch_combine(yw, 1, T, H, k, dtype, out, s));
   }

@@ -123,8 +123,7 @@ bool mfma_supported(int H, int I, int dtype);
 hipError_t launch_gateup_mfma(const void* x, const void* wgu, const float* theta, const int32_t* offsets,
                               const int32_t* perm_token, int T, int H, int E, int k, int I, void* hidden, hipStream_t s);
 hipError_t launch_down_mfma(const void* hidden, const void* wd, const float* w, const int32_t* offsets,
-                            const int32_t* perm_slot, int T, int H, int E, int k, int I, void* yw, int yw_is_bf16,
-                            hipStream_t s);
+                            const int32_t* perm_slot, int T, int H, int E, int k, int I, void* yw, hipStream_t s);
 
 bool stream_supported(int H, int I, int dtype);
 hipError_t launch_gateup_stream(const void* x, const void* wgu, const int32_t* offsets, const int32_t* perm_token,
