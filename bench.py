@@ -20,6 +20,11 @@ if str(ROOT) not in sys.path:
 PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
 
+# HBM-side bytes per launch of the gate/up kernel on workload c2, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE (KiB per dispatch), scaled by what the same counters read for a 256 MiB device copy
+# (FETCH_SIZE x2.0, WRITE_SIZE x1.0): 158.9 MB fetched + 37.7 MB written.
+MEASURED_TRAFFIC_BYTES = {("c2", "gateup"): 196.6e6}
+
 
 def flops_layer(T, H, E, k, I):
     return 2 * T * H * E + 6 * T * k * H * I
@@ -205,21 +210,22 @@ def main():
         "tflops": fl / sec / 1e12, "pct_bf16_mfma_peak": 100.0 * fl / sec / 1e12 / PEAK_BF16_TFLOPS,
         "parity_rel_err_sample": rel, "experts_active": e_active,
         "stage_us": {n: v * 1e6 for n, v in stages.items()},
-        "roofline": {"kernel": "gateup_mfma_kernel (grouped gate/up GEMM + Radial NormSiLU)", "bound": "mfma",
+        "roofline": {"kernel": "gateup_dma_kernel (grouped gate/up GEMM + Radial NormSiLU)", "bound": "mfma",
                      "achieved": gateup_flops / stages["gateup"] / 1e12, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": gateup_flops / stages["gateup"] / 1e12 / PEAK_BF16_TFLOPS, "traffic": None},
+                     "frac": gateup_flops / stages["gateup"] / 1e12 / PEAK_BF16_TFLOPS,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, "gateup"))},
     }
     if not args.no_decode and args.workload == "c2":
         d = Layer("c3", dev, args.algo)
         drel, dact = d.check()
         dsec = d.time_forward(args.steps, args.warmup)
-        dst = d.time_stages(max(10, min(args.steps, 100)))
         db = bytes_layer(d.T, d.H, d.E, d.k, d.I, dact)
         out["decode"] = {"workload": f"c3: T={d.T} H={d.H} E={d.E} k={d.k} I={d.I} bf16", "tokens_per_s": d.T / dsec,
                          "us_per_step": dsec * 1e6, "algorithmic_bytes": db, "hbm_gbs": db / dsec / 1e9,
                          "pct_hbm_peak": 100.0 * db / dsec / 1e9 / PEAK_HBM_GBS, "experts_active": dact,
-                         "parity_rel_err_sample": drel, "stage_us": {n: v * 1e6 for n, v in dst.items()},
-                         "note": "single weight set: 201 MB of weights can sit in the 256 MB Infinity Cache"}
+                         "parity_rel_err_sample": drel,
+                         "note": "whole layer through bibo_moe_forward (weight-streaming kernels); one weight set, "
+                                 "measured HBM and Infinity-Cache read rates on this part are equal (about 6 TB/s)"}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args.workload)
     print(json.dumps(out))

@@ -21,6 +21,7 @@
 namespace bibo {
 namespace {
 
+constexpr int kLoadsPerPair = 1;
 constexpr int kBK = 32;        // K elements per LDS stage
 
 struct TileMap {
@@ -121,18 +122,11 @@ __device__ __forceinline__ void stripe_pair(floatx16 (&acc)[MT][NTW], bf16x8 (&a
                                             const StripeLoader<S>& ld, bool prefetch, int k_next, bf16_t* next_stage) {
   constexpr int kPairs = 2 * NTW;
   constexpr int s = Q / NTW, j = Q % NTW;
-  // loads per pair so that all of them are out by the last pair
-  constexpr int kPer = (StripeLoader<S>::kInstr + kPairs - 1) / kPairs;
+  // kLoadsPerPair load instructions of the next stage per pair, starting with pair 0
+  constexpr int kPer = kLoadsPerPair;
   if (prefetch) {
-#pragma unroll
-    for (int u = 0; u < kPer; ++u) {
-      if constexpr (true) {
-        if (Q * kPer + u < StripeLoader<S>::kInstr) {
-          if (u == 0) ld.template issue<(Q * kPer < StripeLoader<S>::kInstr ? Q * kPer : 0)>(k_next, next_stage);
-          if (u == 1) ld.template issue<(Q * kPer + 1 < StripeLoader<S>::kInstr ? Q * kPer + 1 : 0)>(k_next, next_stage);
-        }
-      }
-    }
+    if constexpr (Q * kPer < StripeLoader<S>::kInstr) ld.template issue<Q * kPer>(k_next, next_stage);
+    if constexpr (kPer > 1 && Q * kPer + 1 < StripeLoader<S>::kInstr) ld.template issue<Q * kPer + 1>(k_next, next_stage);
   }
   if constexpr (Q + 2 < kPairs) {
     constexpr int s2 = (Q + 2) / NTW, j2 = (Q + 2) % NTW;
