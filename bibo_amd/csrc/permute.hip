@@ -95,34 +95,41 @@ __global__ __launch_bounds__(64) void permute_small_kernel(const int32_t* __rest
                                                            int32_t* __restrict__ counts, int32_t* __restrict__ offsets,
                                                            int32_t* __restrict__ perm_slot,
                                                            int32_t* __restrict__ perm_token) {
+  constexpr int kChunks = kSmallSlots / kWave;
   const int lane = threadIdx.x;
   const unsigned long long lt = (1ull << lane) - 1ull;
+  int ev[kChunks];                                 // every slot's expert, fetched up front: one memory latency
+#pragma unroll
+  for (int c = 0; c < kChunks; ++c) {
+    const int s = c * kWave + lane;
+    ev[c] = (s < S) ? idx[s] : -1;
+  }
   int total = 0;
-  for (int base = 0; base < S; base += kWave) {
-    const int s = base + lane;
-    int e = 0;
-    bool valid = s < S;
-    if (valid) { e = idx[s]; valid = (unsigned)e < (unsigned)E; }
-    if (!valid) e = 0;
-    unsigned long long peers, mine;
-    match64(e, valid, lane, peers, mine);
-    total += __popcll(mine);
+#pragma unroll
+  for (int c = 0; c < kChunks; ++c) {
+    if (c * kWave < S) {
+      const bool valid = (unsigned)ev[c] < (unsigned)E;
+      unsigned long long peers, mine;
+      match64(valid ? ev[c] : 0, valid, lane, peers, mine);
+      total += __popcll(mine);
+    }
   }
   const int incl = wave_inclusive_scan(total);
   int cnt = incl - total;
   if (lane < E) { counts[lane] = total; offsets[lane] = cnt; }
   if (lane == E - 1) offsets[E] = incl;
-  for (int base = 0; base < S; base += kWave) {
-    const int s = base + lane;
-    int e = 0;
-    bool valid = s < S;
-    if (valid) { e = idx[s]; valid = (unsigned)e < (unsigned)E; }
-    if (!valid) e = 0;
-    unsigned long long peers, mine;
-    match64(e, valid, lane, peers, mine);
-    const int pos = __shfl(cnt, e, kWave) + __popcll(peers & lt);
-    if (valid) { perm_slot[pos] = s; perm_token[pos] = s / k; }
-    cnt += __popcll(mine);
+#pragma unroll
+  for (int c = 0; c < kChunks; ++c) {
+    if (c * kWave < S) {
+      const int s = c * kWave + lane;
+      const bool valid = (unsigned)ev[c] < (unsigned)E;
+      const int e = valid ? ev[c] : 0;
+      unsigned long long peers, mine;
+      match64(e, valid, lane, peers, mine);
+      const int pos = __shfl(cnt, e, kWave) + __popcll(peers & lt);
+      if (valid) { perm_slot[pos] = s; perm_token[pos] = s / k; }
+      cnt += __popcll(mine);
+    }
   }
 }
 

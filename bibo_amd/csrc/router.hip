@@ -249,7 +249,7 @@ __global__ __launch_bounds__(256) void router_mfma_kernel(const bf16_t* __restri
 #pragma unroll
   for (int nt = 0; nt < 4; ++nt) acc[nt] = floatx4{0.f, 0.f, 0.f, 0.f};
   const int nsteps = H / 32;
-  constexpr int kU = 3;                                      // K steps whose loads are issued together
+  constexpr int kU = 8;                                      // K steps whose loads are issued together (160 VGPRs)
   for (int s0 = wave; s0 < nsteps; s0 += 4 * kU) {
     bf16x8 a[kU], b[kU][4];
 #pragma unroll
