@@ -26,11 +26,13 @@ inline bool stream_eligible(int T, int H, int E, int k, int I, int dtype) {
 }
 
 // `composite`: the caller is bibo_moe_experts_fwd / bibo_moe_forward, the only entry points that can run
-// the streaming kernels (they hand fp32 pre-activations, not `hidden`, from one kernel to the next).
+// the streaming kernels (they hand fp32 pre-activations, not `hidden`, from one kernel to the next) and
+// the fused kernel (its activations never reach memory).
 int resolve_algo(int algo, int T, int H, int E, int k, int I, int dtype, bool composite, int* out) {
   switch (algo) {
     case BIBO_ALGO_AUTO:
       if (composite && stream_eligible(T, H, E, k, I, dtype)) *out = BIBO_ALGO_STREAM;
+      else if (composite && fused_supported(H, I, dtype)) *out = BIBO_ALGO_FUSED;
       else *out = mfma_supported(H, I, dtype) ? BIBO_ALGO_MFMA : BIBO_ALGO_GENERIC;
       break;
     case BIBO_ALGO_GENERIC: *out = BIBO_ALGO_GENERIC; break;
@@ -41,6 +43,10 @@ int resolve_algo(int algo, int T, int H, int E, int k, int I, int dtype, bool co
     case BIBO_ALGO_STREAM:
       if (!composite || !stream_supported(H, I, dtype)) return BIBO_ERR_UNSUPPORTED;
       *out = BIBO_ALGO_STREAM;
+      break;
+    case BIBO_ALGO_FUSED:
+      if (!composite || !fused_supported(H, I, dtype)) return BIBO_ERR_UNSUPPORTED;
+      *out = BIBO_ALGO_FUSED;
       break;
     default: return BIBO_ERR_UNSUPPORTED;
   }
@@ -114,6 +120,12 @@ int experts_dispatch(const void* x, const void* wgu, const void* wd, const float
     e = launch_down_stream(gu, wd, theta, w, offsets, perm_slot, T, H, E, k, I, base + ws.hidden, yw, s);
     if (e != hipSuccess) return (int)e;
     return hip_rc(launch_combine(yw, 0, T, H, k, dtype, out, s));
+  }
+  if (algo == BIBO_ALGO_FUSED) {
+    if (!aligned16(x) || !aligned16(wgu) || !aligned16(wd)) return BIBO_ERR_MISALIGNED;
+    hipError_t e = launch_experts_fused(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, T, H, E, k, I, yw, s);
+    if (e != hipSuccess) return (int)e;
+    return hip_rc(launch_combine(yw, 1, T, H, k, dtype, out, s));
   }
   const int rc = gateup_dispatch(x, wgu, theta, offsets, perm_token, T, H, E, k, I, dtype, algo, base + ws.hidden, s);
   if (rc != BIBO_OK) return rc;
@@ -196,6 +208,30 @@ int bibo_moe_down_combine_fwd(const void* hidden, const void* w_down, const floa
   if (workspace_bytes < (size_t)T * k * H * sizeof(float)) return BIBO_ERR_WORKSPACE_TOO_SMALL;
   return down_dispatch(hidden, w_down, w, offsets, perm_slot, T, H, E, k, I, dtype, a, out,
                        static_cast<float*>(workspace), static_cast<hipStream_t>(stream));
+}
+
+int bibo_moe_gateup_down_fwd(const void* x, const void* w_gate_up, const void* w_down, const float* theta,
+                             const float* w, const int32_t* offsets, const int32_t* perm_slot,
+                             const int32_t* perm_token, int T, int H, int E, int k, int I, int dtype, void* yw,
+                             void* stream) {
+  const int rc = check_dims(T, H, E, k, I, dtype);
+  if (rc != BIBO_OK) return rc;
+  if (!fused_supported(H, I, dtype)) return BIBO_ERR_UNSUPPORTED;
+  if (T == 0) return BIBO_OK;
+  if (!x || !w_gate_up || !w_down || !theta || !w || !offsets || !perm_slot || !perm_token || !yw)
+    return BIBO_ERR_NULL_POINTER;
+  if (!aligned16(x) || !aligned16(w_gate_up) || !aligned16(w_down) || !aligned16(yw)) return BIBO_ERR_MISALIGNED;
+  return hip_rc(launch_experts_fused(x, w_gate_up, w_down, theta, w, offsets, perm_slot, perm_token, T, H, E, k, I, yw,
+                                     static_cast<hipStream_t>(stream)));
+}
+
+int bibo_moe_combine_fwd(const void* yw, int yw_is_bf16, int T, int H, int k, int dtype, void* out, void* stream) {
+  const int rc = check_dims(T, H, k, k, 1, dtype);   // no expert dimension here: E := k, I := 1 pass the range checks
+  if (rc != BIBO_OK) return rc;
+  if (yw_is_bf16 && dtype != BIBO_DTYPE_BF16) return BIBO_ERR_BAD_DTYPE;
+  if (T == 0) return BIBO_OK;
+  if (!yw || !out) return BIBO_ERR_NULL_POINTER;
+  return hip_rc(launch_combine(yw, yw_is_bf16 ? 1 : 0, T, H, k, dtype, out, static_cast<hipStream_t>(stream)));
 }
 
 int bibo_moe_experts_fwd(const void* x, const int32_t* idx, const float* w, const void* w_gate_up, const void* w_down,

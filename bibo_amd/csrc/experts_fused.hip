@@ -1,0 +1,290 @@
+// Kernels 3 and 4 in one launch: a workgroup takes 128 permuted rows of one expert through the gate/up
+// projection, Radial NormSiLU and the down projection without the activations leaving the CU.
+//
+// Phase 1 is the gate/up main loop of gateup_dma_kernel (x rows and w_gate_up rows by LDS-DMA, two
+// stages `P` and `Q`).  Phase 2 turns the accumulators into bf16 activations and parks them in LDS as an
+// operand of the second GEMM: rows 0..63 live in P, rows 64..127 in Q, whose stage contents are dead by
+// then; row r keeps 16-byte granule c at position c ^ (r & 15), which spreads the 16 lanes of a fragment
+// read over all banks although the row stride is a multiple of 256 bytes.
+// Phase 3 has no barriers and no LDS traffic for the weights: the eight waves split a block of 128*CT
+// output columns (16*CT each), every wave multiplies ALL 128 resident rows with v_mfma_f32_16x16x32_bf16
+// and pulls its own w_down rows straight from global memory into registers, up to three 128-byte K
+// blocks ahead (lane (r, g) takes bytes [32g, 32g+32) of each line of weight row r; the activation fragments
+// are read with the same K permutation).  Keeping the in-flight bytes in registers instead of LDS is
+// what lets a CU cover the memory latency here: the activations already fill most of the LDS.
+// Each block of columns is scaled by the routing weight, staged through LDS 64 rows at a time and
+// scattered to slot order as whole 16-byte row segments.
+// Reference: BiBoFusedExperts.forward, src/modeling/ffn/moe.py:81-93.
+#include "stripe.h"
+
+namespace bibo {
+namespace {
+
+template <int NT, int CT>
+struct FusedShape {
+  static constexpr int MT = 2, WM = 2, BM = 128;
+  static constexpr int I = 128 * NT;
+  static constexpr int BN2 = 128 * CT;                             // output columns per block: 8 waves x CT x 16
+  using S1 = Stripe<MT, 2 * NT, WM>;
+  static constexpr int kHalfElems = 64 * I;                        // activations of one M half
+  static constexpr int kTailElems = S1::kStageElems - kHalfElems;  // = 4096: free behind the activations
+  static constexpr int kOutElems = 64 * BN2;                       // output staging: 64 rows of a column block
+  static_assert(kTailElems * 2 >= 4 * BM * 4 + 4 * BM * 4, "row scalars do not fit behind the activations");
+};
+
+// this lane's 32 bytes of one 128-byte K block for each of its CT weight tiles
+template <int CT>
+struct WBlock {
+  bf16x8 w[CT][2];
+};
+
+template <int CT>
+__device__ __forceinline__ void load_wblock(WBlock<CT>& b, const bf16_t* __restrict__ wp, size_t tile_stride, int kb) {
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    const bf16_t* p = wp + ct * tile_stride + kb * 64;
+    b.w[ct][0] = *reinterpret_cast<const bf16x8*>(p);
+    b.w[ct][1] = *reinterpret_cast<const bf16x8*>(p + 8);
+  }
+}
+
+template <int NT, int CT>
+__global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wgu,
+                                                            const bf16_t* __restrict__ wd,
+                                                            const float* __restrict__ theta,
+                                                            const float* __restrict__ w,
+                                                            const int32_t* __restrict__ offsets,
+                                                            const int32_t* __restrict__ perm_slot,
+                                                            const int32_t* __restrict__ perm_token, int H, int E,
+                                                            bf16_t* __restrict__ yw) {
+  using F = FusedShape<NT, CT>;
+  using S1 = typename F::S1;
+  constexpr int MT = F::MT, BM = F::BM, I = F::I, NTW = 2 * NT;
+  __shared__ __attribute__((aligned(16))) bf16_t P[S1::kStageElems];
+  __shared__ __attribute__((aligned(16))) bf16_t Q[S1::kStageElems];
+  __shared__ __attribute__((aligned(16))) bf16_t O[F::kOutElems];
+  // row scalars, behind the activations of M half 0 (valid from phase 2 on)
+  float* ssq = reinterpret_cast<float*>(P + F::kHalfElems);        // [4][BM]
+  float* rinv_s = ssq + 4 * BM;                                    // [BM]
+  float* gain_s = rinv_s + BM;                                     // [BM]
+  float* w_s = gain_s + BM;                                        // [BM]
+  int* slot_s = reinterpret_cast<int*>(w_s + BM);                  // [BM]
+
+  const TileMap tm = make_tile_map(offsets, E, BM);
+  const int tile = xcd_tile(blockIdx.x, tm.total);
+  if (tile >= tm.total) return;
+  int e, row0, rows;
+  find_tile(tm, offsets, BM, tile, e, row0, rows);
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int wn = wave & 3, wm = wave >> 2;
+  const int n = lane & 31;
+  const int chunk = dma_chunk(tid);
+  const int mbase = wm * MT * 32;
+
+  // ---- phase 1: gate/up projection (moe.py:81-86) ----
+  floatx16 acc[MT][NTW];
+  {
+    StripeLoader<S1> ld;
+#pragma unroll
+    for (int i = 0; i < S1::A_PER; ++i) {
+      const int m = min((tid >> 2) + i * (S1::kThreads / 4), rows - 1);   // rows past the end re-read the last valid row
+      ld.a_src[i] = x + (size_t)perm_token[row0 + m] * H + chunk * 8;
+    }
+    ld.b_src = wgu + ((size_t)e * 2 * I + (tid >> 2)) * H + chunk * 8;
+    ld.bstep = (size_t)(S1::kThreads / 4) * H;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int j = 0; j < NTW; ++j)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[mt][j][i] = 0.f;
+    auto frag_row = [&](int j) { return (j < NT ? 0 : I) + (wn * NT + (j < NT ? j : j - NT)) * 32; };
+    stripe_mainloop_dma<MT, NTW, F::WM>(acc, ld, H, P, Q, wm, frag_row);
+  }
+  __syncthreads();                         // every wave is done with the gate/up stages
+
+  // ---- phase 2: Radial NormSiLU (moe.py:87-92), activations to LDS ----
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      float sq = 0.f;
+#pragma unroll
+      for (int j = 0; j < NT; ++j) sq = fmaf(acc[mt][j][i], acc[mt][j][i], sq);
+#pragma unroll
+      for (int o = 16; o > 0; o >>= 1) sq += __shfl_xor(sq, o, kWave);
+      if (n == 0) ssq[wn * BM + mbase + mt * 32 + acc_row(i, lane)] = sq;
+    }
+  __syncthreads();
+  if (tid < BM) {
+    const float p = 1.f / (1.f + __expf(-theta[e]));                                  // moe.py:89
+    const float ms = ((ssq[tid] + ssq[BM + tid]) + ssq[2 * BM + tid]) + ssq[3 * BM + tid];
+    const float r2 = ms * (1.f / (float)I) + kNormSiluEps;                            // r^2, moe.py:88
+    rinv_s[tid] = __builtin_amdgcn_rsqf(r2);
+    gain_s[tid] = __builtin_amdgcn_exp2f(0.5f * p * __builtin_amdgcn_logf(r2));       // r^p
+    const int slot = perm_slot[row0 + min(tid, rows - 1)];
+    slot_s[tid] = slot;
+    w_s[tid] = w[slot];
+  }
+  __syncthreads();
+  {
+    bf16_t* hsel = wm ? Q : P;             // activations of this wave's M half, [64][I], granules swizzled
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int ml = mt * 32 + acc_row(i, lane);
+        const float rinv = rinv_s[mbase + ml], gain = gain_s[mbase + ml];
+        bf16_t* hrow = hsel + ml * I + (n & 7);
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+          const float z = acc[mt][j][i] * rinv;
+          const float sg = __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-1.44269504f * z));
+          const int c = (wn * NT + j) * 4 + (n >> 3);                                   // logical granule of this column
+          hrow[(c ^ (ml & 15)) * 8] = (bf16_t)(z * sg * gain * acc[mt][NT + j][i]);     // SiLU(g/r) r^p up
+        }
+      }
+  }
+  __syncthreads();                         // the activation tile is complete
+
+  // ---- phase 3: down projection, routing weight, scatter to slot order (moe.py:92-93) ----
+  constexpr int KB = I / 64;                 // 128-byte K blocks
+  constexpr int G = F::BN2 / 8;              // 16-byte granules per staged output row
+  const int r16 = lane & 15, g4 = lane >> 4;
+  const size_t tile_stride = (size_t)16 * I;
+  // activation fragment of row tile rt, K block kb, half s: granule (8*kb + 2*g4 + s) ^ r16 of row 16*rt + r16
+  const int nblk = H / F::BN2;
+  const bf16_t* wp = wd + ((size_t)e * H + wave * (16 * CT) + r16) * I + g4 * 16;
+  constexpr int D = KB > 3 ? 3 : KB - 1;      // K blocks requested ahead of the one being multiplied
+  constexpr int NB = D + 1;
+  WBlock<CT> wb[NB];
+#pragma unroll
+  for (int d = 0; d < D; ++d) load_wblock<CT>(wb[d], wp, tile_stride, d);
+  for (int nb = 0; nb < nblk; ++nb) {
+    const int n0 = nb * F::BN2;
+    floatx4 acc2[CT][8];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+      for (int rt = 0; rt < 8; ++rt) acc2[ct][rt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    // Activation fragments are read one row tile ahead of the MFMAs that consume them (the fragments of
+    // row tile 0 of the next K block are requested before this block's last MFMAs).
+    auto frag = [&](int kb, int rt, int s) {
+      const int gq = (((kb * 8 + 2 * g4) ^ r16) * 8) ^ (s * 8);
+      return *reinterpret_cast<const bf16x8*>((rt < 4 ? P : Q) + ((rt & 3) * 16 + r16) * I + gq);
+    };
+    bf16x8 xa[2][2];
+    xa[0][0] = frag(0, 0, 0);
+    xa[0][1] = frag(0, 0, 1);
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb) {
+      if (kb + D < KB) load_wblock<CT>(wb[(kb + D) % NB], wp, tile_stride, kb + D);
+      __builtin_amdgcn_sched_barrier(0);     // keep the loads D blocks ahead of their use
+#pragma unroll
+      for (int rt = 0; rt < 8; ++rt) {
+        const int cur = rt & 1, nxt = cur ^ 1;
+        if (rt + 1 < 8) {
+          xa[nxt][0] = frag(kb, rt + 1, 0);
+          xa[nxt][1] = frag(kb, rt + 1, 1);
+        } else if (kb + 1 < KB) {
+          xa[nxt][0] = frag(kb + 1, 0, 0);
+          xa[nxt][1] = frag(kb + 1, 0, 1);
+        }
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+          for (int ct = 0; ct < CT; ++ct)
+            acc2[ct][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb[kb % NB].w[ct][s], xa[cur][s], acc2[ct][rt], 0, 0, 0);
+        if (rt + 1 < 8 || kb + 1 < KB) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 2 * CT, 0);
+      }
+    }
+    wp += (size_t)F::BN2 * I;                                  // next block of columns: in flight during the epilogue
+    if (nb + 1 < nblk) {
+#pragma unroll
+      for (int d = 0; d < D; ++d) load_wblock<CT>(wb[d], wp, tile_stride, d);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // accumulator: lane holds row 16*rt + r16, columns wave*16*CT + 16*ct + 4*g4 + i.  Staged row r keeps
+    // granule c at position c ^ (r & 15): the 8-byte writes of a half wave then cover all banks.
+    // (The thread index goes through an empty asm so the staging addresses are formed here, per block,
+    // instead of being hoisted out of the loop and kept alive across the multiply.)
+    int tid_o = tid;
+    asm volatile("" : "+v"(tid_o));
+    const int r16o = tid_o & 15, g4o = (tid_o >> 4) & 3;
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+      __syncthreads();                       // the previous copy-out is done with O
+#pragma unroll
+      for (int rq = 0; rq < 4; ++rq) {
+        const int rt = hf * 4 + rq;
+        const float ws = w_s[rt * 16 + r16o];                                            // moe.py:93
+        bf16_t* orow = O + (rq * 16 + r16o) * F::BN2 + (g4o & 1) * 4;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+          const int c = wave * (2 * CT) + ct * 2 + (g4o >> 1);
+          bf16x4 v;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) v[i] = (bf16_t)(ws * acc2[ct][rt][i]);
+          *reinterpret_cast<bf16x4*>(orow + (c ^ r16o) * 8) = v;
+        }
+      }
+      __syncthreads();
+#pragma unroll
+      for (int q = 0; q < 64 * G / 512; ++q) {
+        const int idx = q * 512 + tid_o;
+        const int r = idx / G, pc = idx - r * G;
+        const int m = hf * 64 + r;
+        if (m < rows)
+          *reinterpret_cast<u32x4*>(yw + (size_t)slot_s[m] * H + n0 + (pc ^ (r & 15)) * 8) =
+              *reinterpret_cast<const u32x4*>(O + r * F::BN2 + pc * 8);
+      }
+    }
+  }
+}
+
+template <int NT, int CT>
+void launch_fused_t(const bf16_t* x, const bf16_t* wgu, const bf16_t* wd, const float* theta, const float* w,
+                    const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token, int S, int H, int E,
+                    bf16_t* yw, hipStream_t s) {
+  const int grid = ((S / 128 + E + 7) & ~7) + 8;
+  hipLaunchKernelGGL((experts_fused_kernel<NT, CT>), dim3(grid), dim3(512), 0, s, x, wgu, wd, theta, w, offsets,
+                     perm_slot, perm_token, H, E, yw);
+}
+
+template <int NT>
+void launch_fused_nt(const bf16_t* x, const bf16_t* wgu, const bf16_t* wd, const float* theta, const float* w,
+                     const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token, int S, int H, int E,
+                     bf16_t* yw, hipStream_t s) {
+  if (H % 384 == 0) launch_fused_t<NT, 3>(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, S, H, E, yw, s);
+  else if (H % 256 == 0) launch_fused_t<NT, 2>(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, S, H, E, yw, s);
+  else launch_fused_t<NT, 1>(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, S, H, E, yw, s);
+}
+
+}  // namespace
+
+bool fused_supported(int H, int I, int dtype) {
+  // the activation tile plus two weight stages have to fit 160 KB of LDS: I <= 384
+  return dtype == BIBO_DTYPE_BF16 && H >= 128 && (H % 128) == 0 && (I == 128 || I == 256 || I == 384);
+}
+
+hipError_t launch_experts_fused(const void* x, const void* wgu, const void* wd, const float* theta, const float* w,
+                                const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token, int T,
+                                int H, int E, int k, int I, void* yw, hipStream_t s) {
+  const int S = T * k;
+  if (S == 0) return hipSuccess;
+  const bf16_t* xp = static_cast<const bf16_t*>(x);
+  const bf16_t* gp = static_cast<const bf16_t*>(wgu);
+  const bf16_t* dp = static_cast<const bf16_t*>(wd);
+  bf16_t* yp = static_cast<bf16_t*>(yw);
+  switch (I) {
+    case 128: launch_fused_nt<1>(xp, gp, dp, theta, w, offsets, perm_slot, perm_token, S, H, E, yp, s); break;
+    case 256: launch_fused_nt<2>(xp, gp, dp, theta, w, offsets, perm_slot, perm_token, S, H, E, yp, s); break;
+    case 384: launch_fused_nt<3>(xp, gp, dp, theta, w, offsets, perm_slot, perm_token, S, H, E, yp, s); break;
+    default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
+}  // namespace bibo

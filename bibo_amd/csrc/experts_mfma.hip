@@ -14,192 +14,10 @@
 //   kernel 4 (down): N is a 128*NTW wide block of hidden columns; the epilogue multiplies each row by its
 //     routing weight and scatters it to slot order (token-major), where `combine` sums the k rows of a
 //     token.  Reference: src/modeling/ffn/moe.py:92-93,101.
-#include <utility>
-
-#include "common.h"
+#include "stripe.h"
 
 namespace bibo {
 namespace {
-
-constexpr int kLoadsPerPair = 1;
-constexpr int kBK = 32;        // K elements per LDS stage
-
-struct TileMap {
-  int incl;    // lane = expert: inclusive tile count
-  int ntile;   // lane = expert: tiles of this expert
-  int total;
-};
-
-__device__ __forceinline__ TileMap make_tile_map(const int32_t* __restrict__ offsets, int E, int BM) {
-  const int lane = lane_id();
-  int lo = 0, hi = 0;
-  if (lane < E) { lo = offsets[lane]; hi = offsets[lane + 1]; }
-  TileMap tm;
-  tm.ntile = (hi - lo + BM - 1) / BM;
-  tm.incl = wave_inclusive_scan(tm.ntile);
-  tm.total = __shfl(tm.incl, kWave - 1, kWave);
-  return tm;
-}
-
-// tile < tm.total required
-__device__ __forceinline__ void find_tile(const TileMap& tm, const int32_t* __restrict__ offsets, int BM, int tile,
-                                          int& expert, int& row0, int& rows) {
-  const unsigned long long m = __ballot(tm.incl > tile);
-  expert = __ffsll((long long)m) - 1;
-  const int excl = __shfl(tm.incl - tm.ntile, expert, kWave);
-  const int lo = offsets[expert], hi = offsets[expert + 1];
-  row0 = lo + (tile - excl) * BM;
-  rows = min(BM, hi - row0);
-}
-
-// ---- stage layout and loads ----------------------------------------------------------------------
-// Stage layout: rows of 32 bf16 (64 bytes, four 16-byte granules), A rows first, then B rows, no
-// padding.  Granule (row, c) is stored at position c ^ ((row >> 2) & 3) of its row, so the 16 lanes
-// that read one granule column of 16 consecutive rows hit 64 distinct banks.  Tiles arrive by
-// global_load_lds_dwordx4: the hardware writes lane L of a wave to LDS base + 16*L, so thread t of
-// load instruction i fills granule i*256 + t = (row i*64 + t/4, position t%4) and therefore FETCHES
-// logical granule (t%4) ^ ((t/16) & 3) of that row.  Two stages in separate __shared__ arrays: the
-// loads of step s+1 are in flight while step s is multiplied; one barrier per step.
-typedef __attribute__((address_space(3))) void lds_void;
-typedef const __attribute__((address_space(1))) void gbl_void;
-
-__device__ __forceinline__ void dma16(const bf16_t* g, bf16_t* l) {
-  __builtin_amdgcn_global_load_lds((gbl_void*)g, (lds_void*)l, 16, 0, 0);
-}
-
-// WM waves along M (each MT 32-row tiles) x 4 waves along N (each NTW 32-column tiles).
-template <int MT, int NTW, int WM>
-struct Stripe {
-  static constexpr int kThreads = 256 * WM;
-  static constexpr int BM = 32 * MT * WM;
-  static constexpr int BN = 128 * NTW;
-  static constexpr int A_GRAN = BM * 4;                          // 16-byte granules of an A stage
-  static constexpr int A_PER = (A_GRAN + kThreads - 1) / kThreads;
-  static constexpr int B_PER = BN * 4 / kThreads;
-  static constexpr int kStageElems = (BM + BN) * kBK;
-  static_assert(BM % 16 == 0 && (BN * 4) % kThreads == 0 && (kThreads / 16) % 4 == 0, "tile / thread mismatch");
-};
-
-// Everything one thread needs to issue the load instructions of a stage.
-template <typename S>
-struct StripeLoader {
-  const bf16_t* a_src[S::A_PER];   // row base + 8 * (swizzled granule) of the A rows this thread fetches
-  const bf16_t* b_src;             // same for its first B row; later instructions step by `bstep` elements
-  size_t bstep;
-
-  static constexpr int kInstr = S::A_PER + S::B_PER;
-
-  // load instruction `q` (0 .. kInstr-1) of the stage that starts at K offset k0
-  template <int Q>
-  __device__ __forceinline__ void issue(int k0, bf16_t* stage) const {
-    if constexpr (Q < kInstr) {
-      const int wave = threadIdx.x >> 6;
-      if constexpr (Q < S::A_PER) {
-        if (S::A_GRAN % S::kThreads == 0 || (Q * S::kThreads + wave * 64) < S::A_GRAN)      // wave-uniform
-          dma16(a_src[Q] + k0, stage + (Q * S::kThreads + wave * 64) * 8);
-      } else {
-        constexpr int i = Q - S::A_PER;
-        dma16(b_src + i * bstep + k0, stage + S::BM * kBK + (i * S::kThreads + wave * 64) * 8);
-      }
-    }
-  }
-  template <int... Qs>
-  __device__ __forceinline__ void issue_all(int k0, bf16_t* stage, std::integer_sequence<int, Qs...>) const {
-    (issue<Qs>(k0, stage), ...);
-  }
-  __device__ __forceinline__ void issue_stage(int k0, bf16_t* stage) const {
-    issue_all(k0, stage, std::make_integer_sequence<int, kInstr>{});
-  }
-};
-
-// One (k16 sub-step, N tile) pair of the software pipeline below; Q is a compile-time index so the
-// scheduling hints get constant arguments.  Pair Q also issues load instruction Q of the NEXT stage
-// (if there is one): spreading the loads through the MFMAs keeps the waves from queueing up at the
-// texture-address unit before they start multiplying.
-template <int Q, int MT, int NTW, typename S, typename FragRow>
-__device__ __forceinline__ void stripe_pair(floatx16 (&acc)[MT][NTW], bf16x8 (&a)[2][MT], bf16x8 (&b)[3],
-                                            const bf16_t* astage, const bf16_t* bstage, int pos0, FragRow frag_row,
-                                            const StripeLoader<S>& ld, bool prefetch, int k_next, bf16_t* next_stage) {
-  constexpr int kPairs = 2 * NTW;
-  constexpr int s = Q / NTW, j = Q % NTW;
-  // kLoadsPerPair load instructions of the next stage per pair, starting with pair 0
-  constexpr int kPer = kLoadsPerPair;
-  if (prefetch) {
-    if constexpr (Q * kPer < StripeLoader<S>::kInstr) ld.template issue<Q * kPer>(k_next, next_stage);
-    if constexpr (kPer > 1 && Q * kPer + 1 < StripeLoader<S>::kInstr) ld.template issue<Q * kPer + 1>(k_next, next_stage);
-  }
-  if constexpr (Q + 2 < kPairs) {
-    constexpr int s2 = (Q + 2) / NTW, j2 = (Q + 2) % NTW;
-    b[(Q + 2) % 3] = *reinterpret_cast<const bf16x8*>(bstage + frag_row(j2) * kBK + (pos0 ^ (s2 * 16)));
-  }
-  if constexpr (Q < MT) a[1][Q] = *reinterpret_cast<const bf16x8*>(astage + Q * 32 * kBK + (pos0 ^ 16));
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
-    acc[mt][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[s][mt], b[Q % 3], acc[mt][j], 0, 0, 0);
-  constexpr int kReads = (Q + 2 < kPairs ? 1 : 0) + (Q < MT ? 1 : 0);
-  if constexpr (kReads > 0) __builtin_amdgcn_sched_group_barrier(0x100, kReads, 0);
-  __builtin_amdgcn_sched_group_barrier(0x008, MT, 0);
-}
-
-template <int MT, int NTW, typename S, typename FragRow, int... Qs>
-__device__ __forceinline__ void stripe_pairs(floatx16 (&acc)[MT][NTW], bf16x8 (&a)[2][MT], bf16x8 (&b)[3],
-                                             const bf16_t* astage, const bf16_t* bstage, int pos0, FragRow frag_row,
-                                             const StripeLoader<S>& ld, bool prefetch, int k_next, bf16_t* next_stage,
-                                             std::integer_sequence<int, Qs...>) {
-  (stripe_pair<Qs, MT, NTW, S>(acc, a, b, astage, bstage, pos0, frag_row, ld, prefetch, k_next, next_stage), ...);
-}
-
-// Multiply one LDS stage into the accumulators while the load instructions of the next stage are
-// issued.  Software pipeline over the 2*NTW (k16 sub-step, N tile) pairs: B fragments rotate through
-// three buffers and are read two pairs ahead of the MFMAs that consume them; the A fragments of the
-// second sub-step are read while the first sub-step is still multiplying.
-template <int MT, int NTW, int WM, typename FragRow>
-__device__ __forceinline__ void stripe_compute(floatx16 (&acc)[MT][NTW], const bf16_t* stage, int wm, FragRow frag_row,
-                                               const StripeLoader<Stripe<MT, NTW, WM>>& ld, bool prefetch, int k_next,
-                                               bf16_t* next_stage) {
-  using S = Stripe<MT, NTW, WM>;
-  static_assert(StripeLoader<S>::kInstr <= 2 * (2 * NTW), "at most two load instructions per pair");
-  const int lane = threadIdx.x & 63;
-  const int n = lane & 31, h = lane >> 5;
-  const int pos0 = (h ^ ((n >> 2) & 3)) * 8;      // element offset of logical granule h; granule 2+h is pos0 ^ 16
-  const bf16_t* astage = stage + (wm * MT * 32 + n) * kBK;
-  const bf16_t* bstage = stage + (S::BM + n) * kBK;
-  bf16x8 a[2][MT], b[3];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) a[0][mt] = *reinterpret_cast<const bf16x8*>(astage + mt * 32 * kBK + pos0);
-  b[0] = *reinterpret_cast<const bf16x8*>(bstage + frag_row(0) * kBK + pos0);
-  b[1] = *reinterpret_cast<const bf16x8*>(bstage + frag_row(NTW > 1 ? 1 : 0) * kBK + (NTW > 1 ? pos0 : (pos0 ^ 16)));
-  __builtin_amdgcn_sched_group_barrier(0x100, MT + 2, 0);
-  stripe_pairs<MT, NTW, S>(acc, a, b, astage, bstage, pos0, frag_row, ld, prefetch, k_next, next_stage,
-                           std::make_integer_sequence<int, 2 * NTW>{});
-}
-
-__device__ __forceinline__ void wait_loads_and_sync() {
-  __builtin_amdgcn_s_waitcnt(0);   // vmcnt(0): this thread's LDS-DMA transfers have landed
-  __syncthreads();
-}
-
-template <int MT, int NTW, int WM, typename FragRow>
-__device__ __forceinline__ void stripe_mainloop_dma(floatx16 (&acc)[MT][NTW],
-                                                    const StripeLoader<Stripe<MT, NTW, WM>>& ld, int K, bf16_t* st0,
-                                                    bf16_t* st1, int wm, FragRow frag_row) {
-  ld.issue_stage(0, st0);
-  for (int k0 = 0; k0 < K; k0 += 2 * kBK) {
-    wait_loads_and_sync();
-    stripe_compute<MT, NTW, WM>(acc, st0, wm, frag_row, ld, k0 + kBK < K, k0 + kBK, st1);
-    if (k0 + kBK < K) {
-      wait_loads_and_sync();
-      stripe_compute<MT, NTW, WM>(acc, st1, wm, frag_row, ld, k0 + 2 * kBK < K, k0 + 2 * kBK, st0);
-    }
-  }
-}
-
-// logical granule fetched by thread t (see the layout note above)
-__device__ __forceinline__ int dma_chunk(int t) { return (t & 3) ^ ((t >> 4) & 3); }
-
-// Accumulator layout of one 32x32 tile: lane holds column lane%32; register i is row
-// 8*(i/4) + 4*(lane/32) + i%4.
-__device__ __forceinline__ int acc_row(int i, int lane) { return 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3); }
 
 // ---- kernel 3 ------------------------------------------------------------------------------------
 template <int MT, int NT, int WM>

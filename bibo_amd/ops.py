@@ -8,7 +8,8 @@ import torch
 from . import _lib as L
 
 _NORM = {"sum": L.NORM_SUM, True: L.NORM_SUM, "softmax": L.NORM_SOFTMAX, False: L.NORM_NONE, None: L.NORM_NONE}
-_ALGO = {"auto": L.ALGO_AUTO, "generic": L.ALGO_GENERIC, "mfma": L.ALGO_MFMA, "stream": L.ALGO_STREAM}
+_ALGO = {"auto": L.ALGO_AUTO, "generic": L.ALGO_GENERIC, "mfma": L.ALGO_MFMA, "stream": L.ALGO_STREAM,
+         "fused": L.ALGO_FUSED}
 
 
 def norm_mode(v) -> int:
@@ -137,6 +138,40 @@ def down_combine_fwd(hidden, w_down, w, offsets, perm_slot, T, algo="auto"):
         L.check(L.lib().bibo_moe_down_combine_fwd(_ptr(hidden), _ptr(w_down), _ptr(w), _ptr(offsets), _ptr(perm_slot),
                                                   T, H, E, k, I, dc, algo_code(algo), _ptr(out), _ptr(ws), ws.numel(),
                                                   _stream(dev)), "bibo_moe_down_combine_fwd")
+    return out
+
+
+def gateup_down_fwd(x, w_gate_up, w_down, theta, w, offsets, perm_slot, perm_token):
+    """Both projections in one launch -> yw [T*k, H] bf16, routing-weighted rows in slot order."""
+    T, H = x.shape
+    E, two_i, _ = w_gate_up.shape
+    I = two_i // 2
+    k = w.shape[1]
+    dc = _dtype_code(x)
+    _chk(x, "x"); _chk(w_gate_up, "w_gate_up", x.dtype, (E, 2 * I, H)); _chk(w_down, "w_down", x.dtype, (E, H, I))
+    _chk(theta, "theta", torch.float32, (E,)); _chk(w, "w", torch.float32, (T, k))
+    _chk(offsets, "offsets", torch.int32, (E + 1,)); _chk(perm_slot, "perm_slot", torch.int32, (T * k,))
+    _chk(perm_token, "perm_token", torch.int32, (T * k,))
+    yw = torch.zeros(T * k, H, dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        L.check(L.lib().bibo_moe_gateup_down_fwd(_ptr(x), _ptr(w_gate_up), _ptr(w_down), _ptr(theta), _ptr(w),
+                                                 _ptr(offsets), _ptr(perm_slot), _ptr(perm_token), T, H, E, k, I, dc,
+                                                 _ptr(yw), _stream(x.device)), "bibo_moe_gateup_down_fwd")
+    return yw
+
+
+def combine_fwd(yw, T, k, dtype=None):
+    """out[t] = sum_j yw[t*k + j] in fp32, rounded once -> [T,H] in `dtype` (default: yw.dtype)."""
+    H = yw.shape[1]
+    dtype = dtype or yw.dtype
+    _chk(yw, "yw", None, (T * k, H))
+    if yw.dtype not in (torch.bfloat16, torch.float32):
+        raise TypeError("yw must be bf16 or fp32")
+    out = torch.empty(T, H, dtype=dtype, device=yw.device)
+    dc = L.DTYPE_BF16 if dtype == torch.bfloat16 else L.DTYPE_F32
+    with torch.cuda.device(yw.device):
+        L.check(L.lib().bibo_moe_combine_fwd(_ptr(yw), int(yw.dtype == torch.bfloat16), T, H, k, dc, _ptr(out),
+                                             _stream(yw.device)), "bibo_moe_combine_fwd")
     return out
 
 

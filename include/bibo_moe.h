@@ -50,8 +50,12 @@ enum bibo_norm_mode { BIBO_NORM_NONE = 0, BIBO_NORM_SUM = 1, BIBO_NORM_SOFTMAX =
 enum bibo_algo {
   BIBO_ALGO_AUTO = 0,    /* pick by shape */
   BIBO_ALGO_GENERIC = 1, /* one workgroup per routed row, any H and I, bf16 or fp32 */
-  BIBO_ALGO_MFMA = 2,    /* grouped bf16 MFMA tiles; needs H % 32 == 0 and I in {128,256,384,512} */
-  BIBO_ALGO_STREAM = 3   /* weight-streaming kernels for few rows per expert (decode) */
+  BIBO_ALGO_MFMA = 2,    /* grouped bf16 MFMA tiles, one kernel per GEMM; needs bf16, H % 128 == 0 and
+                            I in {128,256,384,512} */
+  BIBO_ALGO_STREAM = 3,  /* weight-streaming kernels for few rows per expert (decode); bf16, H and I
+                            multiples of 64; only bibo_moe_experts_fwd / bibo_moe_forward, T*k <= 32*E */
+  BIBO_ALGO_FUSED = 4    /* both GEMMs of a 128-row tile in one kernel, activations stay in LDS; bf16,
+                            H % 128 == 0, I in {128,256,384}; only bibo_moe_experts_fwd / bibo_moe_forward */
 };
 
 enum bibo_error {
@@ -125,6 +129,24 @@ int bibo_moe_gateup_fwd(const void* x, const void* w_gate_up, const float* theta
 int bibo_moe_down_combine_fwd(const void* hidden, const void* w_down, const float* w, const int32_t* offsets,
                               const int32_t* perm_slot, int T, int H, int E, int k, int I, int dtype, int algo,
                               void* out, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Both grouped projections of a 128-row tile in one launch (BIBO_ALGO_FUSED shapes only: bf16,
+ * H % 128 == 0, I in {128,256,384}); the activations of moe.py:84-92 never reach memory.  Writes the
+ * routing-weighted expert outputs of moe.py:92-93 in slot order: yw bf16 [T*k, H], row t*k + j belongs to
+ * token t and its j-th selected expert.  Slots whose index was outside [0,E) are not written.
+ */
+int bibo_moe_gateup_down_fwd(const void* x, const void* w_gate_up, const void* w_down, const float* theta,
+                             const float* w, const int32_t* offsets, const int32_t* perm_slot,
+                             const int32_t* perm_token, int T, int H, int E, int k, int I, int dtype, void* yw,
+                             void* stream);
+
+/*
+ * out[t, :] = sum_j yw[t*k + j, :], summed in fp32 in ascending j and rounded once to `dtype`
+ * (the index_add_ of moe.py:93 and the cast of moe.py:101).  yw [T*k, H]: bf16 when yw_is_bf16 (then
+ * `dtype` must be bf16), fp32 otherwise; out [T,H] in `dtype`.
+ */
+int bibo_moe_combine_fwd(const void* yw, int yw_is_bf16, int T, int H, int k, int dtype, void* out, void* stream);
 
 /*
  * Seam 2: BiBoFusedExperts.forward(x, idx, w) (moe.py:46-101; the signature of the external

@@ -152,6 +152,48 @@ def test_mfma_and_generic_families_agree():
     assert rel_err(h_m, h_g) <= 1e-2 and rel_err(o_m, o_g) <= 1e-2
 
 
+@pytest.mark.parametrize("T,H,I,k,bias", [(1024, 768, 384, 6, "uniform"), (1024, 768, 384, 6, "hot4"),
+                                          (333, 256, 128, 6, "uniform"), (130, 128, 256, 6, "zero"),
+                                          (777, 512, 256, 6, "uniform"), (515, 640, 384, 8, "uniform"),
+                                          (1, 768, 384, 6, "zero")])
+def test_fused_kernel_matches_oracle_and_the_two_kernel_family(T, H, I, k, bias):
+    """One launch for both GEMMs (activations never leave the CU): same operand rounding as the two MFMA
+    kernels, another accumulation order in the down projection."""
+    p = O.make_inputs(T=T, H=H, E=64, k=k, I=I, bias=bias, theta="normal", seed=T + H + I)
+    idx, w = _route(p)
+    ref = O.experts_forward(p["x"], idx, w, p["w_gate_up"], p["w_down"], p["theta"])
+    out, counts = _gpu_experts(p, idx, w, "fused")
+    assert rel_err(out, ref) <= BF16_TOL
+    assert np.array_equal(counts, O.permute(idx, 64)[0])
+    two, _ = _gpu_experts(p, idx, w, "mfma")
+    assert rel_err(out, two) <= 1e-2
+
+
+def test_fused_stage_entry_points_compose_to_the_composite_call():
+    """permute -> gateup_down -> combine through the stage ABI equals bibo_moe_experts_fwd(fused) bit for bit;
+    the slot buffer holds w[t,j] * expert_j(x_t) (checked against the oracle per slot)."""
+    p = O.make_inputs(T=300, H=768, E=64, k=6, I=384, bias="uniform", theta="normal", seed=77)
+    idx, w = _route(p)
+    idx_d, w_d = torch.from_numpy(idx).to(DEV), torch.from_numpy(w).to(DEV)
+    counts, offsets, perm_slot, perm_token = ops.permute(idx_d, 64)
+    yw = ops.gateup_down_fwd(p["x"].to(DEV), p["w_gate_up"].to(DEV), p["w_down"].to(DEV), p["theta"].to(DEV), w_d,
+                             offsets, perm_slot, perm_token)
+    out = ops.combine_fwd(yw, 300, 6)
+    torch.cuda.synchronize()
+    ref_out, _ = _gpu_experts(p, idx, w, "fused")
+    assert torch.equal(out.cpu(), ref_out)
+    # one-hot routing weights isolate single slots in the oracle
+    for t, j in [(0, 0), (123, 5), (299, 3)]:
+        w1 = np.zeros_like(w[t:t + 1]); w1[0, j] = w[t, j]
+        ref = O.experts_forward(p["x"][t:t + 1], idx[t:t + 1], w1, p["w_gate_up"], p["w_down"], p["theta"])
+        assert rel_err(yw[t * 6 + j].cpu()[None], ref) <= BF16_TOL
+    # fp32 slot rows through the same combine entry point
+    y32 = yw.float()
+    out32 = ops.combine_fwd(y32, 300, 6)
+    torch.cuda.synchronize()
+    assert torch.allclose(out32.cpu(), y32.view(300, 6, 768).cpu().sum(1), atol=1e-5, rtol=1e-5)
+
+
 def test_mfma_with_empty_experts_and_one_hot_expert():
     """Only experts {5, 9} get rows (everything else empty), one of them with a ragged last tile."""
     g = torch.Generator().manual_seed(11)
@@ -160,28 +202,29 @@ def test_mfma_with_empty_experts_and_one_hot_expert():
     idx = np.tile(np.array([[5, 9]], np.int32), (T, 1))
     w = torch.rand(T, 2, generator=g).numpy().astype(np.float32)
     ref = O.experts_forward(p["x"], idx, w, p["w_gate_up"], p["w_down"], p["theta"])
-    for algo in ("generic", "mfma"):
+    for algo in ("generic", "mfma", "fused"):
         out, counts = _gpu_experts(p, idx, w, algo)
         assert rel_err(out, ref) <= BF16_TOL
         assert counts[5] == T and counts[9] == T and counts.sum() == 2 * T
 
 
+@pytest.mark.parametrize("algo", ["mfma", "fused"])
 @pytest.mark.parametrize("name", ["c2", "c4"])
-def test_full_size_prefill_properties(name):
+def test_full_size_prefill_properties(name, algo):
     """Full T: (a) oracle parity on a 256-token sample (a token's output depends only on its own row and
     routing); (b) doubling the routing weights doubles the bf16 output exactly; (c) permuting the tokens
     permutes the output rows exactly."""
     p = O.make_inputs(**O.CONFIGS[name])
     T = p["x"].shape[0]
     idx, w = _route(p)
-    out, counts = _gpu_experts(p, idx, w, "mfma")
+    out, counts = _gpu_experts(p, idx, w, algo)
     assert counts.sum() == T * 6 and np.array_equal(counts, np.bincount(idx.reshape(-1), minlength=64))
     sample = np.random.default_rng(0).choice(T, 256, replace=False)
     ref = O.experts_forward(p["x"][sample], idx[sample], w[sample], p["w_gate_up"], p["w_down"], p["theta"])
     assert rel_err(out[sample], ref) <= BF16_TOL
-    out2, _ = _gpu_experts(p, idx, (2 * w).astype(np.float32), "mfma")
+    out2, _ = _gpu_experts(p, idx, (2 * w).astype(np.float32), algo)
     assert torch.equal(out2.float(), 2 * out.float())
     perm = torch.randperm(T, generator=torch.Generator().manual_seed(1))
     pp = dict(p, x=p["x"][perm].contiguous())
-    outp, _ = _gpu_experts(pp, idx[perm.numpy()], w[perm.numpy()], "mfma")
+    outp, _ = _gpu_experts(pp, idx[perm.numpy()], w[perm.numpy()], algo)
     assert torch.equal(outp, out[perm])
