@@ -79,7 +79,7 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int wn = wave & 3, wm = wave >> 2;
   const int n = lane & 31;
-  const int chunk = dma_chunk(tid);
+  const int chunk = S1::dma_chunk(tid);
   const int mbase = wm * MT * 32;
 
   // ---- phase 1: gate/up projection (moe.py:81-86) ----
@@ -88,11 +88,11 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
     StripeLoader<S1> ld;
 #pragma unroll
     for (int i = 0; i < S1::A_PER; ++i) {
-      const int m = min((tid >> 2) + i * (S1::kThreads / 4), rows - 1);   // rows past the end re-read the last valid row
+      const int m = min(S1::dma_row(tid) + i * S1::kRowsPerInstr, rows - 1);   // rows past the end re-read the last valid row
       ld.a_src[i] = x + (size_t)perm_token[row0 + m] * H + chunk * 8;
     }
-    ld.b_src = wgu + ((size_t)e * 2 * I + (tid >> 2)) * H + chunk * 8;
-    ld.bstep = (size_t)(S1::kThreads / 4) * H;
+    ld.b_src = wgu + ((size_t)e * 2 * I + S1::dma_row(tid)) * H + chunk * 8;
+    ld.bstep = (size_t)S1::kRowsPerInstr * H;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -100,7 +100,7 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[mt][j][i] = 0.f;
     auto frag_row = [&](int j) { return (j < NT ? 0 : I) + (wn * NT + (j < NT ? j : j - NT)) * 32; };
-    stripe_mainloop_dma<MT, NTW, F::WM>(acc, ld, H, P, Q, wm, frag_row);
+    stripe_mainloop_dma<MT, NTW, F::WM, S1::BK>(acc, ld, H, P, Q, wm, frag_row);
   }
   __syncthreads();                         // every wave is done with the gate/up stages
 
@@ -168,35 +168,36 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
     for (int ct = 0; ct < CT; ++ct)
 #pragma unroll
       for (int rt = 0; rt < 8; ++rt) acc2[ct][rt] = floatx4{0.f, 0.f, 0.f, 0.f};
-    // Activation fragments are read one row tile ahead of the MFMAs that consume them (the fragments of
-    // row tile 0 of the next K block are requested before this block's last MFMAs).
+    // Activation fragments are read a row tile ahead of the MFMAs that consume them (across K block
+    // boundaries too).
     auto frag = [&](int kb, int rt, int s) {
       const int gq = (((kb * 8 + 2 * g4) ^ r16) * 8) ^ (s * 8);
       return *reinterpret_cast<const bf16x8*>((rt < 4 ? P : Q) + ((rt & 3) * 16 + r16) * I + gq);
     };
-    bf16x8 xa[2][2];
-    xa[0][0] = frag(0, 0, 0);
-    xa[0][1] = frag(0, 0, 1);
+    constexpr int AD = 1;                    // row tiles whose fragments are requested ahead (2 and 3 measured the same)
+    bf16x8 xa[AD + 1][2];
+#pragma unroll
+    for (int g = 0; g < AD; ++g) {
+      xa[g][0] = frag(g / 8, g % 8, 0);
+      xa[g][1] = frag(g / 8, g % 8, 1);
+    }
 #pragma unroll
     for (int kb = 0; kb < KB; ++kb) {
       if (kb + D < KB) load_wblock<CT>(wb[(kb + D) % NB], wp, tile_stride, kb + D);
       __builtin_amdgcn_sched_barrier(0);     // keep the loads D blocks ahead of their use
 #pragma unroll
       for (int rt = 0; rt < 8; ++rt) {
-        const int cur = rt & 1, nxt = cur ^ 1;
-        if (rt + 1 < 8) {
-          xa[nxt][0] = frag(kb, rt + 1, 0);
-          xa[nxt][1] = frag(kb, rt + 1, 1);
-        } else if (kb + 1 < KB) {
-          xa[nxt][0] = frag(kb + 1, 0, 0);
-          xa[nxt][1] = frag(kb + 1, 0, 1);
+        const int g = kb * 8 + rt;             // running (K block, row tile) index; fragments rotate through AD + 1 buffers
+        if (g + AD < KB * 8) {
+          xa[(g + AD) % (AD + 1)][0] = frag((g + AD) / 8, (g + AD) % 8, 0);
+          xa[(g + AD) % (AD + 1)][1] = frag((g + AD) / 8, (g + AD) % 8, 1);
         }
 #pragma unroll
         for (int s = 0; s < 2; ++s)
 #pragma unroll
           for (int ct = 0; ct < CT; ++ct)
-            acc2[ct][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb[kb % NB].w[ct][s], xa[cur][s], acc2[ct][rt], 0, 0, 0);
-        if (rt + 1 < 8 || kb + 1 < KB) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            acc2[ct][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb[kb % NB].w[ct][s], xa[g % (AD + 1)][s], acc2[ct][rt], 0, 0, 0);
+        if (g + AD < KB * 8) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
         __builtin_amdgcn_sched_group_barrier(0x008, 2 * CT, 0);
       }
     }

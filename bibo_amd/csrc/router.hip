@@ -137,6 +137,15 @@ __global__ __launch_bounds__(256) void router_generic_kernel(const TIn* __restri
   }
 }
 
+// One exchange of a (value, expert) pair with the lane a DPP control selects inside the 16-lane row; the
+// larger value wins, equal values go to the lower expert.
+template <int kCtrl>
+__device__ __forceinline__ void dpp_max_step(float& bv, int& be) {
+  const float ov = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, bv), kCtrl, 0xf, 0xf, false));
+  const int oe = __builtin_amdgcn_update_dpp(0, be, kCtrl, 0xf, 0xf, false);
+  if (ov > bv || (ov == bv && oe < be)) { bv = ov; be = oe; }
+}
+
 // Cooperative selection: 16 lanes per token, lane `seg` owns experts 4*seg .. 4*seg+3.  k rounds of
 // "best remaining candidate": local scan in ascending expert order, then a 16-lane butterfly on
 // (value, expert) where the larger value wins and equal values go to the lower expert.  All 16 lanes
@@ -152,12 +161,12 @@ __device__ __forceinline__ unsigned long long select_mask16(const float (&v)[4],
     for (int q = 0; q < 4; ++q)
       if (!((taken >> q) & 1) && (v[q] > bv || be == kMaxE)) { bv = v[q]; be = seg * 4 + q; }
     if (taken == 0xf) { bv = -INFINITY; be = kMaxE; }
-#pragma unroll
-    for (int o = 1; o < 16; o <<= 1) {
-      const float ov = __shfl_xor(bv, o, kWave);
-      const int oe = __shfl_xor(be, o, kWave);
-      if (ov > bv || (ov == bv && oe < be)) { bv = ov; be = oe; }
-    }
+    // 16-lane butterfly on DPP row operations (a DPP row is exactly one token's 16 lanes): swap within
+    // pairs, swap pairs within quads, mirror within 8 lanes, mirror within 16 lanes.
+    dpp_max_step<0xB1>(bv, be);
+    dpp_max_step<0x4E>(bv, be);
+    dpp_max_step<0x141>(bv, be);
+    dpp_max_step<0x140>(bv, be);
     be &= kMaxE - 1;
     if ((be >> 2) == seg) taken |= 1u << (be & 3);
     mask |= 1ull << be;

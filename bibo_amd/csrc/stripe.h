@@ -10,7 +10,7 @@ namespace bibo {
 namespace {
 
 constexpr int kLoadsPerPair = 1;
-constexpr int kBK = 32;        // K elements per LDS stage
+constexpr int kBK = 32;        // default K elements per LDS stage
 
 struct TileMap {
   int incl;    // lane = expert: inclusive tile count
@@ -41,13 +41,14 @@ __device__ __forceinline__ void find_tile(const TileMap& tm, const int32_t* __re
 }
 
 // ---- stage layout and loads ----------------------------------------------------------------------
-// Stage layout: rows of 32 bf16 (64 bytes, four 16-byte granules), A rows first, then B rows, no
-// padding.  Granule (row, c) is stored at position c ^ ((row >> 2) & 3) of its row, so the 16 lanes
-// that read one granule column of 16 consecutive rows hit 64 distinct banks.  Tiles arrive by
+// Stage layout: rows of BK bf16 (64 bytes = four 16-byte granules for BK = 32, 128 bytes = eight for
+// BK = 64), A rows first, then B rows, no padding.  Granule (row, c) is stored at position
+// c ^ ((row >> 2) & 3) of its row (BK = 32) or c ^ ((row >> 1) & 7) (BK = 64), so the 16 lanes that read
+// one granule column of 16 consecutive rows hit 64 distinct banks.  Tiles arrive by
 // global_load_lds_dwordx4: the hardware writes lane L of a wave to LDS base + 16*L, so thread t of
-// load instruction i fills granule i*256 + t = (row i*64 + t/4, position t%4) and therefore FETCHES
-// logical granule (t%4) ^ ((t/16) & 3) of that row.  Two stages in separate __shared__ arrays: the
-// loads of step s+1 are in flight while step s is multiplied; one barrier per step.
+// load instruction i fills granule i*kThreads + t = (row i*kThreads/GPR + t/GPR, position t%GPR) and
+// therefore FETCHES logical granule (t%GPR) ^ ((t/16) & (GPR-1)) of that row.  Two stages in separate
+// __shared__ arrays: the loads of step s+1 are in flight while step s is multiplied; one barrier per step.
 typedef __attribute__((address_space(3))) void lds_void;
 typedef const __attribute__((address_space(1))) void gbl_void;
 
@@ -56,16 +57,26 @@ __device__ __forceinline__ void dma16(const bf16_t* g, bf16_t* l) {
 }
 
 // WM waves along M (each MT 32-row tiles) x 4 waves along N (each NTW 32-column tiles).
-template <int MT, int NTW, int WM>
+template <int MT, int NTW, int WM, int BK_ = kBK>
 struct Stripe {
+  static constexpr int BK = BK_;                                 // K elements per stage: 32 (64-byte rows) or 64
+  static constexpr int GPR = BK / 8;                             // 16-byte granules per row
+  static constexpr int SS = BK / 16;                             // k16 sub-steps per stage
+  static constexpr int kSwzShift = GPR == 4 ? 2 : 1;             // row -> swizzle term (row >> shift) & (GPR - 1)
   static constexpr int kThreads = 256 * WM;
   static constexpr int BM = 32 * MT * WM;
   static constexpr int BN = 128 * NTW;
-  static constexpr int A_GRAN = BM * 4;                          // 16-byte granules of an A stage
+  static constexpr int A_GRAN = BM * GPR;                        // 16-byte granules of an A stage
   static constexpr int A_PER = (A_GRAN + kThreads - 1) / kThreads;
-  static constexpr int B_PER = BN * 4 / kThreads;
-  static constexpr int kStageElems = (BM + BN) * kBK;
-  static_assert(BM % 16 == 0 && (BN * 4) % kThreads == 0 && (kThreads / 16) % 4 == 0, "tile / thread mismatch");
+  static constexpr int B_PER = BN * GPR / kThreads;
+  static constexpr int kRowsPerInstr = kThreads / GPR;
+  static constexpr int kStageElems = (BM + BN) * BK;
+  static_assert(BK == 32 || BK == 64, "stage rows are 64 or 128 bytes");
+  static_assert(BM % 16 == 0 && (BN * GPR) % kThreads == 0 && kRowsPerInstr % 16 == 0, "tile / thread mismatch");
+  // logical granule fetched by thread t of any load instruction (see the layout note above)
+  __device__ static int dma_chunk(int t) { return (t & (GPR - 1)) ^ ((t >> 4) & (GPR - 1)); }
+  // row (within one instruction's rows) thread t fetches
+  __device__ static int dma_row(int t) { return t / GPR; }
 };
 
 // Everything one thread needs to issue the load instructions of a stage.
@@ -87,7 +98,7 @@ struct StripeLoader {
           dma16(a_src[Q] + k0, stage + (Q * S::kThreads + wave * 64) * 8);
       } else {
         constexpr int i = Q - S::A_PER;
-        dma16(b_src + i * bstep + k0, stage + S::BM * kBK + (i * S::kThreads + wave * 64) * 8);
+        dma16(b_src + i * bstep + k0, stage + S::BM * S::BK + (i * S::kThreads + wave * 64) * 8);
       }
     }
   }
@@ -105,73 +116,83 @@ struct StripeLoader {
 // (if there is one): spreading the loads through the MFMAs keeps the waves from queueing up at the
 // texture-address unit before they start multiplying.  `a1` points at this lane's A fragment of the
 // second sub-step for M tile 0; tile mt is `astride` elements further.
-template <int Q, int MT, int NTW, typename Loader, typename FragRow>
+template <int Q, int MT, int NTW, int BK, typename Loader, typename FragRow>
 __device__ __forceinline__ void stripe_pair(floatx16 (&acc)[MT][NTW], bf16x8 (&a)[2][MT], bf16x8 (&b)[3],
-                                            const bf16_t* a1, int astride, const bf16_t* bstage, int pos0,
+                                            const bf16_t* a0, int astride, const bf16_t* bstage, int pos0,
                                             FragRow frag_row, const Loader& ld, bool prefetch, int k_next,
                                             bf16_t* next_stage) {
-  constexpr int kPairs = 2 * NTW;
+  constexpr int SS = BK / 16;
+  constexpr int kPairs = SS * NTW;
   constexpr int s = Q / NTW, j = Q % NTW;
   // kLoadsPerPair load instructions of the next stage per pair, starting with pair 0
-  constexpr int kPer = kLoadsPerPair;
+  constexpr int kPer = (Loader::kInstr + kPairs - 1) / kPairs > kLoadsPerPair ? (Loader::kInstr + kPairs - 1) / kPairs
+                                                                              : kLoadsPerPair;
   if (prefetch) {
     if constexpr (Q * kPer < Loader::kInstr) ld.template issue<Q * kPer>(k_next, next_stage);
     if constexpr (kPer > 1 && Q * kPer + 1 < Loader::kInstr) ld.template issue<Q * kPer + 1>(k_next, next_stage);
   }
   if constexpr (Q + 2 < kPairs) {
     constexpr int s2 = (Q + 2) / NTW, j2 = (Q + 2) % NTW;
-    b[(Q + 2) % 3] = *reinterpret_cast<const bf16x8*>(bstage + frag_row(j2) * kBK + (pos0 ^ (s2 * 16)));
+    b[(Q + 2) % 3] = *reinterpret_cast<const bf16x8*>(bstage + frag_row(j2) * BK + (pos0 ^ (s2 * 16)));
   }
-  if constexpr (Q < MT) a[1][Q] = *reinterpret_cast<const bf16x8*>(a1 + Q * astride);
+  // A fragments of the next sub-step are read during the pairs of this one: pair j reads M tile j, the
+  // last pair whatever is left
+  constexpr int kAFirst = j, kALast = (s + 1 < SS) ? ((j == NTW - 1) ? MT - 1 : (j < MT ? j : -1)) : -1;
+#pragma unroll
+  for (int mt = kAFirst; mt <= kALast; ++mt)
+    a[(s + 1) & 1][mt] = *reinterpret_cast<const bf16x8*>(a0 + mt * astride + ((pos0 ^ ((s + 1) * 16)) - pos0));
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
-    acc[mt][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[s][mt], b[Q % 3], acc[mt][j], 0, 0, 0);
-  constexpr int kReads = (Q + 2 < kPairs ? 1 : 0) + (Q < MT ? 1 : 0);
+    acc[mt][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[s & 1][mt], b[Q % 3], acc[mt][j], 0, 0, 0);
+  constexpr int kReads = (Q + 2 < kPairs ? 1 : 0) + (kALast >= kAFirst ? kALast - kAFirst + 1 : 0);
   if constexpr (kReads > 0) __builtin_amdgcn_sched_group_barrier(0x100, kReads, 0);
   __builtin_amdgcn_sched_group_barrier(0x008, MT, 0);
 }
 
-template <int MT, int NTW, typename Loader, typename FragRow, int... Qs>
+template <int MT, int NTW, int BK, typename Loader, typename FragRow, int... Qs>
 __device__ __forceinline__ void stripe_pairs(floatx16 (&acc)[MT][NTW], bf16x8 (&a)[2][MT], bf16x8 (&b)[3],
-                                             const bf16_t* a1, int astride, const bf16_t* bstage, int pos0,
+                                             const bf16_t* a0, int astride, const bf16_t* bstage, int pos0,
                                              FragRow frag_row, const Loader& ld, bool prefetch, int k_next,
                                              bf16_t* next_stage, std::integer_sequence<int, Qs...>) {
-  (stripe_pair<Qs, MT, NTW>(acc, a, b, a1, astride, bstage, pos0, frag_row, ld, prefetch, k_next, next_stage), ...);
+  (stripe_pair<Qs, MT, NTW, BK>(acc, a, b, a0, astride, bstage, pos0, frag_row, ld, prefetch, k_next, next_stage), ...);
 }
 
-// Multiply one K step of 32 into the accumulators while the load instructions of the next stage are
-// issued.  Software pipeline over the 2*NTW (k16 sub-step, N tile) pairs: B fragments rotate through
-// three buffers and are read two pairs ahead of the MFMAs that consume them; the A fragments of the
-// second sub-step are read while the first sub-step is still multiplying.  a0 / a1: this lane's A
-// fragment of sub-step 0 / 1 for M tile 0; bstage: this lane's row of the B stage (N tile 0).
-template <int MT, int NTW, typename Loader, typename FragRow>
-__device__ __forceinline__ void stripe_step(floatx16 (&acc)[MT][NTW], const bf16_t* a0, const bf16_t* a1, int astride,
-                                            const bf16_t* bstage, int pos0, FragRow frag_row, const Loader& ld,
-                                            bool prefetch, int k_next, bf16_t* next_stage) {
-  static_assert(Loader::kInstr <= 2 * (2 * NTW), "at most two load instructions per pair");
+// Multiply one K step of BK into the accumulators while the load instructions of the next stage are
+// issued.  Software pipeline over the (BK/16)*NTW (k16 sub-step, N tile) pairs: B fragments rotate
+// through three buffers and are read two pairs ahead of the MFMAs that consume them; the A fragments
+// of the next sub-step are read while the current one is still multiplying.  a0: this lane's A
+// fragment of sub-step 0 for M tile 0 (position pos0 of its row; sub-step s sits at pos0 ^ 16s, M tile
+// mt `astride` elements further); bstage: this lane's row of the B stage (N tile 0).
+template <int MT, int NTW, int BK, typename Loader, typename FragRow>
+__device__ __forceinline__ void stripe_step(floatx16 (&acc)[MT][NTW], const bf16_t* a0, int astride, const bf16_t* bstage,
+                                            int pos0, FragRow frag_row, const Loader& ld, bool prefetch, int k_next,
+                                            bf16_t* next_stage) {
+  constexpr int SS = BK / 16;
+  static_assert(Loader::kInstr <= 2 * (SS * NTW), "at most two load instructions per pair");
   bf16x8 a[2][MT], b[3];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) a[0][mt] = *reinterpret_cast<const bf16x8*>(a0 + mt * astride);
-  b[0] = *reinterpret_cast<const bf16x8*>(bstage + frag_row(0) * kBK + pos0);
-  b[1] = *reinterpret_cast<const bf16x8*>(bstage + frag_row(NTW > 1 ? 1 : 0) * kBK + (NTW > 1 ? pos0 : (pos0 ^ 16)));
+  b[0] = *reinterpret_cast<const bf16x8*>(bstage + frag_row(0) * BK + pos0);
+  b[1] = *reinterpret_cast<const bf16x8*>(bstage + frag_row(NTW > 1 ? 1 : 0) * BK + (NTW > 1 ? pos0 : (pos0 ^ 16)));
   __builtin_amdgcn_sched_group_barrier(0x100, MT + 2, 0);
-  stripe_pairs<MT, NTW>(acc, a, b, a1, astride, bstage, pos0, frag_row, ld, prefetch, k_next, next_stage,
-                        std::make_integer_sequence<int, 2 * NTW>{});
+  stripe_pairs<MT, NTW, BK>(acc, a, b, a0, astride, bstage, pos0, frag_row, ld, prefetch, k_next, next_stage,
+                            std::make_integer_sequence<int, SS * NTW>{});
 }
 
 // A and B both come from `stage` (A rows first).
-template <int MT, int NTW, int WM, typename FragRow>
+template <int MT, int NTW, int WM, int BK, typename FragRow>
 __device__ __forceinline__ void stripe_compute(floatx16 (&acc)[MT][NTW], const bf16_t* stage, int wm, FragRow frag_row,
-                                               const StripeLoader<Stripe<MT, NTW, WM>>& ld, bool prefetch, int k_next,
-                                               bf16_t* next_stage) {
-  using S = Stripe<MT, NTW, WM>;
+                                               const StripeLoader<Stripe<MT, NTW, WM, BK>>& ld, bool prefetch,
+                                               int k_next, bf16_t* next_stage) {
+  using S = Stripe<MT, NTW, WM, BK>;
   const int lane = threadIdx.x & 63;
   const int n = lane & 31, h = lane >> 5;
-  const int pos0 = (h ^ ((n >> 2) & 3)) * 8;      // element offset of logical granule h; granule 2+h is pos0 ^ 16
-  const bf16_t* astage = stage + (wm * MT * 32 + n) * kBK;
-  const bf16_t* bstage = stage + (S::BM + n) * kBK;
-  stripe_step<MT, NTW>(acc, astage + pos0, astage + (pos0 ^ 16), 32 * kBK, bstage, pos0, frag_row, ld, prefetch, k_next,
-                       next_stage);
+  // element offset of logical granule h of row n (all fragment rows are n plus a multiple of 32, which
+  // leaves the swizzle term unchanged); granule 2s + h is pos0 ^ 16s
+  const int pos0 = (h ^ ((n >> S::kSwzShift) & (S::GPR - 1))) * 8;
+  const bf16_t* astage = stage + (wm * MT * 32 + n) * BK;
+  const bf16_t* bstage = stage + (S::BM + n) * BK;
+  stripe_step<MT, NTW, BK>(acc, astage + pos0, 32 * BK, bstage, pos0, frag_row, ld, prefetch, k_next, next_stage);
 }
 
 __device__ __forceinline__ void wait_loads_and_sync() {
@@ -179,23 +200,20 @@ __device__ __forceinline__ void wait_loads_and_sync() {
   __syncthreads();
 }
 
-template <int MT, int NTW, int WM, typename FragRow>
+template <int MT, int NTW, int WM, int BK, typename FragRow>
 __device__ __forceinline__ void stripe_mainloop_dma(floatx16 (&acc)[MT][NTW],
-                                                    const StripeLoader<Stripe<MT, NTW, WM>>& ld, int K, bf16_t* st0,
+                                                    const StripeLoader<Stripe<MT, NTW, WM, BK>>& ld, int K, bf16_t* st0,
                                                     bf16_t* st1, int wm, FragRow frag_row) {
   ld.issue_stage(0, st0);
-  for (int k0 = 0; k0 < K; k0 += 2 * kBK) {
+  for (int k0 = 0; k0 < K; k0 += 2 * BK) {
     wait_loads_and_sync();
-    stripe_compute<MT, NTW, WM>(acc, st0, wm, frag_row, ld, k0 + kBK < K, k0 + kBK, st1);
-    if (k0 + kBK < K) {
+    stripe_compute<MT, NTW, WM, BK>(acc, st0, wm, frag_row, ld, k0 + BK < K, k0 + BK, st1);
+    if (k0 + BK < K) {
       wait_loads_and_sync();
-      stripe_compute<MT, NTW, WM>(acc, st1, wm, frag_row, ld, k0 + 2 * kBK < K, k0 + 2 * kBK, st0);
+      stripe_compute<MT, NTW, WM, BK>(acc, st1, wm, frag_row, ld, k0 + 2 * BK < K, k0 + 2 * BK, st0);
     }
   }
 }
-
-// logical granule fetched by thread t (see the layout note above)
-__device__ __forceinline__ int dma_chunk(int t) { return (t & 3) ^ ((t >> 4) & 3); }
 
 // Accumulator layout of one 32x32 tile: lane holds column lane%32; register i is row
 // 8*(i/4) + 4*(lane/32) + i%4.

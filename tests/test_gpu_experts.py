@@ -110,6 +110,7 @@ def test_bf16_experts_match_oracle_on_named_workloads(name, algo):
 @pytest.mark.parametrize("algo", ["generic", "mfma"])
 @pytest.mark.parametrize("T,H,I,bias,theta", [(1024, 768, 384, "uniform", "normal"), (1024, 768, 384, "hot4", "normal"),
                                               (7, 1024, 512, "zero", "normal"), (333, 256, 128, "uniform", "normal"),
+                                              (300, 384, 256, "uniform", "normal"),
                                               (130, 128, 256, "zero", "zero")])
 def test_bf16_experts_reduced_prefill_and_ragged_shapes(T, H, I, bias, theta, algo):
     p = O.make_inputs(T=T, H=H, E=64, k=6, I=I, bias=bias, theta=theta, seed=T + H)
