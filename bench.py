@@ -75,7 +75,7 @@ class Layer:
         P = lambda t: ctypes.c_void_p(t.data_ptr())
         self._fwd_args = (P(self.x), P(self.wr), P(self.bias), P(self.wgu), P(self.wd), P(self.theta),
                           ctypes.byref(self.shape), L.NORM_SUM, self.algo, P(self.out), P(self.idx), P(self.w),
-                          P(self.counts), None, P(self.ws), self.ws.numel(), self.stream)
+                          None, None, P(self.ws), self.ws.numel(), self.stream)   # eval forward: no counts, no logits
         self._stages = {
             "router": (self.lib.bibo_moe_router_fwd,
                        (P(self.x), P(self.wr), P(self.bias), T, H, E, k, L.DTYPE_BF16, L.NORM_SUM, None, P(self.idx),
@@ -161,7 +161,8 @@ class Layer:
         p = self.host
         ref = O.experts_forward(p["x"][sample], idx[sample], w[sample], p["w_gate_up"], p["w_down"], p["theta"])
         got = self.out.cpu()[sample].double()
-        return ((got - ref.double()).abs().max() / ref.double().abs().max()).item(), int((self.counts > 0).sum())
+        active = int(np.unique(idx).size)                      # experts that received at least one token
+        return ((got - ref.double()).abs().max() / ref.double().abs().max()).item(), active
 
 
 def cpu_baseline(name, budget_s=20.0, sample_tokens=8192):

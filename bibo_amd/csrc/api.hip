@@ -22,7 +22,8 @@ int check_dims(int T, int H, int E, int k, int I, int dtype) {
 constexpr long long kStreamRowsPerExpert = 32;
 
 inline bool stream_eligible(int T, int H, int E, int k, int I, int dtype) {
-  return stream_supported(H, I, dtype) && (long long)T * k <= kStreamRowsPerExpert * E;
+  return stream_supported(H, I, dtype) && (long long)T * k <= kStreamRowsPerExpert * E &&
+         (long long)T * k <= kStreamMaxSlots;
 }
 
 // `composite`: the caller is bibo_moe_experts_fwd / bibo_moe_forward, the only entry points that can run
@@ -90,8 +91,9 @@ int gateup_dispatch(const void* x, const void* wgu, const float* theta, const in
   return hip_rc(launch_gateup_generic(x, wgu, theta, offsets, perm_token, T, H, E, k, I, dtype, hidden, s));
 }
 
-int down_dispatch(const void* hidden, const void* wd, const float* w, const int32_t* offsets, const int32_t* perm_slot,
-                  int T, int H, int E, int k, int I, int dtype, int algo, void* out, float* yw, hipStream_t s) {
+int down_dispatch(const void* hidden, const void* wd, const int32_t* idx, const float* w, const int32_t* offsets,
+                  const int32_t* perm_slot, int T, int H, int E, int k, int I, int dtype, int algo, void* out, float* yw,
+                  hipStream_t s) {
   hipError_t e;
   if (algo == BIBO_ALGO_MFMA) {
     if (!aligned16(hidden) || !aligned16(wd)) return BIBO_ERR_MISALIGNED;
@@ -99,37 +101,38 @@ int down_dispatch(const void* hidden, const void* wd, const float* w, const int3
     // expert output to bf16 as well, moe.py:92)
     e = launch_down_mfma(hidden, wd, w, offsets, perm_slot, T, H, E, k, I, yw, s);
     if (e != hipSuccess) return (int)e;
-    return hip_rc(launch_combine(yw, 1, T, H, k, dtype, out, s));
+    return hip_rc(launch_combine(yw, 1, idx, E, T, H, k, dtype, out, s));
   }
   e = launch_down_generic(hidden, wd, w, offsets, perm_slot, T, H, E, k, I, dtype, yw, s);
   if (e != hipSuccess) return (int)e;
-  return hip_rc(launch_combine(yw, 0, T, H, k, dtype, out, s));
+  return hip_rc(launch_combine(yw, 0, idx, E, T, H, k, dtype, out, s));
 }
 
 // kernels 3 and 4 (+ combine) after the permutation, for the composite entry points
-int experts_dispatch(const void* x, const void* wgu, const void* wd, const float* theta, const float* w,
-                     const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token, int T, int H, int E,
+int experts_dispatch(const void* x, const void* wgu, const void* wd, const float* theta, const int32_t* idx,
+                     const float* w, const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token, int T,
+                     int H, int E,
                      int k, int I, int dtype, int algo, void* out, char* base, const Workspace& ws, hipStream_t s) {
   float* yw = reinterpret_cast<float*>(base + ws.yw);
   if (algo == BIBO_ALGO_STREAM) {
     if (!aligned16(x) || !aligned16(wgu) || !aligned16(wd)) return BIBO_ERR_MISALIGNED;
     if (!stream_eligible(T, H, E, k, I, dtype)) return BIBO_ERR_UNSUPPORTED;     // no pre-activation segment carved
     float* gu = reinterpret_cast<float*>(base + ws.gu);
-    hipError_t e = launch_gateup_stream(x, wgu, offsets, perm_token, T, H, E, k, I, gu, s);
+    hipError_t e = launch_gateup_stream(x, wgu, idx, T, H, E, k, I, gu, s);
     if (e != hipSuccess) return (int)e;
-    e = launch_down_stream(gu, wd, theta, w, offsets, perm_slot, T, H, E, k, I, base + ws.hidden, yw, s);
+    e = launch_down_stream(gu, wd, theta, w, idx, T, H, E, k, I, base + ws.hidden, yw, s);
     if (e != hipSuccess) return (int)e;
-    return hip_rc(launch_combine(yw, 0, T, H, k, dtype, out, s));
+    return hip_rc(launch_combine(yw, 0, idx, E, T, H, k, dtype, out, s));
   }
   if (algo == BIBO_ALGO_FUSED) {
     if (!aligned16(x) || !aligned16(wgu) || !aligned16(wd)) return BIBO_ERR_MISALIGNED;
     hipError_t e = launch_experts_fused(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, T, H, E, k, I, yw, s);
     if (e != hipSuccess) return (int)e;
-    return hip_rc(launch_combine(yw, 1, T, H, k, dtype, out, s));
+    return hip_rc(launch_combine(yw, 1, idx, E, T, H, k, dtype, out, s));
   }
   const int rc = gateup_dispatch(x, wgu, theta, offsets, perm_token, T, H, E, k, I, dtype, algo, base + ws.hidden, s);
   if (rc != BIBO_OK) return rc;
-  return down_dispatch(base + ws.hidden, wd, w, offsets, perm_slot, T, H, E, k, I, dtype, algo, out, yw, s);
+  return down_dispatch(base + ws.hidden, wd, idx, w, offsets, perm_slot, T, H, E, k, I, dtype, algo, out, yw, s);
 }
 
 }  // namespace
@@ -206,7 +209,7 @@ int bibo_moe_down_combine_fwd(const void* hidden, const void* w_down, const floa
   if (T == 0) return BIBO_OK;
   if (!hidden || !w_down || !w || !offsets || !perm_slot || !out || !workspace) return BIBO_ERR_NULL_POINTER;
   if (workspace_bytes < (size_t)T * k * H * sizeof(float)) return BIBO_ERR_WORKSPACE_TOO_SMALL;
-  return down_dispatch(hidden, w_down, w, offsets, perm_slot, T, H, E, k, I, dtype, a, out,
+  return down_dispatch(hidden, w_down, nullptr, w, offsets, perm_slot, T, H, E, k, I, dtype, a, out,
                        static_cast<float*>(workspace), static_cast<hipStream_t>(stream));
 }
 
@@ -231,7 +234,7 @@ int bibo_moe_combine_fwd(const void* yw, int yw_is_bf16, int T, int H, int k, in
   if (yw_is_bf16 && dtype != BIBO_DTYPE_BF16) return BIBO_ERR_BAD_DTYPE;
   if (T == 0) return BIBO_OK;
   if (!yw || !out) return BIBO_ERR_NULL_POINTER;
-  return hip_rc(launch_combine(yw, yw_is_bf16 ? 1 : 0, T, H, k, dtype, out, static_cast<hipStream_t>(stream)));
+  return hip_rc(launch_combine(yw, yw_is_bf16 ? 1 : 0, nullptr, 0, T, H, k, dtype, out, static_cast<hipStream_t>(stream)));
 }
 
 int bibo_moe_experts_fwd(const void* x, const int32_t* idx, const float* w, const void* w_gate_up, const void* w_down,
@@ -253,10 +256,13 @@ int bibo_moe_experts_fwd(const void* x, const int32_t* idx, const float* w, cons
   int32_t* offsets = reinterpret_cast<int32_t*>(base + ws.offsets);
   int32_t* perm_slot = reinterpret_cast<int32_t*>(base + ws.perm_slot);
   int32_t* perm_token = reinterpret_cast<int32_t*>(base + ws.perm_token);
-  if ((rc = hip_rc(launch_permute(idx, T, E, k, counts, offsets, perm_slot, perm_token, base + ws.hist, s))) != BIBO_OK)
+  // the streaming kernels find their rows themselves; the permutation then only serves the counts
+  const bool need_permute = a != BIBO_ALGO_STREAM || counts_out != nullptr || T == 0;
+  if (need_permute &&
+      (rc = hip_rc(launch_permute(idx, T, E, k, counts, offsets, perm_slot, perm_token, base + ws.hist, s))) != BIBO_OK)
     return rc;
   if (T == 0) return BIBO_OK;
-  return experts_dispatch(x, w_gate_up, w_down, theta, w, offsets, perm_slot, perm_token, T, H, E, k, I, dtype, a, out,
+  return experts_dispatch(x, w_gate_up, w_down, theta, idx, w, offsets, perm_slot, perm_token, T, H, E, k, I, dtype, a, out,
                           base, ws, s);
 }
 
@@ -287,10 +293,13 @@ int bibo_moe_forward(const void* x, const void* w_router, const float* bias, con
       (rc = hip_rc(launch_router(x, w_router, bias, T, H, E, k, dtype, norm_mode, logits_out, idx, w, nullptr, s))) !=
           BIBO_OK)
     return rc;
-  if ((rc = hip_rc(launch_permute(idx, T, E, k, counts, offsets, perm_slot, perm_token, base + ws.hist, s))) != BIBO_OK)
+  // the streaming kernels find their rows themselves; the permutation then only serves the counts
+  const bool need_permute = a != BIBO_ALGO_STREAM || counts_out != nullptr || T == 0;
+  if (need_permute &&
+      (rc = hip_rc(launch_permute(idx, T, E, k, counts, offsets, perm_slot, perm_token, base + ws.hist, s))) != BIBO_OK)
     return rc;
   if (T == 0) return BIBO_OK;
-  return experts_dispatch(x, w_gate_up, w_down, theta, w, offsets, perm_slot, perm_token, T, H, E, k, I, dtype, a, out,
+  return experts_dispatch(x, w_gate_up, w_down, theta, idx, w, offsets, perm_slot, perm_token, T, H, E, k, I, dtype, a, out,
                           base, ws, s);
 }
 

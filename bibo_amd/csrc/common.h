@@ -16,6 +16,7 @@ constexpr float kSumNormEps = 1e-20f;   // src/modeling/ffn/router.py:45
 
 // tokens handled by one workgroup of the histogram / permutation kernels
 constexpr int kPermTokens = 256;
+constexpr int kStreamMaxSlots = 2048;   // routed slots the weight-streaming kernels can scan per workgroup
 
 typedef __bf16 bf16_t;
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -118,7 +119,8 @@ hipError_t launch_gateup_generic(const void* x, const void* wgu, const float* th
 hipError_t launch_down_generic(const void* hidden, const void* wd, const float* w, const int32_t* offsets,
                                const int32_t* perm_slot, int T, int H, int E, int k, int I, int dtype, float* yw,
                                hipStream_t s);
-hipError_t launch_combine(const void* yw, int yw_is_bf16, int T, int H, int k, int dtype, void* out, hipStream_t s);
+hipError_t launch_combine(const void* yw, int yw_is_bf16, const int32_t* idx, int E, int T, int H, int k, int dtype,
+                          void* out, hipStream_t s);
 bool mfma_supported(int H, int I, int dtype);
 hipError_t launch_gateup_mfma(const void* x, const void* wgu, const float* theta, const int32_t* offsets,
                               const int32_t* perm_token, int T, int H, int E, int k, int I, void* hidden, hipStream_t s);
@@ -130,10 +132,9 @@ hipError_t launch_experts_fused(const void* x, const void* wgu, const void* wd, 
                                 const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token, int T,
                                 int H, int E, int k, int I, void* yw, hipStream_t s);
 bool stream_supported(int H, int I, int dtype);
-hipError_t launch_gateup_stream(const void* x, const void* wgu, const int32_t* offsets, const int32_t* perm_token,
-                                int T, int H, int E, int k, int I, float* gu, hipStream_t s);
-hipError_t launch_down_stream(const float* gu, const void* wd, const float* theta, const float* w,
-                              const int32_t* offsets, const int32_t* perm_slot, int T, int H, int E, int k, int I,
-                              void* hidden, float* yw, hipStream_t s);
+hipError_t launch_gateup_stream(const void* x, const void* wgu, const int32_t* idx, int T, int H, int E, int k, int I,
+                                float* gu, hipStream_t s);
+hipError_t launch_down_stream(const float* gu, const void* wd, const float* theta, const float* w, const int32_t* idx,
+                              int T, int H, int E, int k, int I, void* hidden, float* yw, hipStream_t s);
 
 }  // namespace bibo

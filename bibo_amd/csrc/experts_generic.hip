@@ -87,22 +87,27 @@ __global__ __launch_bounds__(256) void down_generic_kernel(const TIn* __restrict
   }
 }
 
-// out[t, :] = round(sum_j yw[t*k + j, :])  in fp32, ascending j   (moe.py:93,101)
+// out[t, :] = round(sum_j yw[t*k + j, :])  in fp32, ascending j   (moe.py:93,101).  With `idx` given, slots
+// whose expert index is outside [0,E) are skipped (no kernel wrote their row).
 template <typename TY, typename TOut>
-__global__ __launch_bounds__(256) void combine_kernel(const TY* __restrict__ yw, int T, int H, int k,
-                                                      TOut* __restrict__ out) {
+__global__ __launch_bounds__(256) void combine_kernel(const TY* __restrict__ yw, const int32_t* __restrict__ idx, int E,
+                                                      int T, int H, int k, TOut* __restrict__ out) {
   const size_t n = (size_t)T * H;
   for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
     const size_t t = i / H, h = i - t * H;
     float acc = 0.f;
-    for (int j = 0; j < k; ++j) acc += to_float(yw[(t * k + j) * H + h]);
+    for (int j = 0; j < k; ++j) {
+      if (idx != nullptr && (unsigned)idx[t * k + j] >= (unsigned)E) continue;
+      acc += to_float(yw[(t * k + j) * H + h]);
+    }
     out[i] = from_float<TOut>(acc);
   }
 }
 
 // bf16 slot rows -> bf16 output, 8 columns (16 bytes) per thread, fp32 sum in ascending j   (moe.py:93,101)
-__global__ __launch_bounds__(256) void combine_bf16x8_kernel(const bf16_t* __restrict__ yw, int T, int H8, int k,
-                                                             bf16_t* __restrict__ out) {
+__global__ __launch_bounds__(256) void combine_bf16x8_kernel(const bf16_t* __restrict__ yw,
+                                                             const int32_t* __restrict__ idx, int E, int T, int H8,
+                                                             int k, bf16_t* __restrict__ out) {
   const size_t n = (size_t)T * H8;
   for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
     const size_t t = i / H8, c = i - t * H8;
@@ -111,6 +116,7 @@ __global__ __launch_bounds__(256) void combine_bf16x8_kernel(const bf16_t* __res
     for (int q = 0; q < 8; ++q) acc[q] = 0.f;
     const bf16x8* src = reinterpret_cast<const bf16x8*>(yw) + (t * k) * H8 + c;
     for (int j = 0; j < k; ++j) {
+      if (idx != nullptr && (unsigned)idx[t * k + j] >= (unsigned)E) continue;
       const bf16x8 v = src[(size_t)j * H8];
 #pragma unroll
       for (int q = 0; q < 8; ++q) acc[q] += (float)v[q];
@@ -156,7 +162,8 @@ hipError_t launch_down_generic(const void* hidden, const void* wd, const float* 
   return hipGetLastError();
 }
 
-hipError_t launch_combine(const void* yw, int yw_is_bf16, int T, int H, int k, int dtype, void* out, hipStream_t s) {
+hipError_t launch_combine(const void* yw, int yw_is_bf16, const int32_t* idx, int E, int T, int H, int k, int dtype,
+                          void* out, hipStream_t s) {
   const size_t n = (size_t)T * H;
   if (n == 0) return hipSuccess;
   const int grid = (int)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
@@ -165,17 +172,17 @@ hipError_t launch_combine(const void* yw, int yw_is_bf16, int T, int H, int k, i
     if ((H % 8) == 0 && ((reinterpret_cast<uintptr_t>(yw) | reinterpret_cast<uintptr_t>(out)) & 15) == 0) {
       const size_t n8 = n / 8;
       const int g8 = (int)((n8 + 255) / 256 < 65536 ? (n8 + 255) / 256 : 65536);
-      hipLaunchKernelGGL(combine_bf16x8_kernel, dim3(g8), dim3(256), 0, s, static_cast<const bf16_t*>(yw), T, H / 8, k,
+      hipLaunchKernelGGL(combine_bf16x8_kernel, dim3(g8), dim3(256), 0, s, static_cast<const bf16_t*>(yw), idx, E, T, H / 8, k,
                          static_cast<bf16_t*>(out));
     } else
       hipLaunchKernelGGL((combine_kernel<bf16_t, bf16_t>), dim3(grid), dim3(256), 0, s,
-                         static_cast<const bf16_t*>(yw), T, H, k, static_cast<bf16_t*>(out));
+                         static_cast<const bf16_t*>(yw), idx, E, T, H, k, static_cast<bf16_t*>(out));
   } else if (dtype == BIBO_DTYPE_BF16) {
-    hipLaunchKernelGGL((combine_kernel<float, bf16_t>), dim3(grid), dim3(256), 0, s, static_cast<const float*>(yw), T,
-                       H, k, static_cast<bf16_t*>(out));
+    hipLaunchKernelGGL((combine_kernel<float, bf16_t>), dim3(grid), dim3(256), 0, s, static_cast<const float*>(yw), idx,
+                       E, T, H, k, static_cast<bf16_t*>(out));
   } else {
-    hipLaunchKernelGGL((combine_kernel<float, float>), dim3(grid), dim3(256), 0, s, static_cast<const float*>(yw), T,
-                       H, k, static_cast<float*>(out));
+    hipLaunchKernelGGL((combine_kernel<float, float>), dim3(grid), dim3(256), 0, s, static_cast<const float*>(yw), idx,
+                       E, T, H, k, static_cast<float*>(out));
   }
   return hipGetLastError();
 }

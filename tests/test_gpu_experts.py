@@ -135,6 +135,44 @@ def test_streaming_kernels_match_oracle(T, H, I, k, theta):
     assert rel_err(out, gen) <= 1e-2
 
 
+def test_streaming_kernels_without_the_permutation_pass():
+    """Without a counts request the composite call launches no permutation: the streaming kernels scan the
+    routing indices themselves.  Same bits either way."""
+    p = O.make_inputs(T=64, H=1024, E=64, k=6, I=512, bias="uniform", theta="normal", seed=99)
+    idx, w = _route(p)
+    args = (p["x"].to(DEV), torch.from_numpy(idx).to(DEV), torch.from_numpy(w).to(DEV), p["w_gate_up"].to(DEV),
+            p["w_down"].to(DEV), p["theta"].to(DEV))
+    with_counts, _ = ops.experts_fwd(*args, algo="stream", want_counts=True)
+    without, none = ops.experts_fwd(*args, algo="stream", want_counts=False)
+    torch.cuda.synchronize()
+    assert none is None and torch.equal(with_counts, without)
+    ref = O.experts_forward(p["x"], idx, w, p["w_gate_up"], p["w_down"], p["theta"])
+    assert rel_err(without.cpu(), ref) <= BF16_TOL
+
+
+@pytest.mark.parametrize("algo,T,H,I", [("generic", 40, 256, 128), ("mfma", 400, 256, 128), ("fused", 400, 256, 128),
+                                        ("stream", 40, 256, 128)])
+def test_slots_without_an_expert_contribute_nothing(algo, T, H, I):
+    """Routing indices outside [0,E) (the reference never produces them; a caller might use them as padding) get
+    no row, and the combine skips their slot."""
+    p = O.make_inputs(T=T, H=H, E=64, k=6, I=I, bias="uniform", theta="normal", seed=T + 1)
+    idx, w = _route(p)
+    bad = idx.copy()
+    bad[::3, 1] = 64
+    bad[1::5, 4] = -1
+    w0 = w.copy()
+    w0[::3, 1] = 0.0
+    w0[1::5, 4] = 0.0
+    ref = O.experts_forward(p["x"], idx, w0, p["w_gate_up"], p["w_down"], p["theta"])   # same slots, weight zero
+    # poison the workspace so that an unwritten slot row cannot pass by luck
+    ops.workspace(DEV, 64 << 20).fill_(0x7f)
+    out, counts = _gpu_experts(p, bad, w, algo)
+    assert torch.isfinite(out.float()).all()
+    assert rel_err(out, ref) <= BF16_TOL
+    keep = (bad >= 0) & (bad < 64)
+    assert np.array_equal(counts, np.bincount(bad[keep], minlength=64))
+
+
 def test_streaming_kernels_with_a_crowded_expert():
     """Every row on two experts (far more than 16 rows each): the pass loop re-streams the weights."""
     p = O.make_inputs(T=90, H=512, E=64, k=2, I=256, theta="normal", seed=21)
