@@ -231,16 +231,103 @@ __device__ __forceinline__ void select_tokens16(const float* __restrict__ sc, co
   }
 }
 
-// ---- MFMA router: bf16, H % 32 == 0 -------------------------------------------------------------
-// One workgroup = 16 tokens, 4 waves.  The waves split K (32-wide steps round-robin); each keeps
-// four 16x16 fp32 accumulators (64 experts), partials are summed through LDS in wave order.
+// ---- MFMA router: bf16, H % 128 == 0 ------------------------------------------------------------
+// One workgroup = TOK tokens (16 or 32), TOK/16 x 4 waves: wave (tm, en) owns the 16x16 logits tile of
+// token tile tm and expert tile en over the whole K, so no partial sums cross waves and the fp32
+// accumulation order is fixed.  x rows and w_router rows travel global -> LDS by LDS-DMA in K chunks of
+// 128 elements (256-byte rows, one instruction fetches four whole rows per wave), double-buffered:
+// fetching w_router straight into registers costs a CU about 37 GB/s, the DMA path twice that, and
+// every workgroup needs all of w_router.  Granule c of row r sits at position c ^ (r & 15).
+constexpr int kRouterKC = 128;                       // K elements per chunk
+constexpr int kRouterGran = kRouterKC / 8;           // 16-byte granules per chunk row
+
+typedef __attribute__((address_space(3))) void router_lds_void;
+typedef const __attribute__((address_space(1))) void router_gbl_void;
+
+template <int TOK>
+__global__ __launch_bounds__(TOK * 16) void router_mfma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wr,
+                                                               const float* __restrict__ bias, int T, int H, int E,
+                                                               int k, int norm_mode, float* __restrict__ logits,
+                                                               int32_t* __restrict__ idx, float* __restrict__ w,
+                                                               float* __restrict__ gap) {
+  constexpr int kThreads = TOK * 16;
+  constexpr int kRows = TOK + kMaxE;                 // stage rows: tokens first, then experts
+  constexpr int kPer = kRows * kRouterGran / kThreads;   // load instructions per thread and chunk
+  static_assert(kRows * kRouterGran % kThreads == 0, "stage does not divide over the threads");
+  __shared__ __attribute__((aligned(16))) bf16_t st0[kRows * kRouterKC];
+  __shared__ __attribute__((aligned(16))) bf16_t st1[kRows * kRouterKC];
+  __shared__ float sc[TOK * kRowPad];
+  __shared__ float bias_s[kMaxE];
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63;
+  const int t0 = blockIdx.x * TOK;
+  if (tid < kMaxE) bias_s[tid] = (tid < E) ? bias[tid] : 0.f;
+
+  // thread t of load instruction i fills granule i*kThreads + t = (row, position t % 16) and fetches logical
+  // granule (t % 16) ^ (row % 16) of that row
+  const bf16_t* src[kPer];
+#pragma unroll
+  for (int i = 0; i < kPer; ++i) {
+    const int row = (i * kThreads + tid) / kRouterGran;
+    const int c = (tid & (kRouterGran - 1)) ^ (row & 15);
+    src[i] = (row < TOK ? x + (size_t)min(t0 + row, T - 1) * H : wr + (size_t)min(row - TOK, E - 1) * H) + c * 8;
+  }
+  auto issue = [&](int k0, bf16_t* st) {
+#pragma unroll
+    for (int i = 0; i < kPer; ++i)
+      __builtin_amdgcn_global_load_lds((router_gbl_void*)(src[i] + k0), (router_lds_void*)(st + (i * kThreads + wave * 64) * 8),
+                                       16, 0, 0);
+  };
+  const int tm = wave >> 2, en = wave & 3;
+  const int r16 = lane & 15, kc = lane >> 4;         // fragment row, 8-wide k chunk of a 32-wide step
+  floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+  auto multiply = [&](const bf16_t* st) {
+    const bf16_t* arow = st + (tm * 16 + r16) * kRouterKC;
+    const bf16_t* brow = st + (TOK + en * 16 + r16) * kRouterKC;
+#pragma unroll
+    for (int s = 0; s < kRouterKC / 32; ++s) {
+      const int pos = ((s * 4 + kc) ^ r16) * 8;      // both rows are r16 mod 16
+      const bf16x8 a = *reinterpret_cast<const bf16x8*>(arow + pos);
+      const bf16x8 b = *reinterpret_cast<const bf16x8*>(brow + pos);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+    }
+  };
+  issue(0, st0);
+  for (int k0 = 0; k0 < H; k0 += 2 * kRouterKC) {
+    __builtin_amdgcn_s_waitcnt(0);                   // vmcnt(0): this thread's transfers have landed
+    __syncthreads();
+    if (k0 + kRouterKC < H) issue(k0 + kRouterKC, st1);
+    multiply(st0);
+    if (k0 + kRouterKC < H) {
+      __builtin_amdgcn_s_waitcnt(0);
+      __syncthreads();
+      if (k0 + 2 * kRouterKC < H) issue(k0 + 2 * kRouterKC, st0);
+      multiply(st1);
+    }
+  }
+  // D layout of the 16x16 tile: lane holds column (expert) lane%16, rows (tokens) 4*(lane/16)+i
+  const int ntok = min(TOK, T - t0);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int tl = tm * 16 + kc * 4 + i, e = en * 16 + r16;
+    if (tl < ntok && e < E) {
+      const float lg = acc[i];
+      if (logits != nullptr) logits[(size_t)(t0 + tl) * E + e] = lg;
+      sc[tl * kRowPad + e] = sigmoid32_canonical(lg);          // router.py:31
+    }
+  }
+  __syncthreads();
+  select_tokens16(sc, bias_s, E, k, norm_mode, t0, ntok, idx, w, gap);
+}
+
+// ---- MFMA router for H % 32 == 0 but not % 128: operands straight to registers, K split over 4 waves ----
 constexpr int kMfmaTokens = 16;
 
-__global__ __launch_bounds__(256) void router_mfma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wr,
-                                                          const float* __restrict__ bias, int T, int H, int E, int k,
-                                                          int norm_mode, float* __restrict__ logits,
-                                                          int32_t* __restrict__ idx, float* __restrict__ w,
-                                                          float* __restrict__ gap) {
+__global__ __launch_bounds__(256) void router_mfma_split_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wr,
+                                                                const float* __restrict__ bias, int T, int H, int E,
+                                                                int k, int norm_mode, float* __restrict__ logits,
+                                                                int32_t* __restrict__ idx, float* __restrict__ w,
+                                                                float* __restrict__ gap) {
   __shared__ float part[4 * kMfmaTokens * kRowPad];
   __shared__ float sc[kMfmaTokens * kRowPad];
   __shared__ float bias_s[kMaxE];
@@ -305,9 +392,18 @@ hipError_t launch_router(const void* x, const void* w_router, const float* bias,
                          int norm_mode, float* logits, int32_t* idx, float* w, float* gap, hipStream_t s) {
   if (T == 0) return hipSuccess;
   const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w_router)) & 15) == 0;
-  if (dtype == BIBO_DTYPE_BF16 && (H % 32) == 0 && aligned) {
+  if (dtype == BIBO_DTYPE_BF16 && (H % kRouterKC) == 0 && aligned) {
+    // 32 tokens per workgroup halve the w_router traffic per token; below 256 workgroups' worth of tokens the
+    // smaller tile keeps more CUs busy
+    if (T >= 32 * 256)
+      hipLaunchKernelGGL(router_mfma_kernel<32>, dim3((T + 31) / 32), dim3(512), 0, s, static_cast<const bf16_t*>(x),
+                         static_cast<const bf16_t*>(w_router), bias, T, H, E, k, norm_mode, logits, idx, w, gap);
+    else
+      hipLaunchKernelGGL(router_mfma_kernel<16>, dim3((T + 15) / 16), dim3(256), 0, s, static_cast<const bf16_t*>(x),
+                         static_cast<const bf16_t*>(w_router), bias, T, H, E, k, norm_mode, logits, idx, w, gap);
+  } else if (dtype == BIBO_DTYPE_BF16 && (H % 32) == 0 && aligned) {
     const int grid = (T + kMfmaTokens - 1) / kMfmaTokens;
-    hipLaunchKernelGGL(router_mfma_kernel, dim3(grid), dim3(256), 0, s, static_cast<const bf16_t*>(x),
+    hipLaunchKernelGGL(router_mfma_split_kernel, dim3(grid), dim3(256), 0, s, static_cast<const bf16_t*>(x),
                        static_cast<const bf16_t*>(w_router), bias, T, H, E, k, norm_mode, logits, idx, w, gap);
   } else {
     const int grid = (T + kGenTokens - 1) / kGenTokens;

@@ -46,6 +46,15 @@ def test_router_ragged_token_counts(T):
     _check(p["x"], p["w_router"] * 8, p["bias"], 6)
 
 
+@pytest.mark.parametrize("T,H,E,k", [(8192, 768, 64, 6), (8209, 256, 64, 6), (8200, 128, 33, 3)])
+def test_router_large_token_counts_use_the_32_token_tile(T, H, E, k):
+    g = torch.Generator().manual_seed(T + E)
+    x = torch.randn(T, H, generator=g).bfloat16()
+    wr = (torch.randn(E, H, generator=g) * 0.1).bfloat16()
+    bias = torch.rand(E, generator=g) * 0.02 - 0.01
+    _check(x, wr, bias, k, gap=True)
+
+
 @pytest.mark.parametrize("E,k,H,dtype", [(8, 2, 64, torch.bfloat16), (22, 2, 64, torch.float32),
                                          (4, 1, 40, torch.bfloat16), (5, 5, 64, torch.float32),
                                          (64, 8, 100, torch.bfloat16), (33, 3, 96, torch.bfloat16)])
