@@ -15,7 +15,7 @@ constexpr float kNormSiluEps = 1e-6f;   // src/modeling/ffn/moe.py:16
 constexpr float kSumNormEps = 1e-20f;   // src/modeling/ffn/router.py:45
 
 // tokens handled by one workgroup of the histogram / permutation kernels
-constexpr int kPermTokens = 256;
+constexpr int kPermTokens = 128;   // tokens per permutation workgroup (256 and 64 measured slower)
 constexpr int kStreamMaxSlots = 2048;   // routed slots the weight-streaming kernels can scan per workgroup
 
 typedef __bf16 bf16_t;

@@ -24,7 +24,7 @@ __global__ __launch_bounds__(256) void hist_kernel(const int32_t* __restrict__ i
   if (tid < kMaxE) block_hist[blockIdx.x * kMaxE + tid] = h[tid];
 }
 
-// One workgroup per chunk of kPermTokens tokens, four waves of 64 tokens each, lane = expert for the
+// One workgroup per chunk of kPermTokens tokens, four waves of kPermTokens/4 tokens each, lane = expert for the
 // bookkeeping.  (1) every wave counts its own slots per expert; (2) the chunk histograms are summed
 // (all chunks for the totals, earlier chunks for this chunk's base) with the loads spread over the
 // 256 threads; (3) exclusive scan over experts; (4) every wave ranks its slots 64 at a time, slots of
@@ -36,8 +36,8 @@ __global__ __launch_bounds__(256) void scatter_kernel(const int32_t* __restrict_
   __shared__ int part_tot[4][kMaxE], part_bef[4][kMaxE], wave_cnt[4][kMaxE];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int b = blockIdx.x;
-  const int s0 = (b * kPermTokens + wave * 64) * k;
-  const int s1 = min(S, s0 + 64 * k);
+  const int s0 = (b * kPermTokens + wave * (kPermTokens / 4)) * k;
+  const int s1 = min(S, s0 + (kPermTokens / 4) * k);
   const unsigned long long lt = (1ull << lane) - 1ull;
 
   int mycnt = 0;                                  // slots of expert `lane` among this wave's tokens
@@ -54,10 +54,19 @@ __global__ __launch_bounds__(256) void scatter_kernel(const int32_t* __restrict_
   wave_cnt[wave][lane] = mycnt;
 
   int tot = 0, bef = 0;
-  for (int bb = wave; bb < nblk; bb += 4) {
-    const int v = block_hist[bb * kMaxE + lane];
-    tot += v;
-    bef += (bb < b) ? v : 0;
+  constexpr int kBatch = 16;                       // chunk histograms requested together: one memory latency per batch
+  for (int bb0 = wave; bb0 < nblk; bb0 += 4 * kBatch) {
+    int v[kBatch];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int bb = bb0 + 4 * u;
+      v[u] = (bb < nblk) ? block_hist[bb * kMaxE + lane] : 0;
+    }
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      tot += v[u];
+      bef += (bb0 + 4 * u < b) ? v[u] : 0;
+    }
   }
   part_tot[wave][lane] = tot;
   part_bef[wave][lane] = bef;

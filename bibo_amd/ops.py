@@ -100,7 +100,7 @@ def permute(idx, E):
     offsets = torch.empty(E + 1, dtype=torch.int32, device=dev)
     perm_slot = torch.empty(T * k, dtype=torch.int32, device=dev)
     perm_token = torch.empty(T * k, dtype=torch.int32, device=dev)
-    nb = max(1, (T + 255) // 256) * 64 * 4
+    nb = max(1, (T + 127) // 128) * 64 * 4          # one 64-entry histogram per 128 tokens
     ws = workspace(dev, nb)
     with torch.cuda.device(dev):
         L.check(L.lib().bibo_moe_permute(_ptr(idx), T, E, k, _ptr(counts), _ptr(offsets), _ptr(perm_slot),
