@@ -86,13 +86,15 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
   floatx16 acc[MT][NTW];
   {
     StripeLoader<S1> ld;
+    ld.b_src = wgu + ((size_t)e * 2 * I + S1::dma_row(tid)) * H + chunk * 8;
+    ld.bstep = (size_t)S1::kRowsPerInstr * H;
+    ld.issue_b(0, P);                        // weight rows first: they do not wait for the row indices
 #pragma unroll
     for (int i = 0; i < S1::A_PER; ++i) {
       const int m = min(S1::dma_row(tid) + i * S1::kRowsPerInstr, rows - 1);   // rows past the end re-read the last valid row
       ld.a_src[i] = x + (size_t)perm_token[row0 + m] * H + chunk * 8;
     }
-    ld.b_src = wgu + ((size_t)e * 2 * I + S1::dma_row(tid)) * H + chunk * 8;
-    ld.bstep = (size_t)S1::kRowsPerInstr * H;
+    ld.issue_a(0, P);
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll

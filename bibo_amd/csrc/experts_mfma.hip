@@ -46,13 +46,15 @@ __global__ __launch_bounds__(256 * WM) void gateup_dma_kernel(const bf16_t* __re
   const int wn = wave & 3, wm = wave >> 2;
   const int chunk = S::dma_chunk(tid);
   StripeLoader<S> ld;
+  ld.b_src = wgu + ((size_t)e * 2 * I + S::dma_row(tid)) * H + chunk * 8;
+  ld.bstep = (size_t)S::kRowsPerInstr * H;
+  ld.issue_b(0, st0);                    // weight rows first: they do not wait for the row indices
 #pragma unroll
   for (int i = 0; i < S::A_PER; ++i) {
     const int m = min(S::dma_row(tid) + i * S::kRowsPerInstr, rows - 1);     // rows past the end re-read the last valid row
     ld.a_src[i] = x + (size_t)perm_token[row0 + m] * H + chunk * 8;     // gather, moe.py:81
   }
-  ld.b_src = wgu + ((size_t)e * 2 * I + S::dma_row(tid)) * H + chunk * 8;
-  ld.bstep = (size_t)S::kRowsPerInstr * H;
+  ld.issue_a(0, st0);
   floatx16 acc[MT][NTW];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
@@ -157,6 +159,7 @@ __global__ __launch_bounds__(256 * WM) void down_dma_kernel(const bf16_t* __rest
   const int n0 = nb * BN;
   ld.b_src = wd + ((size_t)e * H + n0 + S::dma_row(tid)) * I + chunk * 8;
   ld.bstep = (size_t)S::kRowsPerInstr * I;
+  ld.issue_stage(0, st0);
   floatx16 acc[MT][NTW];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)

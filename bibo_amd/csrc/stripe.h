@@ -109,6 +109,17 @@ struct StripeLoader {
   __device__ __forceinline__ void issue_stage(int k0, bf16_t* stage) const {
     issue_all(k0, stage, std::make_integer_sequence<int, kInstr>{});
   }
+  // the two halves of a stage separately: the B rows need no row indices and can be requested first
+  template <int... Qs>
+  __device__ __forceinline__ void issue_b_all(int k0, bf16_t* stage, std::integer_sequence<int, Qs...>) const {
+    (issue<S::A_PER + Qs>(k0, stage), ...);
+  }
+  __device__ __forceinline__ void issue_b(int k0, bf16_t* stage) const {
+    issue_b_all(k0, stage, std::make_integer_sequence<int, S::B_PER>{});
+  }
+  __device__ __forceinline__ void issue_a(int k0, bf16_t* stage) const {
+    issue_all(k0, stage, std::make_integer_sequence<int, S::A_PER>{});
+  }
 };
 
 // One (k16 sub-step, N tile) pair of the software pipeline below; Q is a compile-time index so the
@@ -200,11 +211,11 @@ __device__ __forceinline__ void wait_loads_and_sync() {
   __syncthreads();
 }
 
+// The caller has already requested stage 0 into st0 (issue_b, then issue_a once the row indices are known).
 template <int MT, int NTW, int WM, int BK, typename FragRow>
 __device__ __forceinline__ void stripe_mainloop_dma(floatx16 (&acc)[MT][NTW],
                                                     const StripeLoader<Stripe<MT, NTW, WM, BK>>& ld, int K, bf16_t* st0,
                                                     bf16_t* st1, int wm, FragRow frag_row) {
-  ld.issue_stage(0, st0);
   for (int k0 = 0; k0 < K; k0 += 2 * BK) {
     wait_loads_and_sync();
     stripe_compute<MT, NTW, WM, BK>(acc, st0, wm, frag_row, ld, k0 + BK < K, k0 + BK, st1);
