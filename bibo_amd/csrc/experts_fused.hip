@@ -2,7 +2,7 @@
 // projection, Radial NormSiLU and the down projection without the activations leaving the CU.
 //
 // Phase 1 is the gate/up main loop of gateup_dma_kernel (x rows and w_gate_up rows by LDS-DMA, two
-// stages `P` and `Q`).  Phase 2 turns the accumulators into bf16 activations and parks them in LDS as an
+// stages `P` and `Q`) with the MFMA operands swapped, so a lane ends up with one ROW's values.  Phase 2 turns the accumulators into bf16 activations and parks them in LDS as an
 // operand of the second GEMM: rows 0..63 live in P, rows 64..127 in Q, whose stage contents are dead by
 // then; row r keeps 16-byte granule c at position c ^ (r & 15), which spreads the 16 lanes of a fragment
 // read over all banks although the row stride is a multiple of 256 bytes.
@@ -102,22 +102,26 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[mt][j][i] = 0.f;
     auto frag_row = [&](int j) { return (j < NT ? 0 : I) + (wn * NT + (j < NT ? j : j - NT)) * 32; };
-    stripe_mainloop_dma<MT, NTW, F::WM, S1::BK>(acc, ld, H, P, Q, wm, frag_row);
+    stripe_mainloop_dma<MT, NTW, F::WM, S1::BK, true>(acc, ld, H, P, Q, wm, frag_row);
   }
   __syncthreads();                         // every wave is done with the gate/up stages
 
   // ---- phase 2: Radial NormSiLU (moe.py:87-92), activations to LDS ----
+  // The accumulators are transposed (lane = row mbase + 32*mt + n, register i = column acc_row(i, lane) of
+  // its 32-column tile), so a row's sum of gate^2 is a sum over this lane's registers, the lane with the
+  // other half of the columns (lane ^ 32) and the four N waves; and every lane owns runs of four
+  // consecutive columns, which leave as one 8-byte LDS write.
+  const int hh = lane >> 5;
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
+  for (int mt = 0; mt < MT; ++mt) {
+    float sq = 0.f;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      float sq = 0.f;
+    for (int j = 0; j < NT; ++j)
 #pragma unroll
-      for (int j = 0; j < NT; ++j) sq = fmaf(acc[mt][j][i], acc[mt][j][i], sq);
-#pragma unroll
-      for (int o = 16; o > 0; o >>= 1) sq += __shfl_xor(sq, o, kWave);
-      if (n == 0) ssq[wn * BM + mbase + mt * 32 + acc_row(i, lane)] = sq;
-    }
+      for (int i = 0; i < 16; ++i) sq = fmaf(acc[mt][j][i], acc[mt][j][i], sq);
+    sq += __shfl_xor(sq, 32, kWave);
+    if (hh == 0) ssq[wn * BM + mbase + mt * 32 + n] = sq;
+  }
   __syncthreads();
   if (tid < BM) {
     const float p = 1.f / (1.f + __expf(-theta[e]));                                  // moe.py:89
@@ -133,20 +137,26 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
   {
     bf16_t* hsel = wm ? Q : P;             // activations of this wave's M half, [64][I], granules swizzled
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
+    for (int mt = 0; mt < MT; ++mt) {
+      const int ml = mt * 32 + n;
+      const float rinv = rinv_s[mbase + ml];
+      const float nrl = -1.44269504f * rinv, rg = rinv * gain_s[mbase + ml];   // per-row constants folded once
+      bf16_t* hrow = hsel + ml * I + 4 * hh;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int ml = mt * 32 + acc_row(i, lane);
-        const float rinv = rinv_s[mbase + ml], gain = gain_s[mbase + ml];
-        bf16_t* hrow = hsel + ml * I + (n & 7);
+      for (int j = 0; j < NT; ++j)
 #pragma unroll
-        for (int j = 0; j < NT; ++j) {
-          const float z = acc[mt][j][i] * rinv;
-          const float sg = __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-1.44269504f * z));
-          const int c = (wn * NT + j) * 4 + (n >> 3);                                   // logical granule of this column
-          hrow[(c ^ (ml & 15)) * 8] = (bf16_t)(z * sg * gain * acc[mt][NT + j][i]);     // SiLU(g/r) r^p up
+        for (int q = 0; q < 4; ++q) {        // columns (wn*NT + j)*32 + 8*q + 4*hh + 0..3: half of granule (wn*NT + j)*4 + q
+          bf16x4 hv;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const float g = acc[mt][j][4 * q + r];
+            const float sg = __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(g * nrl));   // sigmoid(g/r)
+            hv[r] = (bf16_t)(g * rg * sg * acc[mt][NT + j][4 * q + r]);                // SiLU(g/r) r^p up
+          }
+          const int c = (wn * NT + j) * 4 + q;
+          *reinterpret_cast<bf16x4*>(hrow + (c ^ (ml & 15)) * 8) = hv;
         }
-      }
+    }
   }
   __syncthreads();                         // the activation tile is complete
 

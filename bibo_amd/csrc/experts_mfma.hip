@@ -63,7 +63,7 @@ __global__ __launch_bounds__(256 * WM) void gateup_dma_kernel(const bf16_t* __re
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[mt][j][i] = 0.f;
   auto frag_row = [&](int j) { return (j < NT ? 0 : I) + (wn * NT + (j < NT ? j : j - NT)) * 32; };
-  stripe_mainloop_dma<MT, NTW, WM, S::BK>(acc, ld, H, st0, st1, wm, frag_row);
+  stripe_mainloop_dma<MT, NTW, WM, S::BK, false>(acc, ld, H, st0, st1, wm, frag_row);
 
   // ---- Radial NormSiLU epilogue (moe.py:87-92) ----
   // (1) sum of gate^2 per row: registers -> 32-lane shuffle -> LDS across the four N waves;
@@ -168,7 +168,7 @@ __global__ __launch_bounds__(256 * WM) void down_dma_kernel(const bf16_t* __rest
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[mt][j][i] = 0.f;
   auto frag_row = [&](int j) { return (wn * NTW + j) * 32; };
-  stripe_mainloop_dma<MT, NTW, WM, S::BK>(acc, ld, I, st0, st1, wm, frag_row);
+  stripe_mainloop_dma<MT, NTW, WM, S::BK, false>(acc, ld, I, st0, st1, wm, frag_row);
 
   // Epilogue: scale by the routing weight (moe.py:93), park kPassRows rows at a time in a wave-private
   // LDS tile and scatter them to slot order as 16-byte row segments.

@@ -127,7 +127,7 @@ struct StripeLoader {
 // (if there is one): spreading the loads through the MFMAs keeps the waves from queueing up at the
 // texture-address unit before they start multiplying.  `a1` points at this lane's A fragment of the
 // second sub-step for M tile 0; tile mt is `astride` elements further.
-template <int Q, int MT, int NTW, int BK, typename Loader, typename FragRow>
+template <int Q, int MT, int NTW, int BK, bool TR, typename Loader, typename FragRow>
 __device__ __forceinline__ void stripe_pair(floatx16 (&acc)[MT][NTW], bf16x8 (&a)[2][MT], bf16x8 (&b)[3],
                                             const bf16_t* a0, int astride, const bf16_t* bstage, int pos0,
                                             FragRow frag_row, const Loader& ld, bool prefetch, int k_next,
@@ -154,18 +154,19 @@ __device__ __forceinline__ void stripe_pair(floatx16 (&acc)[MT][NTW], bf16x8 (&a
     a[(s + 1) & 1][mt] = *reinterpret_cast<const bf16x8*>(a0 + mt * astride + ((pos0 ^ ((s + 1) * 16)) - pos0));
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
-    acc[mt][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[s & 1][mt], b[Q % 3], acc[mt][j], 0, 0, 0);
+    acc[mt][j] = TR ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[Q % 3], a[s & 1][mt], acc[mt][j], 0, 0, 0)
+                    : __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[s & 1][mt], b[Q % 3], acc[mt][j], 0, 0, 0);
   constexpr int kReads = (Q + 2 < kPairs ? 1 : 0) + (kALast >= kAFirst ? kALast - kAFirst + 1 : 0);
   if constexpr (kReads > 0) __builtin_amdgcn_sched_group_barrier(0x100, kReads, 0);
   __builtin_amdgcn_sched_group_barrier(0x008, MT, 0);
 }
 
-template <int MT, int NTW, int BK, typename Loader, typename FragRow, int... Qs>
+template <int MT, int NTW, int BK, bool TR, typename Loader, typename FragRow, int... Qs>
 __device__ __forceinline__ void stripe_pairs(floatx16 (&acc)[MT][NTW], bf16x8 (&a)[2][MT], bf16x8 (&b)[3],
                                              const bf16_t* a0, int astride, const bf16_t* bstage, int pos0,
                                              FragRow frag_row, const Loader& ld, bool prefetch, int k_next,
                                              bf16_t* next_stage, std::integer_sequence<int, Qs...>) {
-  (stripe_pair<Qs, MT, NTW, BK>(acc, a, b, a0, astride, bstage, pos0, frag_row, ld, prefetch, k_next, next_stage), ...);
+  (stripe_pair<Qs, MT, NTW, BK, TR>(acc, a, b, a0, astride, bstage, pos0, frag_row, ld, prefetch, k_next, next_stage), ...);
 }
 
 // Multiply one K step of BK into the accumulators while the load instructions of the next stage are
@@ -174,7 +175,7 @@ __device__ __forceinline__ void stripe_pairs(floatx16 (&acc)[MT][NTW], bf16x8 (&
 // of the next sub-step are read while the current one is still multiplying.  a0: this lane's A
 // fragment of sub-step 0 for M tile 0 (position pos0 of its row; sub-step s sits at pos0 ^ 16s, M tile
 // mt `astride` elements further); bstage: this lane's row of the B stage (N tile 0).
-template <int MT, int NTW, int BK, typename Loader, typename FragRow>
+template <int MT, int NTW, int BK, bool TR, typename Loader, typename FragRow>
 __device__ __forceinline__ void stripe_step(floatx16 (&acc)[MT][NTW], const bf16_t* a0, int astride, const bf16_t* bstage,
                                             int pos0, FragRow frag_row, const Loader& ld, bool prefetch, int k_next,
                                             bf16_t* next_stage) {
@@ -186,12 +187,12 @@ __device__ __forceinline__ void stripe_step(floatx16 (&acc)[MT][NTW], const bf16
   b[0] = *reinterpret_cast<const bf16x8*>(bstage + frag_row(0) * BK + pos0);
   b[1] = *reinterpret_cast<const bf16x8*>(bstage + frag_row(NTW > 1 ? 1 : 0) * BK + (NTW > 1 ? pos0 : (pos0 ^ 16)));
   __builtin_amdgcn_sched_group_barrier(0x100, MT + 2, 0);
-  stripe_pairs<MT, NTW, BK>(acc, a, b, a0, astride, bstage, pos0, frag_row, ld, prefetch, k_next, next_stage,
+  stripe_pairs<MT, NTW, BK, TR>(acc, a, b, a0, astride, bstage, pos0, frag_row, ld, prefetch, k_next, next_stage,
                             std::make_integer_sequence<int, SS * NTW>{});
 }
 
 // A and B both come from `stage` (A rows first).
-template <int MT, int NTW, int WM, int BK, typename FragRow>
+template <int MT, int NTW, int WM, int BK, bool TR, typename FragRow>
 __device__ __forceinline__ void stripe_compute(floatx16 (&acc)[MT][NTW], const bf16_t* stage, int wm, FragRow frag_row,
                                                const StripeLoader<Stripe<MT, NTW, WM, BK>>& ld, bool prefetch,
                                                int k_next, bf16_t* next_stage) {
@@ -203,7 +204,7 @@ __device__ __forceinline__ void stripe_compute(floatx16 (&acc)[MT][NTW], const b
   const int pos0 = (h ^ ((n >> S::kSwzShift) & (S::GPR - 1))) * 8;
   const bf16_t* astage = stage + (wm * MT * 32 + n) * BK;
   const bf16_t* bstage = stage + (S::BM + n) * BK;
-  stripe_step<MT, NTW, BK>(acc, astage + pos0, 32 * BK, bstage, pos0, frag_row, ld, prefetch, k_next, next_stage);
+  stripe_step<MT, NTW, BK, TR>(acc, astage + pos0, 32 * BK, bstage, pos0, frag_row, ld, prefetch, k_next, next_stage);
 }
 
 __device__ __forceinline__ void wait_loads_and_sync() {
@@ -212,16 +213,19 @@ __device__ __forceinline__ void wait_loads_and_sync() {
 }
 
 // The caller has already requested stage 0 into st0 (issue_b, then issue_a once the row indices are known).
-template <int MT, int NTW, int WM, int BK, typename FragRow>
+// TR = false: accumulator tile [mt][j] holds rows x columns in the MFMA D layout (lane = column, registers =
+// rows, see acc_row).  TR = true: the operands are swapped and the tile is transposed: lane = ROW (lane % 32),
+// register i = COLUMN acc_row(i, lane), so a lane owns runs of four consecutive columns of one row.
+template <int MT, int NTW, int WM, int BK, bool TR, typename FragRow>
 __device__ __forceinline__ void stripe_mainloop_dma(floatx16 (&acc)[MT][NTW],
                                                     const StripeLoader<Stripe<MT, NTW, WM, BK>>& ld, int K, bf16_t* st0,
                                                     bf16_t* st1, int wm, FragRow frag_row) {
   for (int k0 = 0; k0 < K; k0 += 2 * BK) {
     wait_loads_and_sync();
-    stripe_compute<MT, NTW, WM, BK>(acc, st0, wm, frag_row, ld, k0 + BK < K, k0 + BK, st1);
+    stripe_compute<MT, NTW, WM, BK, TR>(acc, st0, wm, frag_row, ld, k0 + BK < K, k0 + BK, st1);
     if (k0 + BK < K) {
       wait_loads_and_sync();
-      stripe_compute<MT, NTW, WM, BK>(acc, st1, wm, frag_row, ld, k0 + 2 * BK < K, k0 + 2 * BK, st0);
+      stripe_compute<MT, NTW, WM, BK, TR>(acc, st1, wm, frag_row, ld, k0 + 2 * BK < K, k0 + 2 * BK, st0);
     }
   }
 }
