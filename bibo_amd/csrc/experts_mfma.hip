@@ -63,24 +63,26 @@ __global__ __launch_bounds__(256 * WM) void gateup_dma_kernel(const bf16_t* __re
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[mt][j][i] = 0.f;
   auto frag_row = [&](int j) { return (j < NT ? 0 : I) + (wn * NT + (j < NT ? j : j - NT)) * 32; };
-  stripe_mainloop_dma<MT, NTW, WM, S::BK, false>(acc, ld, H, st0, st1, wm, frag_row);
+  stripe_mainloop_dma<MT, NTW, WM, S::BK, true>(acc, ld, H, st0, st1, wm, frag_row);
 
   // ---- Radial NormSiLU epilogue (moe.py:87-92) ----
-  // (1) sum of gate^2 per row: registers -> 32-lane shuffle -> LDS across the four N waves;
-  // (2) one thread per row turns it into 1/r and r^p; (3) every lane applies SiLU(g/r) * r^p * up and
-  // parks its bf16 results in a wave-private LDS tile; (4) the tile leaves as 16-byte row segments.
+  // The accumulators are transposed (lane = row mbase + 32*mt + lane%32, register i = column acc_row(i, lane)
+  // of its 32-column tile).  (1) sum of gate^2 per row: this lane's registers, the lane with the other half
+  // of the columns (lane ^ 32), then LDS across the four N waves; (2) one thread per row turns it into 1/r
+  // and r^p; (3) every lane applies SiLU(g/r) * r^p * up and parks its bf16 results, four consecutive
+  // columns at a time, in a wave-private LDS tile; (4) the tile leaves as 16-byte row segments.
   const int mbase = wm * MT * 32;
+  const int n = lane & 31, hh = lane >> 5;
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
+  for (int mt = 0; mt < MT; ++mt) {
+    float sq = 0.f;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      float sq = 0.f;
+    for (int j = 0; j < NT; ++j)
 #pragma unroll
-      for (int j = 0; j < NT; ++j) sq = fmaf(acc[mt][j][i], acc[mt][j][i], sq);
-#pragma unroll
-      for (int o = 16; o > 0; o >>= 1) sq += __shfl_xor(sq, o, kWave);
-      if ((lane & 31) == 0) ssq[wn * BM + mbase + mt * 32 + acc_row(i, lane)] = sq;
-    }
+      for (int i = 0; i < 16; ++i) sq = fmaf(acc[mt][j][i], acc[mt][j][i], sq);
+    sq += __shfl_xor(sq, 32, kWave);
+    if (hh == 0) ssq[wn * BM + mbase + mt * 32 + n] = sq;
+  }
   __syncthreads();                       // also: every wave is done reading the stage buffers
   if (tid < BM) {
     const float p = 1.f / (1.f + __expf(-theta[e]));                                  // moe.py:89
@@ -91,22 +93,28 @@ __global__ __launch_bounds__(256 * WM) void gateup_dma_kernel(const bf16_t* __re
   }
   __syncthreads();
   constexpr int kOutCols = NT * 32;                 // gate-paired columns owned by this wave
-  constexpr int kOutStride = kOutCols + 8;          // bf16 elements; +16 bytes keeps the two lane halves apart
+  constexpr int kOutStride = kOutCols + 8;          // bf16 elements; +16 bytes staggers the rows over the banks
   bf16_t* otile = (wave < 4 * WM / 2 ? st0 : st1) + (wave % (4 * WM / 2)) * (MT * 32 * kOutStride);
   static_assert((4 * WM / 2) * MT * 32 * kOutStride <= S::kStageElems, "output staging does not fit a stage buffer");
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
+  for (int mt = 0; mt < MT; ++mt) {
+    const int ml = mt * 32 + n;
+    const float rinv = rinv_s[mbase + ml];
+    const float nrl = -1.44269504f * rinv, rg = rinv * gain_s[mbase + ml];            // per-row constants
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int ml = mt * 32 + acc_row(i, lane);
-      const float rinv = rinv_s[mbase + ml], gain = gain_s[mbase + ml];
+    for (int j = 0; j < NT; ++j)
 #pragma unroll
-      for (int j = 0; j < NT; ++j) {
-        const float z = acc[mt][j][i] * rinv;
-        const float sg = __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-1.44269504f * z));
-        otile[ml * kOutStride + j * 32 + (lane & 31)] = (bf16_t)(z * sg * gain * acc[mt][NT + j][i]);   // SiLU(g/r) r^p up
+      for (int q = 0; q < 4; ++q) {
+        bf16x4 hv;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float g = acc[mt][j][4 * q + r];
+          const float sg = __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(g * nrl));     // sigmoid(g/r)
+          hv[r] = (bf16_t)(g * rg * sg * acc[mt][NT + j][4 * q + r]);                  // SiLU(g/r) r^p up
+        }
+        *reinterpret_cast<bf16x4*>(otile + ml * kOutStride + j * 32 + 8 * q + 4 * hh) = hv;
       }
-    }
+  }
   __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): this wave's LDS writes are done (the tile is wave-private)
   __builtin_amdgcn_wave_barrier();
   constexpr int kGranPerRow = kOutCols / 8;
@@ -168,47 +176,45 @@ __global__ __launch_bounds__(256 * WM) void down_dma_kernel(const bf16_t* __rest
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[mt][j][i] = 0.f;
   auto frag_row = [&](int j) { return (wn * NTW + j) * 32; };
-  stripe_mainloop_dma<MT, NTW, WM, S::BK, false>(acc, ld, I, st0, st1, wm, frag_row);
+  stripe_mainloop_dma<MT, NTW, WM, S::BK, true>(acc, ld, I, st0, st1, wm, frag_row);
 
-  // Epilogue: scale by the routing weight (moe.py:93), park kPassRows rows at a time in a wave-private
-  // LDS tile and scatter them to slot order as 16-byte row segments.
+  // Epilogue (accumulators transposed: lane = row, four consecutive columns per register quad): scale by the
+  // routing weight (moe.py:93), park 32 rows at a time in a wave-private LDS tile and scatter them to slot
+  // order as 16-byte row segments.
+  static_assert(sizeof(TY) == 2, "the slot buffer of the MFMA kernels is bf16");
   const int mbase = wm * MT * 32;
+  const int n = lane & 31, hh = lane >> 5;
   constexpr int kOutCols = NTW * 32;
-  constexpr int kEltPer16 = 16 / sizeof(TY);
-  constexpr int kOutStride = kOutCols + kEltPer16;  // +16 bytes keeps the two lane halves on different banks
-  constexpr int kPassRows = sizeof(TY) == 2 ? 32 : 16;   // accumulator registers 8p .. 8p+7 hold rows 16p .. 16p+15
-  constexpr int kPasses = 32 / kPassRows;
-  static_assert((size_t)(4 * WM / 2) * kPassRows * kOutStride * sizeof(TY) <= (size_t)S::kStageElems * sizeof(bf16_t),
-                "output staging does not fit a stage buffer");
+  constexpr int kOutStride = kOutCols + 8;          // +16 bytes staggers the rows over the banks
+  static_assert((4 * WM / 2) * 32 * kOutStride <= S::kStageElems, "output staging does not fit a stage buffer");
   __syncthreads();                       // every wave is done reading the stage buffers
-  TY* otile = reinterpret_cast<TY*>(wave < 4 * WM / 2 ? st0 : st1) + (wave % (4 * WM / 2)) * (kPassRows * kOutStride);
-  constexpr int kGranPerRow = kOutCols / kEltPer16;
+  TY* otile = reinterpret_cast<TY*>(wave < 4 * WM / 2 ? st0 : st1) + (wave % (4 * WM / 2)) * (32 * kOutStride);
+  constexpr int kGranPerRow = kOutCols / 8;
   const int colbase = n0 + wn * kOutCols;
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
+  for (int mt = 0; mt < MT; ++mt) {
+    const float ws = w_s[mbase + mt * 32 + n];
 #pragma unroll
-    for (int ps = 0; ps < kPasses; ++ps) {
+    for (int j = 0; j < NTW; ++j)
 #pragma unroll
-      for (int ii = 0; ii < 16 / kPasses; ++ii) {
-        const int i = ps * (16 / kPasses) + ii;
-        const int ml = acc_row(i, lane) - ps * kPassRows;
-        const float ws = w_s[mbase + mt * 32 + acc_row(i, lane)];
+      for (int q = 0; q < 4; ++q) {
+        bf16x4 hv;
 #pragma unroll
-        for (int j = 0; j < NTW; ++j)
-          otile[ml * kOutStride + j * 32 + (lane & 31)] = from_float<TY>(ws * acc[mt][j][i]);
+        for (int r = 0; r < 4; ++r) hv[r] = (bf16_t)(ws * acc[mt][j][4 * q + r]);
+        *reinterpret_cast<bf16x4*>(otile + n * kOutStride + j * 32 + 8 * q + 4 * hh) = hv;
       }
-      __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
-      __builtin_amdgcn_wave_barrier();
-      for (int g = lane; g < kPassRows * kGranPerRow; g += kWave) {
-        const int ml = g / kGranPerRow, c = g - ml * kGranPerRow;
-        const int m = mbase + mt * 32 + ps * kPassRows + ml;
-        if (m < rows)
-          *reinterpret_cast<u32x4*>(yw + (size_t)slot_s[m] * H + colbase + c * kEltPer16) =
-              *reinterpret_cast<const u32x4*>(otile + ml * kOutStride + c * kEltPer16);
-      }
-      __builtin_amdgcn_s_waitcnt(0xc07f);
-      __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+    __builtin_amdgcn_wave_barrier();
+    for (int g = lane; g < 32 * kGranPerRow; g += kWave) {
+      const int ml = g / kGranPerRow, c = g - ml * kGranPerRow;
+      const int m = mbase + mt * 32 + ml;
+      if (m < rows)
+        *reinterpret_cast<u32x4*>(yw + (size_t)slot_s[m] * H + colbase + c * 8) =
+            *reinterpret_cast<const u32x4*>(otile + ml * kOutStride + c * 8);
     }
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    __builtin_amdgcn_wave_barrier();
+  }
 }
 
 inline int round_up8(int v) { return (v + 7) & ~7; }
