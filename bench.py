@@ -111,6 +111,26 @@ class Layer:
         if rc != 0:
             self.L.check(rc, "bibo_moe_forward")
 
+    def time_ffn_seam(self, steps, warmup):
+        """One call of the block's caller seam, out = h + moe(rmsnorm(h)) (bibo_moe_ffn_forward), per step."""
+        torch, L = self.torch, self.L
+        nbytes = ctypes.c_size_t(0)
+        L.check(self.lib.bibo_moe_ffn_workspace_bytes(ctypes.byref(self.shape), ctypes.byref(nbytes)), "ffn workspace")
+        ws = torch.empty(nbytes.value, dtype=torch.uint8, device=self.dev)
+        nw = torch.ones(self.H, dtype=torch.float32, device=self.dev)
+        P = lambda t: ctypes.c_void_p(t.data_ptr())
+        args = (P(self.x), P(nw), ctypes.c_float(1e-6), P(self.wr), P(self.bias), P(self.wgu), P(self.wd), P(self.theta),
+                ctypes.byref(self.shape), L.NORM_SUM, self.algo, P(self.out), None, None, None, P(ws), ws.numel(),
+                self.stream)
+        for _ in range(warmup):
+            L.check(self.lib.bibo_moe_ffn_forward(*args), "bibo_moe_ffn_forward")
+        torch.cuda.synchronize(self.dev)
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            self.lib.bibo_moe_ffn_forward(*args)
+        torch.cuda.synchronize(self.dev)
+        return (time.perf_counter() - t0) / steps
+
     def stage(self, name):
         fn, args = self._stages[name]
         rc = fn(*args)
@@ -236,6 +256,9 @@ def main():
                      "frac": dom_flops / stages[dom] / 1e12 / PEAK_BF16_TFLOPS,
                      "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, dom))},
     }
+    ffn_sec = layer.time_ffn_seam(args.steps, args.warmup)
+    out["ffn_seam"] = {"entry": "bibo_moe_ffn_forward: out = h + moe(rmsnorm(h))", "us_per_step": ffn_sec * 1e6,
+                       "extra_us_over_layer": (ffn_sec - sec) * 1e6}
     if not args.no_decode and args.workload == "c2":
         d = Layer("c3", dev, args.algo)
         drel, dact = d.check()

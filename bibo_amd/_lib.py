@@ -19,7 +19,8 @@ ABI_VERSION = 1
 SYMBOLS = (
     "bibo_moe_abi_version", "bibo_moe_strerror", "bibo_moe_workspace_bytes", "bibo_moe_router_fwd",
     "bibo_moe_permute", "bibo_moe_gateup_fwd", "bibo_moe_down_combine_fwd", "bibo_moe_gateup_down_fwd",
-    "bibo_moe_combine_fwd", "bibo_moe_experts_fwd", "bibo_moe_forward",
+    "bibo_moe_combine_fwd", "bibo_moe_experts_fwd", "bibo_moe_forward", "bibo_moe_rmsnorm_fwd",
+    "bibo_moe_ffn_workspace_bytes", "bibo_moe_ffn_forward",
 )
 
 
@@ -54,6 +55,13 @@ def _declare(l):
     l.bibo_moe_combine_fwd.argtypes = [vp, ci, ci, ci, ci, ci, vp, vp]
     l.bibo_moe_experts_fwd.restype = ci
     l.bibo_moe_experts_fwd.argtypes = [vp, vp, vp, vp, vp, vp, ctypes.POINTER(Shape), ci, vp, vp, vp, sz, vp]
+    l.bibo_moe_rmsnorm_fwd.restype = ci
+    l.bibo_moe_rmsnorm_fwd.argtypes = [vp, vp, ctypes.c_float, ci, ci, ci, vp, vp]
+    l.bibo_moe_ffn_workspace_bytes.restype = ci
+    l.bibo_moe_ffn_workspace_bytes.argtypes = [ctypes.POINTER(Shape), ctypes.POINTER(sz)]
+    l.bibo_moe_ffn_forward.restype = ci
+    l.bibo_moe_ffn_forward.argtypes = [vp, vp, ctypes.c_float, vp, vp, vp, vp, vp, ctypes.POINTER(Shape), ci, ci, vp, vp, vp,
+                                       vp, vp, sz, vp]
     l.bibo_moe_forward.restype = ci
     l.bibo_moe_forward.argtypes = [vp, vp, vp, vp, vp, vp, ctypes.POINTER(Shape), ci, ci, vp, vp, vp, vp, vp, vp, sz, vp]
 

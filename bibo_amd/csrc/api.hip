@@ -92,8 +92,8 @@ int gateup_dispatch(const void* x, const void* wgu, const float* theta, const in
 }
 
 int down_dispatch(const void* hidden, const void* wd, const int32_t* idx, const float* w, const int32_t* offsets,
-                  const int32_t* perm_slot, int T, int H, int E, int k, int I, int dtype, int algo, void* out, float* yw,
-                  hipStream_t s) {
+                  const int32_t* perm_slot, const void* residual, int T, int H, int E, int k, int I, int dtype, int algo,
+                  void* out, float* yw, hipStream_t s) {
   hipError_t e;
   if (algo == BIBO_ALGO_MFMA) {
     if (!aligned16(hidden) || !aligned16(wd)) return BIBO_ERR_MISALIGNED;
@@ -101,18 +101,18 @@ int down_dispatch(const void* hidden, const void* wd, const int32_t* idx, const 
     // expert output to bf16 as well, moe.py:92)
     e = launch_down_mfma(hidden, wd, w, offsets, perm_slot, T, H, E, k, I, yw, s);
     if (e != hipSuccess) return (int)e;
-    return hip_rc(launch_combine(yw, 1, idx, E, T, H, k, dtype, out, s));
+    return hip_rc(launch_combine(yw, 1, idx, E, residual, T, H, k, dtype, out, s));
   }
   e = launch_down_generic(hidden, wd, w, offsets, perm_slot, T, H, E, k, I, dtype, yw, s);
   if (e != hipSuccess) return (int)e;
-  return hip_rc(launch_combine(yw, 0, idx, E, T, H, k, dtype, out, s));
+  return hip_rc(launch_combine(yw, 0, idx, E, residual, T, H, k, dtype, out, s));
 }
 
 // kernels 3 and 4 (+ combine) after the permutation, for the composite entry points
 int experts_dispatch(const void* x, const void* wgu, const void* wd, const float* theta, const int32_t* idx,
-                     const float* w, const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token, int T,
-                     int H, int E,
-                     int k, int I, int dtype, int algo, void* out, char* base, const Workspace& ws, hipStream_t s) {
+                     const float* w, const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token,
+                     const void* residual, int T, int H, int E, int k, int I, int dtype, int algo, void* out, char* base,
+                     const Workspace& ws, hipStream_t s) {
   float* yw = reinterpret_cast<float*>(base + ws.yw);
   if (algo == BIBO_ALGO_STREAM) {
     if (!aligned16(x) || !aligned16(wgu) || !aligned16(wd)) return BIBO_ERR_MISALIGNED;
@@ -122,18 +122,58 @@ int experts_dispatch(const void* x, const void* wgu, const void* wd, const float
     if (e != hipSuccess) return (int)e;
     e = launch_down_stream(gu, wd, theta, w, idx, T, H, E, k, I, base + ws.hidden, yw, s);
     if (e != hipSuccess) return (int)e;
-    return hip_rc(launch_combine(yw, 0, idx, E, T, H, k, dtype, out, s));
+    return hip_rc(launch_combine(yw, 0, idx, E, residual, T, H, k, dtype, out, s));
   }
   if (algo == BIBO_ALGO_FUSED) {
     if (!aligned16(x) || !aligned16(wgu) || !aligned16(wd)) return BIBO_ERR_MISALIGNED;
     hipError_t e = launch_experts_fused(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, T, H, E, k, I, yw, s);
     if (e != hipSuccess) return (int)e;
-    return hip_rc(launch_combine(yw, 1, idx, E, T, H, k, dtype, out, s));
+    return hip_rc(launch_combine(yw, 1, idx, E, residual, T, H, k, dtype, out, s));
   }
   const int rc = gateup_dispatch(x, wgu, theta, offsets, perm_token, T, H, E, k, I, dtype, algo, base + ws.hidden, s);
   if (rc != BIBO_OK) return rc;
-  return down_dispatch(base + ws.hidden, wd, idx, w, offsets, perm_slot, T, H, E, k, I, dtype, algo, out, yw, s);
+  return down_dispatch(base + ws.hidden, wd, idx, w, offsets, perm_slot, residual, T, H, E, k, I, dtype, algo, out, yw, s);
 }
+
+// The whole layer on `x`; `residual` (or NULL) is added in the combine.  `extra` bytes at the end of the
+// workspace belong to the caller (the normalised activations of bibo_moe_ffn_forward).
+int forward_impl(const void* x, const void* w_router, const float* bias, const void* w_gate_up, const void* w_down,
+                 const float* theta, const bibo_moe_shape* sh, int norm_mode, int algo, const void* residual, void* out,
+                 int32_t* idx_out, float* w_out, int32_t* counts_out, float* logits_out, void* workspace,
+                 size_t workspace_bytes, void* stream) {
+  if (sh == nullptr) return BIBO_ERR_NULL_POINTER;
+  const int T = sh->T, H = sh->H, E = sh->E, k = sh->k, I = sh->I, dtype = sh->dtype;
+  int rc = check_dims(T, H, E, k, I, dtype);
+  if (rc != BIBO_OK) return rc;
+  if (norm_mode < BIBO_NORM_NONE || norm_mode > BIBO_NORM_SOFTMAX) return BIBO_ERR_UNSUPPORTED;
+  int a;
+  if ((rc = resolve_algo(algo, T, H, E, k, I, dtype, true, &a)) != BIBO_OK) return rc;
+  if (!workspace) return BIBO_ERR_NULL_POINTER;
+  if (T > 0 && (!x || !w_router || !bias || !w_gate_up || !w_down || !theta || !out)) return BIBO_ERR_NULL_POINTER;
+  const Workspace ws = carve(T, H, E, k, I, dtype);
+  if (workspace_bytes < ws.total) return BIBO_ERR_WORKSPACE_TOO_SMALL;
+  char* base = static_cast<char*>(workspace);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  int32_t* idx = idx_out ? idx_out : reinterpret_cast<int32_t*>(base + ws.idx);
+  float* w = w_out ? w_out : reinterpret_cast<float*>(base + ws.w);
+  int32_t* counts = counts_out ? counts_out : reinterpret_cast<int32_t*>(base + ws.counts);
+  int32_t* offsets = reinterpret_cast<int32_t*>(base + ws.offsets);
+  int32_t* perm_slot = reinterpret_cast<int32_t*>(base + ws.perm_slot);
+  int32_t* perm_token = reinterpret_cast<int32_t*>(base + ws.perm_token);
+  if (T > 0 &&
+      (rc = hip_rc(launch_router(x, w_router, bias, T, H, E, k, dtype, norm_mode, logits_out, idx, w, nullptr, s))) !=
+          BIBO_OK)
+    return rc;
+  // the streaming kernels find their rows themselves; the permutation then only serves the counts
+  const bool need_permute = a != BIBO_ALGO_STREAM || counts_out != nullptr || T == 0;
+  if (need_permute &&
+      (rc = hip_rc(launch_permute(idx, T, E, k, counts, offsets, perm_slot, perm_token, base + ws.hist, s))) != BIBO_OK)
+    return rc;
+  if (T == 0) return BIBO_OK;
+  return experts_dispatch(x, w_gate_up, w_down, theta, idx, w, offsets, perm_slot, perm_token, residual, T, H, E, k, I,
+                          dtype, a, out, base, ws, s);
+}
+
 
 }  // namespace
 
@@ -209,7 +249,7 @@ int bibo_moe_down_combine_fwd(const void* hidden, const void* w_down, const floa
   if (T == 0) return BIBO_OK;
   if (!hidden || !w_down || !w || !offsets || !perm_slot || !out || !workspace) return BIBO_ERR_NULL_POINTER;
   if (workspace_bytes < (size_t)T * k * H * sizeof(float)) return BIBO_ERR_WORKSPACE_TOO_SMALL;
-  return down_dispatch(hidden, w_down, nullptr, w, offsets, perm_slot, T, H, E, k, I, dtype, a, out,
+  return down_dispatch(hidden, w_down, nullptr, w, offsets, perm_slot, nullptr, T, H, E, k, I, dtype, a, out,
                        static_cast<float*>(workspace), static_cast<hipStream_t>(stream));
 }
 
@@ -234,7 +274,7 @@ int bibo_moe_combine_fwd(const void* yw, int yw_is_bf16, int T, int H, int k, in
   if (yw_is_bf16 && dtype != BIBO_DTYPE_BF16) return BIBO_ERR_BAD_DTYPE;
   if (T == 0) return BIBO_OK;
   if (!yw || !out) return BIBO_ERR_NULL_POINTER;
-  return hip_rc(launch_combine(yw, yw_is_bf16 ? 1 : 0, nullptr, 0, T, H, k, dtype, out, static_cast<hipStream_t>(stream)));
+  return hip_rc(launch_combine(yw, yw_is_bf16 ? 1 : 0, nullptr, 0, nullptr, T, H, k, dtype, out, static_cast<hipStream_t>(stream)));
 }
 
 int bibo_moe_experts_fwd(const void* x, const int32_t* idx, const float* w, const void* w_gate_up, const void* w_down,
@@ -262,45 +302,52 @@ int bibo_moe_experts_fwd(const void* x, const int32_t* idx, const float* w, cons
       (rc = hip_rc(launch_permute(idx, T, E, k, counts, offsets, perm_slot, perm_token, base + ws.hist, s))) != BIBO_OK)
     return rc;
   if (T == 0) return BIBO_OK;
-  return experts_dispatch(x, w_gate_up, w_down, theta, idx, w, offsets, perm_slot, perm_token, T, H, E, k, I, dtype, a, out,
-                          base, ws, s);
+  return experts_dispatch(x, w_gate_up, w_down, theta, idx, w, offsets, perm_slot, perm_token, nullptr, T, H, E, k, I,
+                          dtype, a, out, base, ws, s);
 }
 
 int bibo_moe_forward(const void* x, const void* w_router, const float* bias, const void* w_gate_up, const void* w_down,
                      const float* theta, const bibo_moe_shape* sh, int norm_mode, int algo, void* out, int32_t* idx_out,
                      float* w_out, int32_t* counts_out, float* logits_out, void* workspace, size_t workspace_bytes,
                      void* stream) {
-  if (sh == nullptr) return BIBO_ERR_NULL_POINTER;
-  const int T = sh->T, H = sh->H, E = sh->E, k = sh->k, I = sh->I, dtype = sh->dtype;
-  int rc = check_dims(T, H, E, k, I, dtype);
+  return forward_impl(x, w_router, bias, w_gate_up, w_down, theta, sh, norm_mode, algo, nullptr, out, idx_out, w_out,
+                      counts_out, logits_out, workspace, workspace_bytes, stream);
+}
+
+int bibo_moe_rmsnorm_fwd(const void* x, const float* norm_weight, float eps, int T, int H, int dtype, void* out,
+                         void* stream) {
+  const int rc = check_dims(T, H, 1, 1, 1, dtype);
   if (rc != BIBO_OK) return rc;
-  if (norm_mode < BIBO_NORM_NONE || norm_mode > BIBO_NORM_SOFTMAX) return BIBO_ERR_UNSUPPORTED;
-  int a;
-  if ((rc = resolve_algo(algo, T, H, E, k, I, dtype, true, &a)) != BIBO_OK) return rc;
-  if (!workspace) return BIBO_ERR_NULL_POINTER;
-  if (T > 0 && (!x || !w_router || !bias || !w_gate_up || !w_down || !theta || !out)) return BIBO_ERR_NULL_POINTER;
-  const Workspace ws = carve(T, H, E, k, I, dtype);
-  if (workspace_bytes < ws.total) return BIBO_ERR_WORKSPACE_TOO_SMALL;
-  char* base = static_cast<char*>(workspace);
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  int32_t* idx = idx_out ? idx_out : reinterpret_cast<int32_t*>(base + ws.idx);
-  float* w = w_out ? w_out : reinterpret_cast<float*>(base + ws.w);
-  int32_t* counts = counts_out ? counts_out : reinterpret_cast<int32_t*>(base + ws.counts);
-  int32_t* offsets = reinterpret_cast<int32_t*>(base + ws.offsets);
-  int32_t* perm_slot = reinterpret_cast<int32_t*>(base + ws.perm_slot);
-  int32_t* perm_token = reinterpret_cast<int32_t*>(base + ws.perm_token);
-  if (T > 0 &&
-      (rc = hip_rc(launch_router(x, w_router, bias, T, H, E, k, dtype, norm_mode, logits_out, idx, w, nullptr, s))) !=
-          BIBO_OK)
-    return rc;
-  // the streaming kernels find their rows themselves; the permutation then only serves the counts
-  const bool need_permute = a != BIBO_ALGO_STREAM || counts_out != nullptr || T == 0;
-  if (need_permute &&
-      (rc = hip_rc(launch_permute(idx, T, E, k, counts, offsets, perm_slot, perm_token, base + ws.hist, s))) != BIBO_OK)
-    return rc;
   if (T == 0) return BIBO_OK;
-  return experts_dispatch(x, w_gate_up, w_down, theta, idx, w, offsets, perm_slot, perm_token, T, H, E, k, I, dtype, a, out,
-                          base, ws, s);
+  if (!x || !norm_weight || !out) return BIBO_ERR_NULL_POINTER;
+  return hip_rc(launch_rmsnorm(x, norm_weight, eps, T, H, dtype, out, static_cast<hipStream_t>(stream)));
+}
+
+int bibo_moe_ffn_workspace_bytes(const bibo_moe_shape* sh, size_t* out) {
+  if (sh == nullptr || out == nullptr) return BIBO_ERR_NULL_POINTER;
+  const int rc = check_dims(sh->T, sh->H, sh->E, sh->k, sh->I, sh->dtype);
+  if (rc != BIBO_OK) return rc;
+  *out = carve(sh->T, sh->H, sh->E, sh->k, sh->I, sh->dtype).total + align_up((size_t)sh->T * sh->H * elt_size(sh->dtype));
+  return BIBO_OK;
+}
+
+int bibo_moe_ffn_forward(const void* h, const float* norm_weight, float eps, const void* w_router, const float* bias,
+                         const void* w_gate_up, const void* w_down, const float* theta, const bibo_moe_shape* sh,
+                         int norm_mode, int algo, void* out, int32_t* idx_out, float* w_out, int32_t* counts_out,
+                         void* workspace, size_t workspace_bytes, void* stream) {
+  if (sh == nullptr) return BIBO_ERR_NULL_POINTER;
+  const int rc = check_dims(sh->T, sh->H, sh->E, sh->k, sh->I, sh->dtype);
+  if (rc != BIBO_OK) return rc;
+  if (!workspace) return BIBO_ERR_NULL_POINTER;
+  if (sh->T > 0 && (!h || !norm_weight || !out)) return BIBO_ERR_NULL_POINTER;
+  const size_t inner = carve(sh->T, sh->H, sh->E, sh->k, sh->I, sh->dtype).total;
+  const size_t xn_bytes = align_up((size_t)sh->T * sh->H * elt_size(sh->dtype));
+  if (workspace_bytes < inner + xn_bytes) return BIBO_ERR_WORKSPACE_TOO_SMALL;
+  void* xn = static_cast<char*>(workspace) + inner;              // post_attention_layernorm(h), layers.py:60
+  const hipError_t e = launch_rmsnorm(h, norm_weight, eps, sh->T, sh->H, sh->dtype, xn, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return (int)e;
+  return forward_impl(xn, w_router, bias, w_gate_up, w_down, theta, sh, norm_mode, algo, h, out, idx_out, w_out,
+                      counts_out, nullptr, workspace, inner, stream);
 }
 
 }  // extern "C"

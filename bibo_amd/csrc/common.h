@@ -119,8 +119,10 @@ hipError_t launch_gateup_generic(const void* x, const void* wgu, const float* th
 hipError_t launch_down_generic(const void* hidden, const void* wd, const float* w, const int32_t* offsets,
                                const int32_t* perm_slot, int T, int H, int E, int k, int I, int dtype, float* yw,
                                hipStream_t s);
-hipError_t launch_combine(const void* yw, int yw_is_bf16, const int32_t* idx, int E, int T, int H, int k, int dtype,
-                          void* out, hipStream_t s);
+hipError_t launch_combine(const void* yw, int yw_is_bf16, const int32_t* idx, int E, const void* residual, int T, int H,
+                          int k, int dtype, void* out, hipStream_t s);
+hipError_t launch_rmsnorm(const void* x, const float* weight, float eps, int T, int H, int dtype, void* out,
+                          hipStream_t s);
 bool mfma_supported(int H, int I, int dtype);
 hipError_t launch_gateup_mfma(const void* x, const void* wgu, const float* theta, const int32_t* offsets,
                               const int32_t* perm_token, int T, int H, int E, int k, int I, void* hidden, hipStream_t s);

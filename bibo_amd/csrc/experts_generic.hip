@@ -87,11 +87,13 @@ __global__ __launch_bounds__(256) void down_generic_kernel(const TIn* __restrict
   }
 }
 
-// out[t, :] = round(sum_j yw[t*k + j, :])  in fp32, ascending j   (moe.py:93,101).  With `idx` given, slots
-// whose expert index is outside [0,E) are skipped (no kernel wrote their row).
+// out[t, :] = round(residual[t, :] + sum_j yw[t*k + j, :])  in fp32, ascending j   (moe.py:93,101; the residual
+// add of the caller, src/modeling/layers.py:62, when `residual` is given).  With `idx` given, slots whose
+// expert index is outside [0,E) are skipped (no kernel wrote their row).
 template <typename TY, typename TOut>
 __global__ __launch_bounds__(256) void combine_kernel(const TY* __restrict__ yw, const int32_t* __restrict__ idx, int E,
-                                                      int T, int H, int k, TOut* __restrict__ out) {
+                                                      const TOut* __restrict__ residual, int T, int H, int k,
+                                                      TOut* __restrict__ out) {
   const size_t n = (size_t)T * H;
   for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
     const size_t t = i / H, h = i - t * H;
@@ -100,14 +102,16 @@ __global__ __launch_bounds__(256) void combine_kernel(const TY* __restrict__ yw,
       if (idx != nullptr && (unsigned)idx[t * k + j] >= (unsigned)E) continue;
       acc += to_float(yw[(t * k + j) * H + h]);
     }
+    if (residual != nullptr) acc += to_float(residual[i]);
     out[i] = from_float<TOut>(acc);
   }
 }
 
 // bf16 slot rows -> bf16 output, 8 columns (16 bytes) per thread, fp32 sum in ascending j   (moe.py:93,101)
 __global__ __launch_bounds__(256) void combine_bf16x8_kernel(const bf16_t* __restrict__ yw,
-                                                             const int32_t* __restrict__ idx, int E, int T, int H8,
-                                                             int k, bf16_t* __restrict__ out) {
+                                                             const int32_t* __restrict__ idx, int E,
+                                                             const bf16_t* __restrict__ residual, int T, int H8, int k,
+                                                             bf16_t* __restrict__ out) {
   const size_t n = (size_t)T * H8;
   for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
     const size_t t = i / H8, c = i - t * H8;
@@ -120,6 +124,11 @@ __global__ __launch_bounds__(256) void combine_bf16x8_kernel(const bf16_t* __res
       const bf16x8 v = src[(size_t)j * H8];
 #pragma unroll
       for (int q = 0; q < 8; ++q) acc[q] += (float)v[q];
+    }
+    if (residual != nullptr) {
+      const bf16x8 r = reinterpret_cast<const bf16x8*>(residual)[i];
+#pragma unroll
+      for (int q = 0; q < 8; ++q) acc[q] += (float)r[q];
     }
     bf16x8 o;
 #pragma unroll
@@ -162,27 +171,29 @@ hipError_t launch_down_generic(const void* hidden, const void* wd, const float* 
   return hipGetLastError();
 }
 
-hipError_t launch_combine(const void* yw, int yw_is_bf16, const int32_t* idx, int E, int T, int H, int k, int dtype,
-                          void* out, hipStream_t s) {
+hipError_t launch_combine(const void* yw, int yw_is_bf16, const int32_t* idx, int E, const void* residual, int T, int H,
+                          int k, int dtype, void* out, hipStream_t s) {
   const size_t n = (size_t)T * H;
   if (n == 0) return hipSuccess;
   const int grid = (int)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
   if (yw_is_bf16) {
     if (dtype != BIBO_DTYPE_BF16) return hipErrorInvalidValue;
-    if ((H % 8) == 0 && ((reinterpret_cast<uintptr_t>(yw) | reinterpret_cast<uintptr_t>(out)) & 15) == 0) {
+    if ((H % 8) == 0 && ((reinterpret_cast<uintptr_t>(yw) | reinterpret_cast<uintptr_t>(out) |
+                          reinterpret_cast<uintptr_t>(residual)) & 15) == 0) {
       const size_t n8 = n / 8;
       const int g8 = (int)((n8 + 255) / 256 < 65536 ? (n8 + 255) / 256 : 65536);
-      hipLaunchKernelGGL(combine_bf16x8_kernel, dim3(g8), dim3(256), 0, s, static_cast<const bf16_t*>(yw), idx, E, T, H / 8, k,
+      hipLaunchKernelGGL(combine_bf16x8_kernel, dim3(g8), dim3(256), 0, s, static_cast<const bf16_t*>(yw), idx, E, static_cast<const bf16_t*>(residual), T, H / 8, k,
                          static_cast<bf16_t*>(out));
     } else
       hipLaunchKernelGGL((combine_kernel<bf16_t, bf16_t>), dim3(grid), dim3(256), 0, s,
-                         static_cast<const bf16_t*>(yw), idx, E, T, H, k, static_cast<bf16_t*>(out));
+                         static_cast<const bf16_t*>(yw), idx, E, static_cast<const bf16_t*>(residual), T, H, k,
+                         static_cast<bf16_t*>(out));
   } else if (dtype == BIBO_DTYPE_BF16) {
     hipLaunchKernelGGL((combine_kernel<float, bf16_t>), dim3(grid), dim3(256), 0, s, static_cast<const float*>(yw), idx,
-                       E, T, H, k, static_cast<bf16_t*>(out));
+                       E, static_cast<const bf16_t*>(residual), T, H, k, static_cast<bf16_t*>(out));
   } else {
     hipLaunchKernelGGL((combine_kernel<float, float>), dim3(grid), dim3(256), 0, s, static_cast<const float*>(yw), idx,
-                       E, T, H, k, static_cast<float*>(out));
+                       E, static_cast<const float*>(residual), T, H, k, static_cast<float*>(out));
   }
   return hipGetLastError();
 }

@@ -51,7 +51,7 @@ def _compute_dtype(x: torch.Tensor) -> torch.dtype:
     if x.dtype == torch.bfloat16:
         return torch.bfloat16
     if x.dtype == torch.float32:
-        if torch.is_autocast_enabled() and torch.get_autocast_gpu_dtype() == torch.bfloat16:
+        if torch.is_autocast_enabled() and torch.get_autocast_dtype("cuda") == torch.bfloat16:
             return torch.bfloat16
         return torch.float32
     raise TypeError(f"hidden states must be bfloat16 or float32, got {x.dtype}")
@@ -236,3 +236,40 @@ class BiBoMoELayer(nn.Module):
             if tpe is not None:
                 self.update_bias(tpe)
         return out.view(bsz, seq, hdim)
+
+    @_no_compile
+    def ffn_forward(self, hidden_states: torch.Tensor, norm_weight: torch.Tensor, eps: float,
+                    bf16_stream: bool = False) -> torch.Tensor:
+        """The caller's seam, BiBoDecoderLayer._ffn_forward (src/modeling/layers.py:57-67):
+        `hidden_states + self(rmsnorm(hidden_states))` with `norm_weight`/`eps` of post_attention_layernorm
+        (src/modeling/norm.py:19-24), as ONE library call: the norm feeds the block from the workspace and the
+        residual is added in the combine kernel.  With hooks or a gap probe present, or with an fp32 stream
+        under bf16 autocast, the block runs as in forward and norm and residual are ordinary tensor operations
+        around it."""
+        bsz, seq, hdim = hidden_states.shape
+        num_tokens = bsz * seq
+        if self._hooks_present() or hidden_states.dtype != _compute_dtype(hidden_states):
+            # (an fp32 residual stream under bf16 autocast keeps its fp32 norm and fp32 residual add)
+            xf = hidden_states.float()
+            xn = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)).to(hidden_states.dtype)    # norm.py:21-24
+            out = hidden_states + self.forward(norm_weight * xn).to(hidden_states.dtype)               # layers.py:60-64
+            return out.to(torch.bfloat16) if bf16_stream else out
+        balancing = self.training and self.bias_update_factor > 0
+        _forward_only_guard(hidden_states, self.gate.gate_proj.weight, self.experts.gate_up_proj)
+        cd = _compute_dtype(hidden_states)
+        h = hidden_states.detach().reshape(num_tokens, hdim)
+        h = (h.to(cd) if h.dtype != cd else h).contiguous()
+        gu, dn, th = self.experts._weights(cd)
+        wr = self.gate._cache.get("w", self.gate.gate_proj.weight, cd)
+        b = self.gate._cache.get("b", self.gate.bias, torch.float32)
+        nw = norm_weight.detach().float().contiguous()
+        out, _, _, counts = ops.ffn_forward(h, nw, float(eps), wr, b, gu, dn, th, self.num_experts_per_tok,
+                                            norm=self.gate.norm_topk_prob, algo=self.experts.algo, want_counts=balancing)
+        if balancing:                                          # exactly once per training forward
+            tpe = self._balance_step(None, num_tokens, counts=counts)
+            if tpe is not None:
+                self.update_bias(tpe)
+        out = out.view(bsz, seq, hdim)
+        out = out if out.dtype == hidden_states.dtype else out.to(hidden_states.dtype)
+        return out.to(torch.bfloat16) if bf16_stream else out
+

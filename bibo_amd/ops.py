@@ -221,3 +221,41 @@ def moe_forward(x, w_router, bias, w_gate_up, w_down, theta, k, norm="sum", algo
                                          _ptr(idx), _ptr(w), _ptr(counts), _ptr(logits), _ptr(ws), ws.numel(),
                                          _stream(dev)), "bibo_moe_forward")
     return out, idx, w, counts, logits
+
+
+def rmsnorm_fwd(x, norm_weight, eps):
+    """out = norm_weight * round(x * rsqrt(mean(x^2) + eps)) in x.dtype (the block's input norm, norm.py:19-24)."""
+    T, H = x.shape
+    _chk(x, "x"); _chk(norm_weight, "norm_weight", torch.float32, (H,))
+    out = torch.empty_like(x)
+    with torch.cuda.device(x.device):
+        L.check(L.lib().bibo_moe_rmsnorm_fwd(_ptr(x), _ptr(norm_weight), ctypes.c_float(eps), T, H, _dtype_code(x),
+                                             _ptr(out), _stream(x.device)), "bibo_moe_rmsnorm_fwd")
+    return out
+
+
+def ffn_forward(h, norm_weight, eps, w_router, bias, w_gate_up, w_down, theta, k, norm="sum", algo="auto",
+                want_routing=False, want_counts=False):
+    """Seam 3 (the block's caller).  -> out = h + moe(rmsnorm(h)) [T,H], idx|None, w|None, counts|None."""
+    T, H = h.shape
+    E, two_i, _ = w_gate_up.shape
+    I = two_i // 2
+    dc = _dtype_code(h)
+    _chk(h, "h"); _chk(norm_weight, "norm_weight", torch.float32, (H,)); _chk(w_router, "w_router", h.dtype, (E, H))
+    _chk(bias, "bias", torch.float32, (E,)); _chk(w_gate_up, "w_gate_up", h.dtype, (E, 2 * I, H))
+    _chk(w_down, "w_down", h.dtype, (E, H, I)); _chk(theta, "theta", torch.float32, (E,))
+    dev = h.device
+    out = torch.empty(T, H, dtype=h.dtype, device=dev)
+    idx = torch.empty(T, k, dtype=torch.int32, device=dev) if want_routing else None
+    w = torch.empty(T, k, dtype=torch.float32, device=dev) if want_routing else None
+    counts = torch.empty(E, dtype=torch.int32, device=dev) if want_counts else None
+    sh = L.Shape(T, H, E, k, I, dc)
+    nbytes = ctypes.c_size_t(0)
+    L.check(L.lib().bibo_moe_ffn_workspace_bytes(ctypes.byref(sh), ctypes.byref(nbytes)), "bibo_moe_ffn_workspace_bytes")
+    ws = workspace(dev, nbytes.value)
+    with torch.cuda.device(dev):
+        L.check(L.lib().bibo_moe_ffn_forward(_ptr(h), _ptr(norm_weight), ctypes.c_float(eps), _ptr(w_router), _ptr(bias),
+                                             _ptr(w_gate_up), _ptr(w_down), _ptr(theta), ctypes.byref(sh),
+                                             norm_mode(norm), algo_code(algo), _ptr(out), _ptr(idx), _ptr(w),
+                                             _ptr(counts), _ptr(ws), ws.numel(), _stream(dev)), "bibo_moe_ffn_forward")
+    return out, idx, w, counts

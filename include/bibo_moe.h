@@ -169,6 +169,21 @@ int bibo_moe_forward(const void* x, const void* w_router, const float* bias, con
                      void* out, int32_t* idx_out, float* w_out, int32_t* counts_out, float* logits_out,
                      void* workspace, size_t workspace_bytes, void* stream);
 
+/*
+ * Seam 3: the caller of the block, BiBoDecoderLayer._ffn_forward (src/modeling/layers.py:57-67):
+ *   out = h + moe(post_attention_layernorm(h)),  RMSNorm as BiBoRMSNorm.forward (src/modeling/norm.py:19-24)
+ * with norm_weight fp32 [H].  The normalised activations live in the workspace; the residual add happens in
+ * the combine, in fp32, before the single rounding to `dtype` (the reference rounds the block output first).
+ * h, out [T,H] in `dtype` (out may not alias h).  Workspace size: bibo_moe_ffn_workspace_bytes.
+ */
+int bibo_moe_rmsnorm_fwd(const void* x, const float* norm_weight, float eps, int T, int H, int dtype, void* out,
+                         void* stream);                 /* the norm alone: out = weight * round(x * rsqrt(mean x^2 + eps)) */
+int bibo_moe_ffn_workspace_bytes(const bibo_moe_shape* shape, size_t* out_bytes);
+int bibo_moe_ffn_forward(const void* h, const float* norm_weight, float eps, const void* w_router, const float* bias,
+                         const void* w_gate_up, const void* w_down, const float* theta, const bibo_moe_shape* shape,
+                         int norm_mode, int algo, void* out, int32_t* idx_out, float* w_out, int32_t* counts_out,
+                         void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

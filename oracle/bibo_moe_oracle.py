@@ -198,6 +198,28 @@ def moe_forward(x, w_router, bias, w_gate_up, w_down, theta, k, dtype=torch.floa
 
 
 # --------------------------------------------------------------------------------------
+# the caller of the block: RMSNorm in front, residual behind  (src/modeling/layers.py:57-67)
+# --------------------------------------------------------------------------------------
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """BiBoRMSNorm.forward (src/modeling/norm.py:19-24): statistics in fp32, the normalised row rounded to
+    the input dtype, then multiplied by the weight; returned in the input dtype."""
+    xf = x.float()
+    var = xf.pow(2).mean(-1, keepdim=True)                                    # norm.py:22
+    xn = (xf * torch.rsqrt(var + eps)).to(x.dtype)                            # norm.py:23-24
+    return (weight.float() * xn.float()).to(x.dtype)
+
+
+def ffn_forward(h, norm_weight, eps, w_router, bias, w_gate_up, w_down, theta, k, logits=None):
+    """BiBoDecoderLayer._ffn_forward (layers.py:57-67): h + moe(post_attention_layernorm(h)), the block and the
+    sum evaluated in fp32.  Returns (out fp32, xn in h's dtype, idx, w)."""
+    xn = rmsnorm(h, norm_weight, eps)                                         # layers.py:60
+    if logits is None:
+        logits = router_logits(xn, w_router)
+    y, idx, w = moe_forward(xn, w_router, bias, w_gate_up, w_down, theta, k, logits=logits)   # layers.py:61
+    return h.float() + y.float(), xn, idx, w                                  # layers.py:64
+
+
+# --------------------------------------------------------------------------------------
 # the reference's eager CPU path, for timing (moe.py:46-101 + router.py:28-51 as written)
 # --------------------------------------------------------------------------------------
 @torch.no_grad()

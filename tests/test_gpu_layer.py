@@ -6,6 +6,7 @@ import torch
 
 import bibo_amd
 from oracle import bibo_moe_oracle as O
+from bibo_amd import ops
 from conftest import rel_err
 
 pytestmark = pytest.mark.gpu
@@ -175,3 +176,73 @@ def test_fused_forward_routing_equals_standalone_router(T):
     assert np.array_equal(counts.cpu().numpy(), O.permute(oi, 64)[0])
     ref = O.experts_forward(p["x"], oi, ow, p["w_gate_up"], p["w_down"], p["theta"])
     assert rel_err(out.cpu(), ref) <= 2e-2
+
+
+# ------------------------------------------------------------------ the caller's seam: RMSNorm in front, residual behind
+@pytest.mark.parametrize("T,H,I,algo", [(64, 1024, 512, "auto"), (700, 768, 384, "auto"), (300, 256, 128, "generic"),
+                                        (300, 200, 72, "auto")])
+def test_ffn_forward_matches_oracle(T, H, I, algo):
+    """bibo_moe_ffn_forward = h + moe(rmsnorm(h)) (layers.py:57-67): routing bit-exact on the kernel's own
+    normalised input, output within the bf16 tolerance of the fp32 oracle."""
+    p = O.make_inputs(T=T, H=H, E=64, k=6, I=I, bias="uniform", theta="normal", seed=T + H)
+    g = torch.Generator().manual_seed(T)
+    nw = torch.rand(H, generator=g) + 0.5
+    h = (p["x"].float() * 3).bfloat16()
+    dev = torch.device("cuda:0")
+    out, idx, w, counts = ops.ffn_forward(h.to(dev), nw.to(dev), 1e-6, p["w_router"].to(dev), p["bias"].to(dev),
+                                          p["w_gate_up"].to(dev), p["w_down"].to(dev), p["theta"].to(dev), 6, algo=algo,
+                                          want_routing=True, want_counts=True)
+    # the norm kernel against the oracle: equal up to one bf16 step where the fp32 statistics round differently
+    xn_k = ops.rmsnorm_fwd(h.to(dev), nw.to(dev), 1e-6)
+    torch.cuda.synchronize()
+    xn = O.rmsnorm(h, nw, 1e-6)
+    d = (xn_k.cpu().float() - xn.float()).abs()
+    assert (d <= xn.float().abs() * 2.0 ** -7 + 1e-30).all() and (d > 0).float().mean() < 0.01
+    # the parity protocol on the kernel's own normalised rows: routing from the router kernel's logits on them
+    _, _, logits, _ = ops.router_fwd(xn_k, p["w_router"].to(dev), p["bias"].to(dev), 6, want_logits=True)
+    y, oi, ow = O.moe_forward(xn_k.cpu(), p["w_router"], p["bias"], p["w_gate_up"], p["w_down"], p["theta"], 6,
+                              logits=logits.cpu().numpy())
+    ref = h.float() + y.float()
+    assert np.array_equal(idx.cpu().numpy(), oi) and np.array_equal(w.cpu().numpy(), ow)
+    assert np.array_equal(counts.cpu().numpy(), np.bincount(oi.reshape(-1), minlength=64))
+    assert rel_err(out.cpu(), ref) <= 2e-2
+
+
+def test_ffn_forward_fp32_isolates_the_block_contribution():
+    """In fp32 the sum is not rounded to bf16, so out - h must be the block's output itself (in the bf16 case
+    above it is mostly below the resolution of the residual)."""
+    p = O.make_inputs(T=90, H=96, E=16, k=3, I=40, bias="uniform", theta="normal", seed=8, dtype=torch.float32)
+    nw = torch.rand(96, generator=torch.Generator().manual_seed(1)) + 0.5
+    h = p["x"] * 2
+    dev = torch.device("cuda:0")
+    out, idx, w, _ = ops.ffn_forward(h.to(dev), nw.to(dev), 1e-6, p["w_router"].to(dev), p["bias"].to(dev),
+                                     p["w_gate_up"].to(dev), p["w_down"].to(dev), p["theta"].to(dev), 3, want_routing=True)
+    xn_k = ops.rmsnorm_fwd(h.to(dev), nw.to(dev), 1e-6)
+    torch.cuda.synchronize()
+    assert torch.allclose(xn_k.cpu(), O.rmsnorm(h, nw, 1e-6), rtol=1e-5, atol=1e-6)
+    y = O.experts_forward(xn_k.cpu(), idx.cpu().numpy(), w.cpu().numpy(), p["w_gate_up"], p["w_down"], p["theta"])
+    assert rel_err(out.cpu() - h, y) <= 1e-4
+
+
+def test_layer_ffn_forward_equals_norm_block_residual_composition():
+    torch.manual_seed(3)
+    cfg = make_config(hidden_size=256, moe_intermediate_size=128, num_routed_experts=64, num_experts_per_tok=6)
+    layer = bibo_amd.BiBoMoELayer(cfg).to("cuda:0").bfloat16().eval()
+    with torch.no_grad():
+        layer.experts.radial_theta.normal_(0, 0.5)
+    h = (torch.randn(2, 100, 256, device="cuda:0") * 2).bfloat16()
+    nw = (torch.rand(256, device="cuda:0") + 0.5).bfloat16()
+    with torch.no_grad():
+        fused = layer.ffn_forward(h, nw, 1e-6)
+        hf = h.float()
+        xn = (hf * torch.rsqrt(hf.pow(2).mean(-1, keepdim=True) + 1e-6)).bfloat16()
+        composed = h + layer(nw * xn)                              # layers.py:59-64 with stock ops around the block
+    assert fused.dtype == torch.bfloat16 and fused.shape == h.shape
+    assert rel_err(fused.cpu(), composed.cpu().float()) <= 1e-2     # one rounding less on the fused side
+    # an fp32 stream under bf16 autocast keeps its fp32 residual
+    layer32 = bibo_amd.BiBoMoELayer(cfg).to("cuda:0").eval()
+    h32 = torch.randn(1, 50, 256, device="cuda:0")
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        o32 = layer32.ffn_forward(h32, torch.ones(256, device="cuda:0"), 1e-6)
+    assert o32.dtype == torch.float32
+    assert (o32 - h32).abs().max() < 1.0 and torch.isfinite(o32).all()

@@ -50,6 +50,16 @@ def test_argument_errors_are_reported_without_a_gpu():
     # the streaming kernels exist only behind the composite entry points
     assert lib.bibo_moe_gateup_fwd(None, None, None, None, None, 4, 1024, 64, 6, 512, 0, L.ALGO_STREAM, None, None) == -6
     assert lib.bibo_moe_permute(None, 4, 8, 2, None, None, None, None, None, 0, None) == -1
+    # fused-kernel and caller-seam entry points
+    assert lib.bibo_moe_gateup_down_fwd(None, None, None, None, None, None, None, None, 4, 768, 64, 6, 512, 0, None, None) == -6
+    assert lib.bibo_moe_gateup_down_fwd(None, None, None, None, None, None, None, None, 4, 768, 64, 6, 384, 0, None, None) == -1
+    assert lib.bibo_moe_combine_fwd(None, 1, 4, 64, 2, L.DTYPE_F32, None, None) == -3      # bf16 slot rows need a bf16 output
+    assert lib.bibo_moe_rmsnorm_fwd(None, None, ctypes.c_float(1e-6), 4, 64, 0, None, None) == -1
+    ffn = ctypes.c_size_t(0)
+    assert lib.bibo_moe_ffn_workspace_bytes(ctypes.byref(ok), ctypes.byref(ffn)) == 0
+    assert ffn.value >= out.value + 8192 * 768 * 2                 # the block's workspace plus the normalised activations
+    assert lib.bibo_moe_ffn_forward(None, None, ctypes.c_float(1e-6), None, None, None, None, None, ctypes.byref(ok), 1, 0,
+                                    None, None, None, None, None, 0, None) == -1
     assert b"workspace" in lib.bibo_moe_strerror(-4)
     with pytest.raises(RuntimeError, match="workspace"):
         L.check(-4, "x")

@@ -244,3 +244,48 @@ def test_workload_table_matches_the_named_shapes():
     p = O.make_inputs(**{**c["c4"], "T": 32})
     assert (p["bias"][:4] == 2.0).all() and p["bias"][4:].abs().max() <= 0.01
     assert p["x"].dtype == torch.bfloat16 and p["bias"].dtype == torch.float32
+
+
+# ------------------------------------------------------------------ caller seam: RMSNorm + residual
+def test_rmsnorm_matches_library_routine_and_closed_form():
+    """norm.py:19-24.  Pins: torch.nn.functional.rms_norm (an independent library routine) in fp32; a scalar
+    pure-Python evaluation; scale invariance rmsnorm(a*x) == rmsnorm(x) when eps is negligible; a row of
+    equal magnitudes maps to sign(x) * weight."""
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(5, 48, generator=g) * 3
+    wgt = torch.rand(48, generator=g) + 0.5
+    got = O.rmsnorm(x, wgt, 1e-6)
+    lib = torch.nn.functional.rms_norm(x, (48,), wgt, 1e-6)
+    assert torch.allclose(got, lib, rtol=1e-6, atol=1e-6)
+    r = 2
+    ms = sum(float(v) ** 2 for v in x[r]) / 48
+    want = [float(wgt[c]) * float(x[r, c]) / math.sqrt(ms + 1e-6) for c in range(48)]
+    assert np.allclose(got[r].numpy(), want, rtol=1e-5, atol=1e-6)
+    assert torch.allclose(O.rmsnorm(7.0 * x, wgt, 1e-12), O.rmsnorm(x, wgt, 1e-12), rtol=1e-5, atol=1e-6)
+    s = torch.tensor([[2.0, -2.0, 2.0, -2.0]])
+    assert torch.allclose(O.rmsnorm(s, torch.tensor([1.0, 2.0, 3.0, 4.0]), 0.0), torch.tensor([[1.0, -2.0, 3.0, -4.0]]))
+
+
+def test_rmsnorm_rounds_the_normalised_row_before_the_weight_in_bf16():
+    """norm.py:24 multiplies the weight with the row ALREADY cast back to the input dtype."""
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(3, 64, generator=g).bfloat16()
+    wgt = (torch.rand(64, generator=g) + 0.5)
+    xf = x.float()
+    xn = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-6)).bfloat16()
+    assert torch.equal(O.rmsnorm(x, wgt, 1e-6), (wgt * xn.float()).bfloat16())
+    assert O.rmsnorm(x, wgt, 1e-6).dtype == torch.bfloat16
+
+
+def test_ffn_forward_is_residual_plus_block_of_the_normalised_input():
+    p = O.make_inputs(T=24, H=32, E=8, k=2, I=16, bias="uniform", theta="normal", seed=12, dtype=torch.float32)
+    g = torch.Generator().manual_seed(6)
+    wgt = torch.rand(32, generator=g) + 0.5
+    out, xn, idx, w = O.ffn_forward(p["x"], wgt, 1e-6, p["w_router"], p["bias"], p["w_gate_up"], p["w_down"], p["theta"], 2)
+    y, idx2, w2 = O.moe_forward(xn, p["w_router"], p["bias"], p["w_gate_up"], p["w_down"], p["theta"], 2)
+    assert np.array_equal(idx, idx2) and np.array_equal(w, w2)
+    assert torch.allclose(out, p["x"] + y, rtol=0, atol=0)
+    # a zero block (w_down = 0) leaves the residual untouched
+    out0, *_ = O.ffn_forward(p["x"], wgt, 1e-6, p["w_router"], p["bias"], p["w_gate_up"], torch.zeros_like(p["w_down"]),
+                             p["theta"], 2)
+    assert torch.equal(out0, p["x"])
