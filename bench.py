@@ -22,9 +22,9 @@ PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
 
 # HBM-side bytes per launch of the dominant expert kernel on workload c2, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE (KiB per dispatch), scaled by what the same counters read for a 256 MiB device copy
-# (FETCH_SIZE x2.0, WRITE_SIZE x1.0).  Fused kernel: 208.0 MB fetched + 75.5 MB written; gate/up kernel of the
-# two-kernel family: 158.9 MB + 37.7 MB.
-MEASURED_TRAFFIC_BYTES = {("c2", "gateup_down"): 283.5e6, ("c2", "gateup"): 196.6e6}
+# (FETCH_SIZE x2.0, WRITE_SIZE x1.0).  Fused kernel: 208.0 MB fetched + 76.4 MB written; gate/up kernel of the
+# two-kernel family: 158.4 MB + 37.7 MB.
+MEASURED_TRAFFIC_BYTES = {("c2", "gateup_down"): 284.4e6, ("c2", "gateup"): 196.1e6}
 
 
 def flops_layer(T, H, E, k, I):
