@@ -64,7 +64,8 @@ Workspace carve(int T, int H, int E, int k, int I, int dtype) {
   const size_t S = (size_t)T * k;
   Workspace ws;
   size_t o = 0;
-  ws.hist = o;       o += align_up(permute_workspace_bytes(T));
+  ws.hist = o;       o += align_up(permute_workspace_bytes(T) > router_hist_bytes(T) ? permute_workspace_bytes(T)
+                                                                                    : router_hist_bytes(T));
   ws.idx = o;        o += align_up(S * sizeof(int32_t));
   ws.w = o;          o += align_up(S * sizeof(float));
   ws.counts = o;     o += align_up(kMaxE * sizeof(int32_t));
@@ -111,9 +112,12 @@ int down_dispatch(const void* hidden, const void* wd, const int32_t* idx, const 
 // kernels 3 and 4 (+ combine) after the permutation, for the composite entry points
 int experts_dispatch(const void* x, const void* wgu, const void* wd, const float* theta, const int32_t* idx,
                      const float* w, const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token,
-                     const void* residual, int T, int H, int E, int k, int I, int dtype, int algo, void* out, char* base,
-                     const Workspace& ws, hipStream_t s) {
+                     const void* residual, bool idx_trusted, int T, int H, int E, int k, int I, int dtype, int algo,
+                     void* out, char* base, const Workspace& ws, hipStream_t s) {
   float* yw = reinterpret_cast<float*>(base + ws.yw);
+  // indices that come straight from the router kernel are in range; a caller's may hold padding values,
+  // whose slots the combine then has to skip
+  const int32_t* cidx = idx_trusted ? nullptr : idx;
   if (algo == BIBO_ALGO_STREAM) {
     if (!aligned16(x) || !aligned16(wgu) || !aligned16(wd)) return BIBO_ERR_MISALIGNED;
     if (!stream_eligible(T, H, E, k, I, dtype)) return BIBO_ERR_UNSUPPORTED;     // no pre-activation segment carved
@@ -122,21 +126,20 @@ int experts_dispatch(const void* x, const void* wgu, const void* wd, const float
     if (e != hipSuccess) return (int)e;
     e = launch_down_stream(gu, wd, theta, w, idx, T, H, E, k, I, base + ws.hidden, yw, s);
     if (e != hipSuccess) return (int)e;
-    return hip_rc(launch_combine(yw, 0, idx, E, residual, T, H, k, dtype, out, s));
+    return hip_rc(launch_combine(yw, 0, cidx, E, residual, T, H, k, dtype, out, s));
   }
   if (algo == BIBO_ALGO_FUSED) {
     if (!aligned16(x) || !aligned16(wgu) || !aligned16(wd)) return BIBO_ERR_MISALIGNED;
     hipError_t e = launch_experts_fused(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, T, H, E, k, I, yw, s);
     if (e != hipSuccess) return (int)e;
-    return hip_rc(launch_combine(yw, 1, idx, E, residual, T, H, k, dtype, out, s));
+    return hip_rc(launch_combine(yw, 1, cidx, E, residual, T, H, k, dtype, out, s));
   }
   const int rc = gateup_dispatch(x, wgu, theta, offsets, perm_token, T, H, E, k, I, dtype, algo, base + ws.hidden, s);
   if (rc != BIBO_OK) return rc;
-  return down_dispatch(base + ws.hidden, wd, idx, w, offsets, perm_slot, residual, T, H, E, k, I, dtype, algo, out, yw, s);
+  return down_dispatch(base + ws.hidden, wd, cidx, w, offsets, perm_slot, residual, T, H, E, k, I, dtype, algo, out, yw, s);
 }
 
-// The whole layer on `x`; `residual` (or NULL) is added in the combine.  `extra` bytes at the end of the
-// workspace belong to the caller (the normalised activations of bibo_moe_ffn_forward).
+// The whole layer on `x`; `residual` (or NULL) is added in the combine.
 int forward_impl(const void* x, const void* w_router, const float* bias, const void* w_gate_up, const void* w_down,
                  const float* theta, const bibo_moe_shape* sh, int norm_mode, int algo, const void* residual, void* out,
                  int32_t* idx_out, float* w_out, int32_t* counts_out, float* logits_out, void* workspace,
@@ -160,18 +163,26 @@ int forward_impl(const void* x, const void* w_router, const float* bias, const v
   int32_t* offsets = reinterpret_cast<int32_t*>(base + ws.offsets);
   int32_t* perm_slot = reinterpret_cast<int32_t*>(base + ws.perm_slot);
   int32_t* perm_token = reinterpret_cast<int32_t*>(base + ws.perm_token);
-  if (T > 0 &&
-      (rc = hip_rc(launch_router(x, w_router, bias, T, H, E, k, dtype, norm_mode, logits_out, idx, w, nullptr, s))) !=
-          BIBO_OK)
-    return rc;
   // the streaming kernels find their rows themselves; the permutation then only serves the counts
   const bool need_permute = a != BIBO_ALGO_STREAM || counts_out != nullptr || T == 0;
-  if (need_permute &&
-      (rc = hip_rc(launch_permute(idx, T, E, k, counts, offsets, perm_slot, perm_token, base + ws.hist, s))) != BIBO_OK)
+  // the router kernel can leave per-workgroup histograms of its selections, which save the permutation its
+  // histogram launch and its counting pass
+  int32_t* hist = reinterpret_cast<int32_t*>(base + ws.hist);
+  int hist_tokens = 0;
+  const bool want_hist = need_permute && T > 0 && permute_takes_router_hist(T, k);
+  if (T > 0 && (rc = hip_rc(launch_router(x, w_router, bias, T, H, E, k, dtype, norm_mode, logits_out, idx, w, nullptr,
+                                          want_hist ? hist : nullptr, &hist_tokens, s))) != BIBO_OK)
     return rc;
+  if (need_permute) {
+    const hipError_t e = (want_hist && hist_tokens > 0)
+                             ? launch_permute_from_hist(idx, T, E, k, hist, hist_tokens, counts, offsets, perm_slot,
+                                                        perm_token, s)
+                             : launch_permute(idx, T, E, k, counts, offsets, perm_slot, perm_token, hist, s);
+    if (e != hipSuccess) return (int)e;
+  }
   if (T == 0) return BIBO_OK;
-  return experts_dispatch(x, w_gate_up, w_down, theta, idx, w, offsets, perm_slot, perm_token, residual, T, H, E, k, I,
-                          dtype, a, out, base, ws, s);
+  return experts_dispatch(x, w_gate_up, w_down, theta, idx, w, offsets, perm_slot, perm_token, residual, true, T, H, E, k,
+                          I, dtype, a, out, base, ws, s);
 }
 
 
@@ -211,7 +222,7 @@ int bibo_moe_router_fwd(const void* x, const void* w_router, const float* bias, 
   if (norm_mode < BIBO_NORM_NONE || norm_mode > BIBO_NORM_SOFTMAX) return BIBO_ERR_UNSUPPORTED;
   if (T == 0) return BIBO_OK;
   if (!x || !w_router || !bias || !idx || !w) return BIBO_ERR_NULL_POINTER;
-  return hip_rc(launch_router(x, w_router, bias, T, H, E, k, dtype, norm_mode, logits, idx, w, gap,
+  return hip_rc(launch_router(x, w_router, bias, T, H, E, k, dtype, norm_mode, logits, idx, w, gap, nullptr, nullptr,
                               static_cast<hipStream_t>(stream)));
 }
 
@@ -302,8 +313,8 @@ int bibo_moe_experts_fwd(const void* x, const int32_t* idx, const float* w, cons
       (rc = hip_rc(launch_permute(idx, T, E, k, counts, offsets, perm_slot, perm_token, base + ws.hist, s))) != BIBO_OK)
     return rc;
   if (T == 0) return BIBO_OK;
-  return experts_dispatch(x, w_gate_up, w_down, theta, idx, w, offsets, perm_slot, perm_token, nullptr, T, H, E, k, I,
-                          dtype, a, out, base, ws, s);
+  return experts_dispatch(x, w_gate_up, w_down, theta, idx, w, offsets, perm_slot, perm_token, nullptr, false, T, H, E, k,
+                          I, dtype, a, out, base, ws, s);
 }
 
 int bibo_moe_forward(const void* x, const void* w_router, const float* bias, const void* w_gate_up, const void* w_down,

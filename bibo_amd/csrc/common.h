@@ -108,11 +108,19 @@ __device__ __forceinline__ int xcd_tile(int bid, int total) {
 }
 
 // ---- host-side launchers (one per translation unit) -------------------------------------------
+// `chunk_hist` (or NULL): per-workgroup histograms of the selected experts, [ceil(T / *hist_tokens)][64]; *hist_tokens
+// comes back 0 when the kernel that ran does not write them.
 hipError_t launch_router(const void* x, const void* w_router, const float* bias, int T, int H, int E, int k, int dtype,
-                         int norm_mode, float* logits, int32_t* idx, float* w, float* gap, hipStream_t s);
+                         int norm_mode, float* logits, int32_t* idx, float* w, float* gap, int32_t* chunk_hist,
+                         int* hist_tokens, hipStream_t s);
 size_t permute_workspace_bytes(int T);
 hipError_t launch_permute(const int32_t* idx, int T, int E, int k, int32_t* counts, int32_t* offsets,
                           int32_t* perm_slot, int32_t* perm_token, void* ws, hipStream_t s);
+size_t router_hist_bytes(int T);
+bool permute_takes_router_hist(int T, int k);
+hipError_t launch_permute_from_hist(const int32_t* idx, int T, int E, int k, const int32_t* hist, int hist_tokens,
+                                    int32_t* counts, int32_t* offsets, int32_t* perm_slot, int32_t* perm_token,
+                                    hipStream_t s);
 hipError_t launch_gateup_generic(const void* x, const void* wgu, const float* theta, const int32_t* offsets,
                                  const int32_t* perm_token, int T, int H, int E, int k, int I, int dtype, void* hidden,
                                  hipStream_t s);

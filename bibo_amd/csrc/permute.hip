@@ -25,47 +25,62 @@ __global__ __launch_bounds__(256) void hist_kernel(const int32_t* __restrict__ i
 }
 
 // One workgroup per chunk of kPermTokens tokens, four waves of kPermTokens/4 tokens each, lane = expert for the
-// bookkeeping.  (1) every wave counts its own slots per expert; (2) the chunk histograms are summed
-// (all chunks for the totals, earlier chunks for this chunk's base) with the loads spread over the
-// 256 threads; (3) exclusive scan over experts; (4) every wave ranks its slots 64 at a time, slots of
-// one expert keeping ascending slot order.
+// bookkeeping.  (1) every wave gets the per-expert counts of its own slots; (2) the chunk histograms are
+// summed (all chunks for the totals, earlier chunks for this workgroup's base), the loads issued in batches;
+// (3) exclusive scan over experts; (4) every wave ranks its slots 64 at a time, slots of one expert keeping
+// ascending slot order.
+// HT = tokens per histogram in `hist`: kPermTokens for hist_kernel's output (the wave counts its own slots
+// with ballots), 16 or 32 for the histograms the router kernel wrote per workgroup (a wave's count is the sum
+// of its 32/HT histograms and no counting pass is needed).
+template <int HT>
 __global__ __launch_bounds__(256) void scatter_kernel(const int32_t* __restrict__ idx, int S, int E, int k,
-                                                      const int32_t* __restrict__ block_hist, int nblk,
+                                                      const int32_t* __restrict__ hist, int nhist,
                                                       int32_t* __restrict__ counts, int32_t* __restrict__ offsets,
                                                       int32_t* __restrict__ perm_slot, int32_t* __restrict__ perm_token) {
+  static_assert(kPermTokens == 128 && (HT == kPermTokens || HT == 16 || HT == 32), "a wave owns 32 tokens");
   __shared__ int part_tot[4][kMaxE], part_bef[4][kMaxE], wave_cnt[4][kMaxE];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int b = blockIdx.x;
   const int s0 = (b * kPermTokens + wave * (kPermTokens / 4)) * k;
   const int s1 = min(S, s0 + (kPermTokens / 4) * k);
   const unsigned long long lt = (1ull << lane) - 1ull;
+  constexpr int kPerWg = kPermTokens / HT;          // histograms that cover this workgroup's tokens
+  const int h0 = b * kPerWg;                        // the first of them
 
   int mycnt = 0;                                  // slots of expert `lane` among this wave's tokens
-  for (int base = s0; base < s1; base += kWave) {
-    const int s = base + lane;
-    int e = 0;
-    bool valid = s < s1;
-    if (valid) { e = idx[s]; valid = (unsigned)e < (unsigned)E; }
-    if (!valid) e = 0;
-    unsigned long long peers, mine;
-    match64(e, valid, lane, peers, mine);
-    mycnt += __popcll(mine);
+  if constexpr (HT == kPermTokens) {
+    for (int base = s0; base < s1; base += kWave) {
+      const int s = base + lane;
+      int e = 0;
+      bool valid = s < s1;
+      if (valid) { e = idx[s]; valid = (unsigned)e < (unsigned)E; }
+      if (!valid) e = 0;
+      unsigned long long peers, mine;
+      match64(e, valid, lane, peers, mine);
+      mycnt += __popcll(mine);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < kPerWg / 4; ++i) {
+      const int hh = h0 + wave * (kPerWg / 4) + i;
+      if (hh < nhist) mycnt += hist[hh * kMaxE + lane];
+    }
   }
   wave_cnt[wave][lane] = mycnt;
 
   int tot = 0, bef = 0;
-  constexpr int kBatch = 16;                       // chunk histograms requested together: one memory latency per batch
-  for (int bb0 = wave; bb0 < nblk; bb0 += 4 * kBatch) {
+  constexpr int kBatch = 16;                       // histograms requested together: one memory latency per batch
+  for (int bb0 = wave; bb0 < nhist; bb0 += 4 * kBatch) {
     int v[kBatch];
 #pragma unroll
     for (int u = 0; u < kBatch; ++u) {
       const int bb = bb0 + 4 * u;
-      v[u] = (bb < nblk) ? block_hist[bb * kMaxE + lane] : 0;
+      v[u] = (bb < nhist) ? hist[bb * kMaxE + lane] : 0;
     }
 #pragma unroll
     for (int u = 0; u < kBatch; ++u) {
       tot += v[u];
-      bef += (bb0 + 4 * u < b) ? v[u] : 0;
+      bef += (bb0 + 4 * u < h0) ? v[u] : 0;
     }
   }
   part_tot[wave][lane] = tot;
@@ -149,6 +164,9 @@ size_t permute_workspace_bytes(int T) {
   return (nblk > 0 ? nblk : 1) * kMaxE * sizeof(int32_t);
 }
 
+// room for the histograms the router kernel writes, one per 16 tokens at the finest
+size_t router_hist_bytes(int T) { return ((size_t)(T + 15) / 16 + 1) * kMaxE * sizeof(int32_t); }
+
 hipError_t launch_permute(const int32_t* idx, int T, int E, int k, int32_t* counts, int32_t* offsets,
                           int32_t* perm_slot, int32_t* perm_token, void* ws, hipStream_t s) {
   const int nblk = (T + kPermTokens - 1) / kPermTokens;
@@ -161,8 +179,28 @@ hipError_t launch_permute(const int32_t* idx, int T, int E, int k, int32_t* coun
   }
   const int grid = nblk;
   hipLaunchKernelGGL(hist_kernel, dim3(grid), dim3(256), 0, s, idx, S, E, k, block_hist);
-  hipLaunchKernelGGL(scatter_kernel, dim3(grid), dim3(256), 0, s, idx, S, E, k, block_hist, grid, counts, offsets,
-                     perm_slot, perm_token);
+  hipLaunchKernelGGL(scatter_kernel<kPermTokens>, dim3(grid), dim3(256), 0, s, idx, S, E, k, block_hist, grid, counts,
+                     offsets, perm_slot, perm_token);
+  return hipGetLastError();
+}
+
+bool permute_takes_router_hist(int T, int k) { return T * k > kSmallSlots; }
+
+// The same permutation from the per-workgroup histograms the router kernel wrote (one per `hist_tokens` tokens):
+// no histogram launch and no counting pass.
+hipError_t launch_permute_from_hist(const int32_t* idx, int T, int E, int k, const int32_t* hist, int hist_tokens,
+                                    int32_t* counts, int32_t* offsets, int32_t* perm_slot, int32_t* perm_token,
+                                    hipStream_t s) {
+  const int grid = (T + kPermTokens - 1) / kPermTokens;
+  const int nhist = (T + hist_tokens - 1) / hist_tokens;
+  if (hist_tokens == 32)
+    hipLaunchKernelGGL(scatter_kernel<32>, dim3(grid), dim3(256), 0, s, idx, T * k, E, k, hist, nhist, counts, offsets,
+                       perm_slot, perm_token);
+  else if (hist_tokens == 16)
+    hipLaunchKernelGGL(scatter_kernel<16>, dim3(grid), dim3(256), 0, s, idx, T * k, E, k, hist, nhist, counts, offsets,
+                       perm_slot, perm_token);
+  else
+    return hipErrorInvalidValue;
   return hipGetLastError();
 }
 

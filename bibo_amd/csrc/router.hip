@@ -177,9 +177,11 @@ __device__ __forceinline__ unsigned long long select_mask16(const float (&v)[4],
 
 // Selection for the tokens of one workgroup whose scores sit in LDS rows `sc` (stride kRowPad):
 // thread = (token tid>>4, segment tid&15); needs blockDim.x >= 16 * ntok_max.
-__device__ __forceinline__ void select_tokens16(const float* __restrict__ sc, const float* __restrict__ bias_s, int E,
-                                                int k, int norm_mode, int t0, int ntok, int32_t* __restrict__ idx,
-                                                float* __restrict__ w, float* __restrict__ gap) {
+// Returns the bit mask of the experts chosen for this thread's token (0 for a token past the end).
+__device__ __forceinline__ unsigned long long select_tokens16(const float* __restrict__ sc,
+                                                              const float* __restrict__ bias_s, int E, int k,
+                                                              int norm_mode, int t0, int ntok, int32_t* __restrict__ idx,
+                                                              float* __restrict__ w, float* __restrict__ gap) {
   const int tid = threadIdx.x;
   const int tl = tid >> 4, seg = tid & 15;
   const bool live = tl < ntok;                       // whole 16-lane groups are live or not
@@ -229,6 +231,7 @@ __device__ __forceinline__ void select_tokens16(const float* __restrict__ sc, co
     }
     if (gap != nullptr) gap[t] = (k < E) ? (g_hi - g_lo) : 0.f;
   }
+  return live ? mask : 0ull;
 }
 
 // ---- MFMA router: bf16, H % 128 == 0 ------------------------------------------------------------
@@ -249,7 +252,8 @@ __global__ __launch_bounds__(TOK * 16) void router_mfma_kernel(const bf16_t* __r
                                                                const float* __restrict__ bias, int T, int H, int E,
                                                                int k, int norm_mode, float* __restrict__ logits,
                                                                int32_t* __restrict__ idx, float* __restrict__ w,
-                                                               float* __restrict__ gap) {
+                                                               float* __restrict__ gap,
+                                                               int32_t* __restrict__ chunk_hist) {
   constexpr int kThreads = TOK * 16;
   constexpr int kRows = TOK + kMaxE;                 // stage rows: tokens first, then experts
   constexpr int kPer = kRows * kRouterGran / kThreads;   // load instructions per thread and chunk
@@ -317,7 +321,18 @@ __global__ __launch_bounds__(TOK * 16) void router_mfma_kernel(const bf16_t* __r
     }
   }
   __syncthreads();
-  select_tokens16(sc, bias_s, E, k, norm_mode, t0, ntok, idx, w, gap);
+  const unsigned long long mask = select_tokens16(sc, bias_s, E, k, norm_mode, t0, ntok, idx, w, gap);
+  if (chunk_hist != nullptr) {           // histogram of this workgroup's selections, for the permutation kernel
+    __shared__ unsigned long long mask_s[TOK];
+    if ((tid & 15) == 0) mask_s[tid >> 4] = mask;
+    __syncthreads();
+    if (tid < kMaxE) {
+      int c = 0;
+#pragma unroll
+      for (int t = 0; t < TOK; ++t) c += (int)((mask_s[t] >> tid) & 1ull);
+      chunk_hist[blockIdx.x * kMaxE + tid] = c;
+    }
+  }
 }
 
 // ---- MFMA router for H % 32 == 0 but not % 128: operands straight to registers, K split over 4 waves ----
@@ -389,7 +404,9 @@ __global__ __launch_bounds__(256) void router_mfma_split_kernel(const bf16_t* __
 }  // namespace
 
 hipError_t launch_router(const void* x, const void* w_router, const float* bias, int T, int H, int E, int k, int dtype,
-                         int norm_mode, float* logits, int32_t* idx, float* w, float* gap, hipStream_t s) {
+                         int norm_mode, float* logits, int32_t* idx, float* w, float* gap, int32_t* chunk_hist,
+                         int* hist_tokens, hipStream_t s) {
+  if (hist_tokens != nullptr) *hist_tokens = 0;
   if (T == 0) return hipSuccess;
   const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w_router)) & 15) == 0;
   if (dtype == BIBO_DTYPE_BF16 && (H % kRouterKC) == 0 && aligned) {
@@ -397,10 +414,13 @@ hipError_t launch_router(const void* x, const void* w_router, const float* bias,
     // smaller tile keeps more CUs busy
     if (T >= 32 * 256)
       hipLaunchKernelGGL(router_mfma_kernel<32>, dim3((T + 31) / 32), dim3(512), 0, s, static_cast<const bf16_t*>(x),
-                         static_cast<const bf16_t*>(w_router), bias, T, H, E, k, norm_mode, logits, idx, w, gap);
+                         static_cast<const bf16_t*>(w_router), bias, T, H, E, k, norm_mode, logits, idx, w, gap,
+                         chunk_hist);
     else
       hipLaunchKernelGGL(router_mfma_kernel<16>, dim3((T + 15) / 16), dim3(256), 0, s, static_cast<const bf16_t*>(x),
-                         static_cast<const bf16_t*>(w_router), bias, T, H, E, k, norm_mode, logits, idx, w, gap);
+                         static_cast<const bf16_t*>(w_router), bias, T, H, E, k, norm_mode, logits, idx, w, gap,
+                         chunk_hist);
+    if (hist_tokens != nullptr && chunk_hist != nullptr) *hist_tokens = T >= 32 * 256 ? 32 : 16;
   } else if (dtype == BIBO_DTYPE_BF16 && (H % 32) == 0 && aligned) {
     const int grid = (T + kMfmaTokens - 1) / kMfmaTokens;
     hipLaunchKernelGGL(router_mfma_split_kernel, dim3(grid), dim3(256), 0, s, static_cast<const bf16_t*>(x),
