@@ -31,7 +31,8 @@ constexpr int kScan = kStreamMaxSlots / 256;   // routing indices each thread in
 
 // Slots routed to expert e, ascending, into rows_s; returns how many.  All 256 threads call it; slot
 // s = 256*q + tid, so slot order is (q, wave, lane).  Ends with a barrier.
-__device__ __forceinline__ int expert_rows(const int32_t* __restrict__ idx, int S, int e, int* rows_s, int* cnt_s) {
+__device__ __forceinline__ int expert_rows(const int32_t* __restrict__ idx, int S, int e, unsigned short* rows_s,
+                                           int* cnt_s) {
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const unsigned long long lt = (1ull << lane) - 1ull;
   int v[kScan];
@@ -53,7 +54,7 @@ __device__ __forceinline__ int expert_rows(const int32_t* __restrict__ idx, int 
   for (int q = 0; q < kScan; ++q)
 #pragma unroll
     for (int ww = 0; ww < 4; ++ww) {
-      if (ww == wave && v[q] == e) rows_s[run + rank[q]] = q * 256 + tid;
+      if (ww == wave && v[q] == e) rows_s[run + rank[q]] = (unsigned short)(q * 256 + tid);
       run += cnt_s[q * 4 + ww];
     }
   __syncthreads();
@@ -101,11 +102,11 @@ __device__ __forceinline__ floatx4 stream_rows(const bf16_t* __restrict__ wrow, 
 }
 
 // grid = (2I / 64, E).  gu[slot, c] = x[slot / k] . w_gate_up[e, c, :]
-__global__ __launch_bounds__(256) void gateup_stream_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wgu,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void gateup_stream_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wgu,
                                                             const int32_t* __restrict__ idx, int S, int k, int H, int I,
                                                             float* __restrict__ gu) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  __shared__ int rows_s[kStreamMaxSlots];
+  __shared__ unsigned short rows_s[kStreamMaxSlots];   // 16-bit slot ids keep four workgroups within a CU's LDS
   __shared__ int cnt_s[kScan * 4];
   bf16_t* xs = reinterpret_cast<bf16_t*>(smem_raw);            // [kTok][H + 8]
   const int e = blockIdx.y;
@@ -160,11 +161,11 @@ __global__ __launch_bounds__(256) void activate_rows_kernel(const float* __restr
 }
 
 // grid = (H / 64, E).  yw[slot, c] = w[slot] * (hidden[slot] . w_down[e, c, :])
-__global__ __launch_bounds__(256) void down_stream_kernel(const bf16_t* __restrict__ hidden, const bf16_t* __restrict__ wd,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void down_stream_kernel(const bf16_t* __restrict__ hidden, const bf16_t* __restrict__ wd,
                                                           const float* __restrict__ w, const int32_t* __restrict__ idx,
                                                           int S, int H, int I, float* __restrict__ yw) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  __shared__ int rows_s[kStreamMaxSlots];
+  __shared__ unsigned short rows_s[kStreamMaxSlots];   // 16-bit slot ids keep four workgroups within a CU's LDS
   __shared__ int cnt_s[kScan * 4];
   bf16_t* hs = reinterpret_cast<bf16_t*>(smem_raw);            // [kTok][I + 8] activations of this pass
   const int e = blockIdx.y;
