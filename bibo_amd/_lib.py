@@ -13,20 +13,20 @@ DTYPE_BF16, DTYPE_F32 = 0, 1
 NORM_NONE, NORM_SUM, NORM_SOFTMAX = 0, 1, 2
 ALGO_AUTO, ALGO_GENERIC, ALGO_MFMA, ALGO_STREAM, ALGO_FUSED = 0, 1, 2, 3, 4
 MAX_EXPERTS, MAX_TOPK = 64, 8
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 # every symbol include/bibo_moe.h declares
 SYMBOLS = (
     "bibo_moe_abi_version", "bibo_moe_strerror", "bibo_moe_workspace_bytes", "bibo_moe_router_fwd",
     "bibo_moe_permute", "bibo_moe_gateup_fwd", "bibo_moe_down_combine_fwd", "bibo_moe_gateup_down_fwd",
-    "bibo_moe_combine_fwd", "bibo_moe_experts_fwd", "bibo_moe_forward", "bibo_moe_rmsnorm_fwd",
+    "bibo_moe_combine_fwd", "bibo_moe_combine_ex_fwd", "bibo_moe_experts_fwd", "bibo_moe_forward", "bibo_moe_rmsnorm_fwd",
     "bibo_moe_ffn_workspace_bytes", "bibo_moe_ffn_forward",
 )
 
 
 class Shape(ctypes.Structure):
     _fields_ = [("T", ctypes.c_int32), ("H", ctypes.c_int32), ("E", ctypes.c_int32), ("k", ctypes.c_int32),
-                ("I", ctypes.c_int32), ("dtype", ctypes.c_int32)]
+                ("I", ctypes.c_int32), ("dtype", ctypes.c_int32), ("n_pos", ctypes.c_int32), ("n_neg", ctypes.c_int32)]
 
 
 _lock = threading.Lock()
@@ -53,6 +53,8 @@ def _declare(l):
     l.bibo_moe_gateup_down_fwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, vp, vp]
     l.bibo_moe_combine_fwd.restype = ci
     l.bibo_moe_combine_fwd.argtypes = [vp, ci, ci, ci, ci, ci, vp, vp]
+    l.bibo_moe_combine_ex_fwd.restype = ci
+    l.bibo_moe_combine_ex_fwd.argtypes = [vp, ci, vp, vp, vp, ci, ci, ci, vp, ci, ci, ci, ci, vp, vp]
     l.bibo_moe_experts_fwd.restype = ci
     l.bibo_moe_experts_fwd.argtypes = [vp, vp, vp, vp, vp, vp, ctypes.POINTER(Shape), ci, vp, vp, vp, sz, vp]
     l.bibo_moe_rmsnorm_fwd.restype = ci

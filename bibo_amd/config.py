@@ -11,7 +11,7 @@ class BiBoMoEConfig:
                  num_routed_experts=6, special_expert_pairs=1, pos_identity_expert=True, neg_identity_expert=True,
                  num_pos_identity_experts=None, num_neg_identity_experts=None, use_shared_expert=False,
                  shared_expert_type="mlp", num_shared_experts=1, norm_topk_prob="sum", bias_update_factor=None,
-                 bias_update_threshold=8000, initializer_range=0.02, **unused):
+                 bias_update_threshold=8000, initializer_range=0.02, hidden_act="silu", **unused):
         self.hidden_size = hidden_size
         self.intermediate_size = intermediate_size
         self.num_experts_per_tok = num_experts_per_tok
@@ -36,6 +36,7 @@ class BiBoMoEConfig:
         self.bias_update_factor = 0.4 if bias_update_factor is None else bias_update_factor
         self.bias_update_threshold = 8000 if bias_update_threshold is None else bias_update_threshold
         self.initializer_range = initializer_range
+        self.hidden_act = hidden_act
         if not 1 <= num_experts_per_tok <= num_routed_experts:
             raise ValueError(f"num_experts_per_tok ({num_experts_per_tok}) must be in "
                              f"[1, num_routed_experts={num_routed_experts}]")

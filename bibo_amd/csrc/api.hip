@@ -11,7 +11,8 @@ inline size_t align_up(size_t v) { return (v + kAlign - 1) & ~(kAlign - 1); }
 inline size_t elt_size(int dtype) { return dtype == BIBO_DTYPE_BF16 ? 2 : 4; }
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-int check_dims(int T, int H, int E, int k, int I, int dtype) {
+int check_dims(int T, int H, int E, int k, int I, int dtype, int n_pos = 0, int n_neg = 0) {
+  if (n_pos < 0 || n_neg < 0 || n_pos + n_neg >= E) return BIBO_ERR_BAD_SHAPE;     // at least one GLU expert
   if (dtype != BIBO_DTYPE_BF16 && dtype != BIBO_DTYPE_F32) return BIBO_ERR_BAD_DTYPE;
   if (T < 0 || H < 1 || I < 1 || E < 1 || E > kMaxE || k < 1 || k > kMaxK || k > E) return BIBO_ERR_BAD_SHAPE;
   if ((long long)T * k > 0x3fffffffLL) return BIBO_ERR_BAD_SHAPE;
@@ -92,9 +93,10 @@ int gateup_dispatch(const void* x, const void* wgu, const float* theta, const in
   return hip_rc(launch_gateup_generic(x, wgu, theta, offsets, perm_token, T, H, E, k, I, dtype, hidden, s));
 }
 
-int down_dispatch(const void* hidden, const void* wd, const int32_t* idx, const float* w, const int32_t* offsets,
-                  const int32_t* perm_slot, const void* residual, int T, int H, int E, int k, int I, int dtype, int algo,
-                  void* out, float* yw, hipStream_t s) {
+// E here and in gateup_dispatch counts the GLU experts (those that have weights)
+int down_dispatch(const void* hidden, const void* wd, const float* w, const int32_t* offsets, const int32_t* perm_slot,
+                  const CombineArgs& ca, int T, int H, int E, int k, int I, int dtype, int algo, void* out, float* yw,
+                  hipStream_t s) {
   hipError_t e;
   if (algo == BIBO_ALGO_MFMA) {
     if (!aligned16(hidden) || !aligned16(wd)) return BIBO_ERR_MISALIGNED;
@@ -102,41 +104,44 @@ int down_dispatch(const void* hidden, const void* wd, const int32_t* idx, const 
     // expert output to bf16 as well, moe.py:92)
     e = launch_down_mfma(hidden, wd, w, offsets, perm_slot, T, H, E, k, I, yw, s);
     if (e != hipSuccess) return (int)e;
-    return hip_rc(launch_combine(yw, 1, idx, E, residual, T, H, k, dtype, out, s));
+    return hip_rc(launch_combine(yw, 1, ca, T, H, k, dtype, out, s));
   }
   e = launch_down_generic(hidden, wd, w, offsets, perm_slot, T, H, E, k, I, dtype, yw, s);
   if (e != hipSuccess) return (int)e;
-  return hip_rc(launch_combine(yw, 0, idx, E, residual, T, H, k, dtype, out, s));
+  return hip_rc(launch_combine(yw, 0, ca, T, H, k, dtype, out, s));
 }
 
 // kernels 3 and 4 (+ combine) after the permutation, for the composite entry points
+// Eg = GLU experts (with weights), np / nn = +/-Identity specials behind them (moe.py:39-44).
 int experts_dispatch(const void* x, const void* wgu, const void* wd, const float* theta, const int32_t* idx,
                      const float* w, const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token,
-                     const void* residual, bool idx_trusted, int T, int H, int E, int k, int I, int dtype, int algo,
-                     void* out, char* base, const Workspace& ws, hipStream_t s) {
+                     const void* residual, bool idx_trusted, int T, int H, int Eg, int np, int nn, int k, int I, int dtype,
+                     int algo, void* out, char* base, const Workspace& ws, hipStream_t s) {
   float* yw = reinterpret_cast<float*>(base + ws.yw);
-  // indices that come straight from the router kernel are in range; a caller's may hold padding values,
-  // whose slots the combine then has to skip
-  const int32_t* cidx = idx_trusted ? nullptr : idx;
+  CombineArgs ca;
+  ca.residual = residual;
+  // indices that come straight from the router kernel are in range; a caller's may hold padding values, whose
+  // slots the combine has to skip; specials are the combine's work either way (moe.py:95-99)
+  if (!idx_trusted || np + nn > 0) { ca.idx = idx; ca.w = w; ca.x = x; ca.E_glu = Eg; ca.n_pos = np; ca.n_neg = nn; }
   if (algo == BIBO_ALGO_STREAM) {
     if (!aligned16(x) || !aligned16(wgu) || !aligned16(wd)) return BIBO_ERR_MISALIGNED;
-    if (!stream_eligible(T, H, E, k, I, dtype)) return BIBO_ERR_UNSUPPORTED;     // no pre-activation segment carved
+    if (!stream_eligible(T, H, Eg + np + nn, k, I, dtype)) return BIBO_ERR_UNSUPPORTED;   // no pre-activation segment carved
     float* gu = reinterpret_cast<float*>(base + ws.gu);
-    hipError_t e = launch_gateup_stream(x, wgu, idx, T, H, E, k, I, gu, s);
+    hipError_t e = launch_gateup_stream(x, wgu, idx, T, H, Eg, k, I, gu, s);
     if (e != hipSuccess) return (int)e;
-    e = launch_down_stream(gu, wd, theta, w, idx, T, H, E, k, I, base + ws.hidden, yw, s);
+    e = launch_down_stream(gu, wd, theta, w, idx, T, H, Eg, k, I, base + ws.hidden, yw, s);
     if (e != hipSuccess) return (int)e;
-    return hip_rc(launch_combine(yw, 0, cidx, E, residual, T, H, k, dtype, out, s));
+    return hip_rc(launch_combine(yw, 0, ca, T, H, k, dtype, out, s));
   }
   if (algo == BIBO_ALGO_FUSED) {
     if (!aligned16(x) || !aligned16(wgu) || !aligned16(wd)) return BIBO_ERR_MISALIGNED;
-    hipError_t e = launch_experts_fused(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, T, H, E, k, I, yw, s);
+    hipError_t e = launch_experts_fused(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, T, H, Eg, k, I, yw, s);
     if (e != hipSuccess) return (int)e;
-    return hip_rc(launch_combine(yw, 1, cidx, E, residual, T, H, k, dtype, out, s));
+    return hip_rc(launch_combine(yw, 1, ca, T, H, k, dtype, out, s));
   }
-  const int rc = gateup_dispatch(x, wgu, theta, offsets, perm_token, T, H, E, k, I, dtype, algo, base + ws.hidden, s);
+  const int rc = gateup_dispatch(x, wgu, theta, offsets, perm_token, T, H, Eg, k, I, dtype, algo, base + ws.hidden, s);
   if (rc != BIBO_OK) return rc;
-  return down_dispatch(base + ws.hidden, wd, cidx, w, offsets, perm_slot, residual, T, H, E, k, I, dtype, algo, out, yw, s);
+  return down_dispatch(base + ws.hidden, wd, w, offsets, perm_slot, ca, T, H, Eg, k, I, dtype, algo, out, yw, s);
 }
 
 // The whole layer on `x`; `residual` (or NULL) is added in the combine.
@@ -146,8 +151,9 @@ int forward_impl(const void* x, const void* w_router, const float* bias, const v
                  size_t workspace_bytes, void* stream) {
   if (sh == nullptr) return BIBO_ERR_NULL_POINTER;
   const int T = sh->T, H = sh->H, E = sh->E, k = sh->k, I = sh->I, dtype = sh->dtype;
-  int rc = check_dims(T, H, E, k, I, dtype);
+  int rc = check_dims(T, H, E, k, I, dtype, sh->n_pos, sh->n_neg);
   if (rc != BIBO_OK) return rc;
+  const int Eg = E - sh->n_pos - sh->n_neg;
   if (norm_mode < BIBO_NORM_NONE || norm_mode > BIBO_NORM_SOFTMAX) return BIBO_ERR_UNSUPPORTED;
   int a;
   if ((rc = resolve_algo(algo, T, H, E, k, I, dtype, true, &a)) != BIBO_OK) return rc;
@@ -181,8 +187,8 @@ int forward_impl(const void* x, const void* w_router, const float* bias, const v
     if (e != hipSuccess) return (int)e;
   }
   if (T == 0) return BIBO_OK;
-  return experts_dispatch(x, w_gate_up, w_down, theta, idx, w, offsets, perm_slot, perm_token, residual, true, T, H, E, k,
-                          I, dtype, a, out, base, ws, s);
+  return experts_dispatch(x, w_gate_up, w_down, theta, idx, w, offsets, perm_slot, perm_token, residual, true, T, H, Eg,
+                          sh->n_pos, sh->n_neg, k, I, dtype, a, out, base, ws, s);
 }
 
 
@@ -196,7 +202,8 @@ const char* bibo_moe_strerror(int code) {
   switch (code) {
     case BIBO_OK: return "success";
     case BIBO_ERR_NULL_POINTER: return "a required pointer is NULL";
-    case BIBO_ERR_BAD_SHAPE: return "bad shape: need T >= 0, H, I >= 1, 1 <= E <= 64, 1 <= k <= min(E, 8)";
+    case BIBO_ERR_BAD_SHAPE:
+      return "bad shape: need T >= 0, H, I >= 1, 1 <= E <= 64, 1 <= k <= min(E, 8), n_pos, n_neg >= 0, n_pos + n_neg < E";
     case BIBO_ERR_BAD_DTYPE: return "dtype must be BIBO_DTYPE_BF16 or BIBO_DTYPE_F32";
     case BIBO_ERR_WORKSPACE_TOO_SMALL: return "workspace smaller than bibo_moe_workspace_bytes() for this shape";
     case BIBO_ERR_MISALIGNED: return "tensor base pointers must be 16-byte aligned";
@@ -209,7 +216,7 @@ const char* bibo_moe_strerror(int code) {
 
 int bibo_moe_workspace_bytes(const bibo_moe_shape* sh, size_t* bytes) {
   if (sh == nullptr || bytes == nullptr) return BIBO_ERR_NULL_POINTER;
-  const int rc = check_dims(sh->T, sh->H, sh->E, sh->k, sh->I, sh->dtype);
+  const int rc = check_dims(sh->T, sh->H, sh->E, sh->k, sh->I, sh->dtype, sh->n_pos, sh->n_neg);
   if (rc != BIBO_OK) return rc;
   *bytes = carve(sh->T, sh->H, sh->E, sh->k, sh->I, sh->dtype).total;
   return BIBO_OK;
@@ -260,7 +267,7 @@ int bibo_moe_down_combine_fwd(const void* hidden, const void* w_down, const floa
   if (T == 0) return BIBO_OK;
   if (!hidden || !w_down || !w || !offsets || !perm_slot || !out || !workspace) return BIBO_ERR_NULL_POINTER;
   if (workspace_bytes < (size_t)T * k * H * sizeof(float)) return BIBO_ERR_WORKSPACE_TOO_SMALL;
-  return down_dispatch(hidden, w_down, nullptr, w, offsets, perm_slot, nullptr, T, H, E, k, I, dtype, a, out,
+  return down_dispatch(hidden, w_down, w, offsets, perm_slot, CombineArgs{}, T, H, E, k, I, dtype, a, out,
                        static_cast<float*>(workspace), static_cast<hipStream_t>(stream));
 }
 
@@ -285,7 +292,22 @@ int bibo_moe_combine_fwd(const void* yw, int yw_is_bf16, int T, int H, int k, in
   if (yw_is_bf16 && dtype != BIBO_DTYPE_BF16) return BIBO_ERR_BAD_DTYPE;
   if (T == 0) return BIBO_OK;
   if (!yw || !out) return BIBO_ERR_NULL_POINTER;
-  return hip_rc(launch_combine(yw, yw_is_bf16 ? 1 : 0, nullptr, 0, nullptr, T, H, k, dtype, out, static_cast<hipStream_t>(stream)));
+  return hip_rc(launch_combine(yw, yw_is_bf16 ? 1 : 0, CombineArgs{}, T, H, k, dtype, out, static_cast<hipStream_t>(stream)));
+}
+
+int bibo_moe_combine_ex_fwd(const void* yw, int yw_is_bf16, const int32_t* idx, const float* w, const void* x, int E_glu,
+                            int n_pos, int n_neg, const void* residual, int T, int H, int k, int dtype, void* out,
+                            void* stream) {
+  const int rc = check_dims(T, H, k, k, 1, dtype);   // no expert dimension here: E := k, I := 1 pass the range checks
+  if (rc != BIBO_OK) return rc;
+  if (yw_is_bf16 && dtype != BIBO_DTYPE_BF16) return BIBO_ERR_BAD_DTYPE;
+  if (E_glu < 0 || n_pos < 0 || n_neg < 0 || E_glu + n_pos + n_neg > kMaxE) return BIBO_ERR_BAD_SHAPE;
+  if (T == 0) return BIBO_OK;
+  if (!yw || !out) return BIBO_ERR_NULL_POINTER;
+  if (n_pos + n_neg > 0 && (!idx || !w || !x)) return BIBO_ERR_NULL_POINTER;
+  CombineArgs ca;
+  ca.idx = idx; ca.w = w; ca.x = x; ca.E_glu = E_glu; ca.n_pos = n_pos; ca.n_neg = n_neg; ca.residual = residual;
+  return hip_rc(launch_combine(yw, yw_is_bf16 ? 1 : 0, ca, T, H, k, dtype, out, static_cast<hipStream_t>(stream)));
 }
 
 int bibo_moe_experts_fwd(const void* x, const int32_t* idx, const float* w, const void* w_gate_up, const void* w_down,
@@ -293,8 +315,9 @@ int bibo_moe_experts_fwd(const void* x, const int32_t* idx, const float* w, cons
                          void* workspace, size_t workspace_bytes, void* stream) {
   if (sh == nullptr) return BIBO_ERR_NULL_POINTER;
   const int T = sh->T, H = sh->H, E = sh->E, k = sh->k, I = sh->I, dtype = sh->dtype;
-  int rc = check_dims(T, H, E, k, I, dtype);
+  int rc = check_dims(T, H, E, k, I, dtype, sh->n_pos, sh->n_neg);
   if (rc != BIBO_OK) return rc;
+  const int Eg = E - sh->n_pos - sh->n_neg;
   int a;
   if ((rc = resolve_algo(algo, T, H, E, k, I, dtype, true, &a)) != BIBO_OK) return rc;
   if (!workspace) return BIBO_ERR_NULL_POINTER;
@@ -313,8 +336,8 @@ int bibo_moe_experts_fwd(const void* x, const int32_t* idx, const float* w, cons
       (rc = hip_rc(launch_permute(idx, T, E, k, counts, offsets, perm_slot, perm_token, base + ws.hist, s))) != BIBO_OK)
     return rc;
   if (T == 0) return BIBO_OK;
-  return experts_dispatch(x, w_gate_up, w_down, theta, idx, w, offsets, perm_slot, perm_token, nullptr, false, T, H, E, k,
-                          I, dtype, a, out, base, ws, s);
+  return experts_dispatch(x, w_gate_up, w_down, theta, idx, w, offsets, perm_slot, perm_token, nullptr, false, T, H, Eg,
+                          sh->n_pos, sh->n_neg, k, I, dtype, a, out, base, ws, s);
 }
 
 int bibo_moe_forward(const void* x, const void* w_router, const float* bias, const void* w_gate_up, const void* w_down,
@@ -336,7 +359,7 @@ int bibo_moe_rmsnorm_fwd(const void* x, const float* norm_weight, float eps, int
 
 int bibo_moe_ffn_workspace_bytes(const bibo_moe_shape* sh, size_t* out) {
   if (sh == nullptr || out == nullptr) return BIBO_ERR_NULL_POINTER;
-  const int rc = check_dims(sh->T, sh->H, sh->E, sh->k, sh->I, sh->dtype);
+  const int rc = check_dims(sh->T, sh->H, sh->E, sh->k, sh->I, sh->dtype, sh->n_pos, sh->n_neg);
   if (rc != BIBO_OK) return rc;
   *out = carve(sh->T, sh->H, sh->E, sh->k, sh->I, sh->dtype).total + align_up((size_t)sh->T * sh->H * elt_size(sh->dtype));
   return BIBO_OK;
@@ -347,7 +370,7 @@ int bibo_moe_ffn_forward(const void* h, const float* norm_weight, float eps, con
                          int norm_mode, int algo, void* out, int32_t* idx_out, float* w_out, int32_t* counts_out,
                          void* workspace, size_t workspace_bytes, void* stream) {
   if (sh == nullptr) return BIBO_ERR_NULL_POINTER;
-  const int rc = check_dims(sh->T, sh->H, sh->E, sh->k, sh->I, sh->dtype);
+  const int rc = check_dims(sh->T, sh->H, sh->E, sh->k, sh->I, sh->dtype, sh->n_pos, sh->n_neg);
   if (rc != BIBO_OK) return rc;
   if (!workspace) return BIBO_ERR_NULL_POINTER;
   if (sh->T > 0 && (!h || !norm_weight || !out)) return BIBO_ERR_NULL_POINTER;

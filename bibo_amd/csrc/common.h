@@ -127,8 +127,16 @@ hipError_t launch_gateup_generic(const void* x, const void* wgu, const float* th
 hipError_t launch_down_generic(const void* hidden, const void* wd, const float* w, const int32_t* offsets,
                                const int32_t* perm_slot, int T, int H, int E, int k, int I, int dtype, float* yw,
                                hipStream_t s);
-hipError_t launch_combine(const void* yw, int yw_is_bf16, const int32_t* idx, int E, const void* residual, int T, int H,
-                          int k, int dtype, void* out, hipStream_t s);
+// What the combine folds in besides the slot rows; every pointer may be NULL (see combine_kernel).
+struct CombineArgs {
+  const int32_t* idx = nullptr;    // [T,k]; needed for specials and for skipping out-of-range slots
+  const float* w = nullptr;        // [T,k]; needed for specials
+  const void* x = nullptr;         // [T,H] in the output dtype; needed for specials
+  int E_glu = 0, n_pos = 0, n_neg = 0;
+  const void* residual = nullptr;  // [T,H] in the output dtype
+};
+hipError_t launch_combine(const void* yw, int yw_is_bf16, const CombineArgs& a, int T, int H, int k, int dtype,
+                          void* out, hipStream_t s);
 hipError_t launch_rmsnorm(const void* x, const float* weight, float eps, int T, int H, int dtype, void* out,
                           hipStream_t s);
 bool mfma_supported(int H, int I, int dtype);

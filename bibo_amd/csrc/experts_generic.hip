@@ -87,19 +87,36 @@ __global__ __launch_bounds__(256) void down_generic_kernel(const TIn* __restrict
   }
 }
 
-// out[t, :] = round(residual[t, :] + sum_j yw[t*k + j, :])  in fp32, ascending j   (moe.py:93,101; the residual
-// add of the caller, src/modeling/layers.py:62, when `residual` is given).  With `idx` given, slots whose
-// expert index is outside [0,E) are skipped (no kernel wrote their row).
+// out[t, :] = round(residual[t, :] + sum_j contribution(t, j))  in fp32, ascending j   (moe.py:93-101; the residual
+// add of the caller, src/modeling/layers.py:62, when `residual` is given).  contribution = yw[t*k + j, :] for a GLU
+// expert; with `idx` given, +/- w[t,j] * x[t, :] for a +/-Identity special (moe.py:95-99) and nothing for an index
+// outside [0, E_glu + n_pos + n_neg) (no kernel wrote that slot's row).
+template <typename TX>
+__device__ __forceinline__ bool special_slot(const CombineArgs& a, size_t slot, int* sign) {
+  *sign = 0;
+  if (a.idx == nullptr) return false;
+  const int e = a.idx[slot];
+  if ((unsigned)e >= (unsigned)(a.E_glu + a.n_pos + a.n_neg)) return true;       // skipped
+  if (e < a.E_glu) return false;
+  *sign = e < a.E_glu + a.n_pos ? 1 : -1;
+  return true;
+}
+
 template <typename TY, typename TOut>
-__global__ __launch_bounds__(256) void combine_kernel(const TY* __restrict__ yw, const int32_t* __restrict__ idx, int E,
-                                                      const TOut* __restrict__ residual, int T, int H, int k,
+__global__ __launch_bounds__(256) void combine_kernel(const TY* __restrict__ yw, CombineArgs a, int T, int H, int k,
                                                       TOut* __restrict__ out) {
   const size_t n = (size_t)T * H;
+  const TOut* x = static_cast<const TOut*>(a.x);
+  const TOut* residual = static_cast<const TOut*>(a.residual);
   for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
     const size_t t = i / H, h = i - t * H;
     float acc = 0.f;
     for (int j = 0; j < k; ++j) {
-      if (idx != nullptr && (unsigned)idx[t * k + j] >= (unsigned)E) continue;
+      int sign;
+      if (special_slot<TOut>(a, t * k + j, &sign)) {
+        if (sign != 0) acc += (float)sign * a.w[t * k + j] * to_float(x[i]);
+        continue;
+      }
       acc += to_float(yw[(t * k + j) * H + h]);
     }
     if (residual != nullptr) acc += to_float(residual[i]);
@@ -107,11 +124,9 @@ __global__ __launch_bounds__(256) void combine_kernel(const TY* __restrict__ yw,
   }
 }
 
-// bf16 slot rows -> bf16 output, 8 columns (16 bytes) per thread, fp32 sum in ascending j   (moe.py:93,101)
-__global__ __launch_bounds__(256) void combine_bf16x8_kernel(const bf16_t* __restrict__ yw,
-                                                             const int32_t* __restrict__ idx, int E,
-                                                             const bf16_t* __restrict__ residual, int T, int H8, int k,
-                                                             bf16_t* __restrict__ out) {
+// bf16 slot rows -> bf16 output, 8 columns (16 bytes) per thread, fp32 sum in ascending j
+__global__ __launch_bounds__(256) void combine_bf16x8_kernel(const bf16_t* __restrict__ yw, CombineArgs a, int T, int H8,
+                                                             int k, bf16_t* __restrict__ out) {
   const size_t n = (size_t)T * H8;
   for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
     const size_t t = i / H8, c = i - t * H8;
@@ -120,13 +135,22 @@ __global__ __launch_bounds__(256) void combine_bf16x8_kernel(const bf16_t* __res
     for (int q = 0; q < 8; ++q) acc[q] = 0.f;
     const bf16x8* src = reinterpret_cast<const bf16x8*>(yw) + (t * k) * H8 + c;
     for (int j = 0; j < k; ++j) {
-      if (idx != nullptr && (unsigned)idx[t * k + j] >= (unsigned)E) continue;
+      int sign;
+      if (special_slot<bf16_t>(a, t * k + j, &sign)) {
+        if (sign != 0) {
+          const float sw = (float)sign * a.w[t * k + j];
+          const bf16x8 xv = reinterpret_cast<const bf16x8*>(a.x)[i];
+#pragma unroll
+          for (int q = 0; q < 8; ++q) acc[q] += sw * (float)xv[q];
+        }
+        continue;
+      }
       const bf16x8 v = src[(size_t)j * H8];
 #pragma unroll
       for (int q = 0; q < 8; ++q) acc[q] += (float)v[q];
     }
-    if (residual != nullptr) {
-      const bf16x8 r = reinterpret_cast<const bf16x8*>(residual)[i];
+    if (a.residual != nullptr) {
+      const bf16x8 r = reinterpret_cast<const bf16x8*>(a.residual)[i];
 #pragma unroll
       for (int q = 0; q < 8; ++q) acc[q] += (float)r[q];
     }
@@ -171,29 +195,28 @@ hipError_t launch_down_generic(const void* hidden, const void* wd, const float* 
   return hipGetLastError();
 }
 
-hipError_t launch_combine(const void* yw, int yw_is_bf16, const int32_t* idx, int E, const void* residual, int T, int H,
-                          int k, int dtype, void* out, hipStream_t s) {
+hipError_t launch_combine(const void* yw, int yw_is_bf16, const CombineArgs& a, int T, int H, int k, int dtype,
+                          void* out, hipStream_t s) {
   const size_t n = (size_t)T * H;
   if (n == 0) return hipSuccess;
   const int grid = (int)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
   if (yw_is_bf16) {
     if (dtype != BIBO_DTYPE_BF16) return hipErrorInvalidValue;
     if ((H % 8) == 0 && ((reinterpret_cast<uintptr_t>(yw) | reinterpret_cast<uintptr_t>(out) |
-                          reinterpret_cast<uintptr_t>(residual)) & 15) == 0) {
+                          reinterpret_cast<uintptr_t>(a.residual) | reinterpret_cast<uintptr_t>(a.x)) & 15) == 0) {
       const size_t n8 = n / 8;
       const int g8 = (int)((n8 + 255) / 256 < 65536 ? (n8 + 255) / 256 : 65536);
-      hipLaunchKernelGGL(combine_bf16x8_kernel, dim3(g8), dim3(256), 0, s, static_cast<const bf16_t*>(yw), idx, E, static_cast<const bf16_t*>(residual), T, H / 8, k,
+      hipLaunchKernelGGL(combine_bf16x8_kernel, dim3(g8), dim3(256), 0, s, static_cast<const bf16_t*>(yw), a, T, H / 8, k,
                          static_cast<bf16_t*>(out));
     } else
       hipLaunchKernelGGL((combine_kernel<bf16_t, bf16_t>), dim3(grid), dim3(256), 0, s,
-                         static_cast<const bf16_t*>(yw), idx, E, static_cast<const bf16_t*>(residual), T, H, k,
-                         static_cast<bf16_t*>(out));
+                         static_cast<const bf16_t*>(yw), a, T, H, k, static_cast<bf16_t*>(out));
   } else if (dtype == BIBO_DTYPE_BF16) {
-    hipLaunchKernelGGL((combine_kernel<float, bf16_t>), dim3(grid), dim3(256), 0, s, static_cast<const float*>(yw), idx,
-                       E, static_cast<const bf16_t*>(residual), T, H, k, static_cast<bf16_t*>(out));
+    hipLaunchKernelGGL((combine_kernel<float, bf16_t>), dim3(grid), dim3(256), 0, s, static_cast<const float*>(yw), a, T,
+                       H, k, static_cast<bf16_t*>(out));
   } else {
-    hipLaunchKernelGGL((combine_kernel<float, float>), dim3(grid), dim3(256), 0, s, static_cast<const float*>(yw), idx,
-                       E, static_cast<const float*>(residual), T, H, k, static_cast<float*>(out));
+    hipLaunchKernelGGL((combine_kernel<float, float>), dim3(grid), dim3(256), 0, s, static_cast<const float*>(yw), a, T,
+                       H, k, static_cast<float*>(out));
   }
   return hipGetLastError();
 }

@@ -115,10 +115,10 @@ class BiBoFusedExperts(nn.Module):
         self.pos_end = self.pos_start + num_pos
         self.neg_start = self.pos_end
         self.neg_end = self.neg_start + num_neg
-        if self.num_glu_experts != self.num_routed_experts:
-            raise NotImplementedError(
-                "+/-Identity special experts are not implemented by the HIP kernels: configure "
-                "special_expert_pairs=0 (num_glu_experts must equal num_routed_experts)")
+        self.num_pos, self.num_neg = num_pos, num_neg
+        if self.neg_end != self.num_routed_experts:
+            raise ValueError(f"{self.num_glu_experts} GLU + {num_pos} +Identity + {num_neg} -Identity experts do not add "
+                             f"up to num_routed_experts={self.num_routed_experts}")
         if self.num_routed_experts > L.MAX_EXPERTS:
             raise NotImplementedError(f"the HIP kernels support at most {L.MAX_EXPERTS} experts")
         std = getattr(config, "initializer_range", 0.02)
@@ -144,9 +144,29 @@ class BiBoFusedExperts(nn.Module):
         idx = top_k_indices.detach().to(torch.int32).contiguous()
         w = top_k_weights.detach().to(torch.float32).contiguous()
         gu, dn, th = self._weights(cd)
-        out, counts = ops.experts_fwd(x, idx, w, gu, dn, th, algo=self.algo, want_counts=_want_counts)
+        out, counts = ops.experts_fwd(x, idx, w, gu, dn, th, algo=self.algo, want_counts=_want_counts,
+                                      n_pos=self.num_pos, n_neg=self.num_neg)          # specials: moe.py:95-99
         out = out if out.dtype == hidden_states.dtype else out.to(hidden_states.dtype)   # moe.py:101
         return (out, counts) if _want_counts else out
+
+
+class BiBoSharedMLP(nn.Module):
+    """The shared expert: BiBoMLP (src/modeling/ffn/mlp.py:9-35) at width moe_intermediate_size * num_shared_experts;
+    same parameter names, so `shared_experts_list.0.*` of a reference checkpoint loads."""
+
+    def __init__(self, config, intermediate_size):
+        super().__init__()
+        act = getattr(config, "hidden_act", "silu")
+        if act != "silu":
+            raise NotImplementedError(f"shared expert with hidden_act={act!r}; only 'silu' is implemented")
+        self.hidden_size = config.hidden_size
+        self.intermediate_size = intermediate_size
+        self.gate_proj = nn.Linear(self.hidden_size, intermediate_size, bias=False)
+        self.up_proj = nn.Linear(self.hidden_size, intermediate_size, bias=False)
+        self.down_proj = nn.Linear(intermediate_size, self.hidden_size, bias=False)
+
+    def forward(self, x):
+        return self.down_proj(nn.functional.silu(self.gate_proj(x)) * self.up_proj(x))         # mlp.py:34-35
 
 
 class BiBoMoELayer(nn.Module):
@@ -166,7 +186,12 @@ class BiBoMoELayer(nn.Module):
         self.use_shared_expert = getattr(config, "use_shared_expert", False)
         self.shared_experts_list = nn.ModuleList()
         if self.use_shared_expert:
-            raise NotImplementedError("use_shared_expert=True is not implemented by the HIP MoE layer")
+            # moe.py:118-127.  The shared expert is a dense SwiGLU over every token: stock GEMMs, not part of the
+            # sparse path, so it runs as ordinary tensor operations next to the library call.
+            if getattr(config, "shared_expert_type", "mlp") != "mlp":
+                raise NotImplementedError("shared_expert_type='conv' is not implemented; use 'mlp'")
+            n_sh = int(getattr(config, "num_shared_experts", 1))
+            self.shared_experts_list.append(BiBoSharedMLP(config, config.moe_intermediate_size * n_sh))
         self.gate = BiBoMoERouter(config)
 
     # ---- balancing (host logic over device tensors, moe.py:131-155) ----
@@ -228,14 +253,18 @@ class BiBoMoELayer(nn.Module):
             b = self.gate._cache.get("b", self.gate.bias, torch.float32)
             out, _, _, counts, _ = ops.moe_forward(x, wr, b, gu, dn, th, self.num_experts_per_tok,
                                                    norm=self.gate.norm_topk_prob, algo=self.experts.algo,
-                                                   want_counts=balancing)
+                                                   want_counts=balancing, n_pos=self.experts.num_pos,
+                                                   n_neg=self.experts.num_neg)
             out = out if out.dtype == hidden_states.dtype else out.to(hidden_states.dtype)
             top_idx = None
+        out = out.view(bsz, seq, hdim)
+        if self.use_shared_expert:                             # moe.py:174-176
+            out = out + self.shared_experts_list[0](hidden_states).to(out.dtype)
         if balancing:                                          # exactly once per training forward
             tpe = self._balance_step(top_idx, num_tokens, counts=counts)
             if tpe is not None:
                 self.update_bias(tpe)
-        return out.view(bsz, seq, hdim)
+        return out
 
     @_no_compile
     def ffn_forward(self, hidden_states: torch.Tensor, norm_weight: torch.Tensor, eps: float,
@@ -248,7 +277,7 @@ class BiBoMoELayer(nn.Module):
         around it."""
         bsz, seq, hdim = hidden_states.shape
         num_tokens = bsz * seq
-        if self._hooks_present() or hidden_states.dtype != _compute_dtype(hidden_states):
+        if self._hooks_present() or self.use_shared_expert or hidden_states.dtype != _compute_dtype(hidden_states):
             # (an fp32 residual stream under bf16 autocast keeps its fp32 norm and fp32 residual add)
             xf = hidden_states.float()
             xn = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)).to(hidden_states.dtype)    # norm.py:21-24
@@ -264,7 +293,8 @@ class BiBoMoELayer(nn.Module):
         b = self.gate._cache.get("b", self.gate.bias, torch.float32)
         nw = norm_weight.detach().float().contiguous()
         out, _, _, counts = ops.ffn_forward(h, nw, float(eps), wr, b, gu, dn, th, self.num_experts_per_tok,
-                                            norm=self.gate.norm_topk_prob, algo=self.experts.algo, want_counts=balancing)
+                                            norm=self.gate.norm_topk_prob, algo=self.experts.algo, want_counts=balancing,
+                                            n_pos=self.experts.num_pos, n_neg=self.experts.num_neg)
         if balancing:                                          # exactly once per training forward
             tpe = self._balance_step(None, num_tokens, counts=counts)
             if tpe is not None:

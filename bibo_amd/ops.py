@@ -160,36 +160,50 @@ def gateup_down_fwd(x, w_gate_up, w_down, theta, w, offsets, perm_slot, perm_tok
     return yw
 
 
-def combine_fwd(yw, T, k, dtype=None):
-    """out[t] = sum_j yw[t*k + j] in fp32, rounded once -> [T,H] in `dtype` (default: yw.dtype)."""
+def combine_fwd(yw, T, k, dtype=None, idx=None, w=None, x=None, n_glu=0, n_pos=0, n_neg=0, residual=None):
+    """out[t] = residual[t] + sum_j contribution(t, j) in fp32, rounded once -> [T,H] in `dtype` (default: yw.dtype).
+    contribution = yw[t*k + j]; with idx (and w, x) given, +/- w[t,j] * x[t] for the +/-Identity specials and nothing
+    for an index outside [0, n_glu + n_pos + n_neg)."""
     H = yw.shape[1]
     dtype = dtype or yw.dtype
     _chk(yw, "yw", None, (T * k, H))
     if yw.dtype not in (torch.bfloat16, torch.float32):
         raise TypeError("yw must be bf16 or fp32")
+    for t_, n_, d_, sh_ in ((idx, "idx", torch.int32, (T, k)), (w, "w", torch.float32, (T, k)), (x, "x", dtype, (T, H)),
+                            (residual, "residual", dtype, (T, H))):
+        if t_ is not None:
+            _chk(t_, n_, d_, sh_)
     out = torch.empty(T, H, dtype=dtype, device=yw.device)
     dc = L.DTYPE_BF16 if dtype == torch.bfloat16 else L.DTYPE_F32
     with torch.cuda.device(yw.device):
-        L.check(L.lib().bibo_moe_combine_fwd(_ptr(yw), int(yw.dtype == torch.bfloat16), T, H, k, dc, _ptr(out),
-                                             _stream(yw.device)), "bibo_moe_combine_fwd")
+        if idx is None and residual is None:
+            L.check(L.lib().bibo_moe_combine_fwd(_ptr(yw), int(yw.dtype == torch.bfloat16), T, H, k, dc, _ptr(out),
+                                                 _stream(yw.device)), "bibo_moe_combine_fwd")
+        else:
+            L.check(L.lib().bibo_moe_combine_ex_fwd(_ptr(yw), int(yw.dtype == torch.bfloat16), _ptr(idx), _ptr(w), _ptr(x),
+                                                    n_glu, n_pos, n_neg, _ptr(residual), T, H, k, dc, _ptr(out),
+                                                    _stream(yw.device)), "bibo_moe_combine_ex_fwd")
     return out
 
 
-def experts_fwd(x, idx, w, w_gate_up, w_down, theta, algo="auto", want_counts=False):
-    """Seam 2.  x [T,H]; idx int32 [T,k]; w fp32 [T,k] -> out [T,H] (x.dtype), counts int32 [E]|None."""
+def experts_fwd(x, idx, w, w_gate_up, w_down, theta, algo="auto", want_counts=False, n_pos=0, n_neg=0):
+    """Seam 2.  x [T,H]; idx int32 [T,k]; w fp32 [T,k] -> out [T,H] (x.dtype), counts int32 [E]|None.
+    The weight tensors hold the GLU experts; expert ids Eg .. Eg+n_pos-1 are +Identity, the next n_neg -Identity
+    specials (moe.py:39-44,95-99), and E = Eg + n_pos + n_neg."""
     T, H = x.shape
-    E, two_i, _ = w_gate_up.shape
+    Eg, two_i, _ = w_gate_up.shape
+    E = Eg + n_pos + n_neg
     I = two_i // 2
     k = idx.shape[1]
     dc = _dtype_code(x)
     _chk(x, "x"); _chk(idx, "idx", torch.int32, (T, k)); _chk(w, "w", torch.float32, (T, k))
-    _chk(w_gate_up, "w_gate_up", x.dtype, (E, 2 * I, H)); _chk(w_down, "w_down", x.dtype, (E, H, I))
-    _chk(theta, "theta", torch.float32, (E,))
+    _chk(w_gate_up, "w_gate_up", x.dtype, (Eg, 2 * I, H)); _chk(w_down, "w_down", x.dtype, (Eg, H, I))
+    _chk(theta, "theta", torch.float32, (Eg,))
     dev = x.device
     out = torch.empty(T, H, dtype=x.dtype, device=dev)
     counts = torch.empty(E, dtype=torch.int32, device=dev) if want_counts else None
     ws = workspace(dev, workspace_bytes(T, H, E, k, I, dc))
-    sh = L.Shape(T, H, E, k, I, dc)
+    sh = L.Shape(T, H, E, k, I, dc, n_pos, n_neg)
     with torch.cuda.device(dev):
         L.check(L.lib().bibo_moe_experts_fwd(_ptr(x), _ptr(idx), _ptr(w), _ptr(w_gate_up), _ptr(w_down), _ptr(theta),
                                              ctypes.byref(sh), algo_code(algo), _ptr(out), _ptr(counts), _ptr(ws),
@@ -198,15 +212,17 @@ def experts_fwd(x, idx, w, w_gate_up, w_down, theta, algo="auto", want_counts=Fa
 
 
 def moe_forward(x, w_router, bias, w_gate_up, w_down, theta, k, norm="sum", algo="auto", want_routing=False,
-                want_counts=False, want_logits=False):
-    """Seam 1.  -> out [T,H], idx int32 [T,k]|None, w fp32 [T,k]|None, counts int32 [E]|None, logits fp32 [T,E]|None."""
+                want_counts=False, want_logits=False, n_pos=0, n_neg=0):
+    """Seam 1.  -> out [T,H], idx int32 [T,k]|None, w fp32 [T,k]|None, counts int32 [E]|None, logits fp32 [T,E]|None.
+    w_router / bias have E = Eg + n_pos + n_neg rows, the expert weights Eg (see experts_fwd)."""
     T, H = x.shape
-    E, two_i, _ = w_gate_up.shape
+    Eg, two_i, _ = w_gate_up.shape
+    E = Eg + n_pos + n_neg
     I = two_i // 2
     dc = _dtype_code(x)
     _chk(x, "x"); _chk(w_router, "w_router", x.dtype, (E, H)); _chk(bias, "bias", torch.float32, (E,))
-    _chk(w_gate_up, "w_gate_up", x.dtype, (E, 2 * I, H)); _chk(w_down, "w_down", x.dtype, (E, H, I))
-    _chk(theta, "theta", torch.float32, (E,))
+    _chk(w_gate_up, "w_gate_up", x.dtype, (Eg, 2 * I, H)); _chk(w_down, "w_down", x.dtype, (Eg, H, I))
+    _chk(theta, "theta", torch.float32, (Eg,))
     dev = x.device
     out = torch.empty(T, H, dtype=x.dtype, device=dev)
     idx = torch.empty(T, k, dtype=torch.int32, device=dev) if want_routing else None
@@ -214,7 +230,7 @@ def moe_forward(x, w_router, bias, w_gate_up, w_down, theta, k, norm="sum", algo
     counts = torch.empty(E, dtype=torch.int32, device=dev) if want_counts else None
     logits = torch.empty(T, E, dtype=torch.float32, device=dev) if want_logits else None
     ws = workspace(dev, workspace_bytes(T, H, E, k, I, dc))
-    sh = L.Shape(T, H, E, k, I, dc)
+    sh = L.Shape(T, H, E, k, I, dc, n_pos, n_neg)
     with torch.cuda.device(dev):
         L.check(L.lib().bibo_moe_forward(_ptr(x), _ptr(w_router), _ptr(bias), _ptr(w_gate_up), _ptr(w_down),
                                          _ptr(theta), ctypes.byref(sh), norm_mode(norm), algo_code(algo), _ptr(out),
@@ -235,21 +251,22 @@ def rmsnorm_fwd(x, norm_weight, eps):
 
 
 def ffn_forward(h, norm_weight, eps, w_router, bias, w_gate_up, w_down, theta, k, norm="sum", algo="auto",
-                want_routing=False, want_counts=False):
+                want_routing=False, want_counts=False, n_pos=0, n_neg=0):
     """Seam 3 (the block's caller).  -> out = h + moe(rmsnorm(h)) [T,H], idx|None, w|None, counts|None."""
     T, H = h.shape
-    E, two_i, _ = w_gate_up.shape
+    Eg, two_i, _ = w_gate_up.shape
+    E = Eg + n_pos + n_neg
     I = two_i // 2
     dc = _dtype_code(h)
     _chk(h, "h"); _chk(norm_weight, "norm_weight", torch.float32, (H,)); _chk(w_router, "w_router", h.dtype, (E, H))
-    _chk(bias, "bias", torch.float32, (E,)); _chk(w_gate_up, "w_gate_up", h.dtype, (E, 2 * I, H))
-    _chk(w_down, "w_down", h.dtype, (E, H, I)); _chk(theta, "theta", torch.float32, (E,))
+    _chk(bias, "bias", torch.float32, (E,)); _chk(w_gate_up, "w_gate_up", h.dtype, (Eg, 2 * I, H))
+    _chk(w_down, "w_down", h.dtype, (Eg, H, I)); _chk(theta, "theta", torch.float32, (Eg,))
     dev = h.device
     out = torch.empty(T, H, dtype=h.dtype, device=dev)
     idx = torch.empty(T, k, dtype=torch.int32, device=dev) if want_routing else None
     w = torch.empty(T, k, dtype=torch.float32, device=dev) if want_routing else None
     counts = torch.empty(E, dtype=torch.int32, device=dev) if want_counts else None
-    sh = L.Shape(T, H, E, k, I, dc)
+    sh = L.Shape(T, H, E, k, I, dc, n_pos, n_neg)
     nbytes = ctypes.c_size_t(0)
     L.check(L.lib().bibo_moe_ffn_workspace_bytes(ctypes.byref(sh), ctypes.byref(nbytes)), "bibo_moe_ffn_workspace_bytes")
     ws = workspace(dev, nbytes.value)

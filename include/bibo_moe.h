@@ -37,7 +37,7 @@
 extern "C" {
 #endif
 
-#define BIBO_MOE_ABI_VERSION 1
+#define BIBO_MOE_ABI_VERSION 2
 #define BIBO_MOE_MAX_EXPERTS 64
 #define BIBO_MOE_MAX_TOPK 8
 
@@ -71,11 +71,13 @@ enum bibo_error {
 typedef struct bibo_moe_shape {
   int32_t T; /* tokens = B*S */
   int32_t H; /* hidden size */
-  int32_t E; /* routed experts (all GLU) */
+  int32_t E; /* routed experts = rows of w_router: GLU experts first, then +Identity, then -Identity */
   int32_t k; /* experts per token */
   int32_t I; /* expert intermediate size */
   int32_t dtype;
-} bibo_moe_shape;
+  int32_t n_pos; /* +Identity specials (moe.py:39-44,95-96): out += w * x; usually 0 */
+  int32_t n_neg; /* -Identity specials (moe.py:97-99): out -= w * x; usually 0 */
+} bibo_moe_shape; /* w_gate_up, w_down and theta hold E - n_pos - n_neg (GLU) experts */
 
 int bibo_moe_abi_version(void);
 
@@ -148,6 +150,16 @@ int bibo_moe_gateup_down_fwd(const void* x, const void* w_gate_up, const void* w
  * `dtype` must be bf16), fp32 otherwise; out [T,H] in `dtype`.
  */
 int bibo_moe_combine_fwd(const void* yw, int yw_is_bf16, int T, int H, int k, int dtype, void* out, void* stream);
+
+/*
+ * The same sum with everything the composite entry points fold into it (each pointer may be NULL):
+ *   idx int32 [T,k], E_glu, n_pos, n_neg: slots with idx outside [0, E_glu+n_pos+n_neg) are skipped, slots of a
+ *   +/-Identity special add +/- w[slot] * x[t, :] instead of a row of yw (moe.py:95-99; needs w fp32 [T,k] and
+ *   x [T,H] in `dtype`);  residual [T,H] in `dtype` is added before the rounding (layers.py:62-64).
+ */
+int bibo_moe_combine_ex_fwd(const void* yw, int yw_is_bf16, const int32_t* idx, const float* w, const void* x,
+                            int E_glu, int n_pos, int n_neg, const void* residual, int T, int H, int k, int dtype,
+                            void* out, void* stream);
 
 /*
  * Seam 2: BiBoFusedExperts.forward(x, idx, w) (moe.py:46-101; the signature of the external

@@ -155,18 +155,20 @@ def expert_hidden(x_rows: torch.Tensor, w_gate_up_e: torch.Tensor, theta_e: torc
     return radial_normsilu(gate, theta_e) * up
 
 
-def experts_forward(x, idx, w, w_gate_up, w_down, theta, dtype=torch.float32, return_hidden=False):
-    """Weighted sum over each token's experts, evaluated in `dtype` (moe.py:46-101, GLU branch).
+def experts_forward(x, idx, w, w_gate_up, w_down, theta, dtype=torch.float32, return_hidden=False, n_pos=0, n_neg=0):
+    """Weighted sum over each token's experts, evaluated in `dtype` (moe.py:46-101).
 
-    x [T,H]; idx [T,k] integer; w [T,k]; w_gate_up [E,2I,H]; w_down [E,H,I]; theta [E].
-    Returns [T,H] in `dtype` (the caller rounds to the model dtype, moe.py:101).  With
-    return_hidden=True also returns the [S,I] activations in canonical sorted-row order.
+    x [T,H]; idx [T,k] integer; w [T,k]; w_gate_up [Eg,2I,H]; w_down [Eg,H,I]; theta [Eg] hold the GLU experts;
+    expert ids Eg .. Eg+n_pos-1 are +Identity (out += w*x, moe.py:95-96), the next n_neg -Identity (out -= w*x,
+    moe.py:98-99).  Returns [T,H] in `dtype` (the caller rounds to the model dtype, moe.py:101).  With
+    return_hidden=True also returns the [S,I] activations of the GLU rows in canonical sorted-row order.
     """
     x = x.to(dtype)
     idx_np = idx.cpu().numpy() if isinstance(idx, torch.Tensor) else np.asarray(idx)
     w_t = (w if isinstance(w, torch.Tensor) else torch.from_numpy(np.asarray(w))).to(dtype)
     T, H = x.shape
-    E = w_gate_up.shape[0]
+    Eg = w_gate_up.shape[0]
+    E = Eg + n_pos + n_neg
     k = idx_np.shape[1]
     counts, offsets, perm_slot, perm_token = permute(idx_np, E)
     out = torch.zeros(T, H, dtype=dtype)
@@ -178,6 +180,10 @@ def experts_forward(x, idx, w, w_gate_up, w_down, theta, dtype=torch.float32, re
             continue
         tok = torch.from_numpy(perm_token[lo:hi].astype(np.int64))
         slot = torch.from_numpy(perm_slot[lo:hi].astype(np.int64))
+        if e >= Eg:                                                           # moe.py:95-99
+            sign = 1.0 if e < Eg + n_pos else -1.0
+            out.index_add_(0, tok, x[tok] * (sign * w_flat[slot]).unsqueeze(-1))
+            continue
         h = expert_hidden(x[tok], w_gate_up[e].to(dtype), theta[e])
         if return_hidden:
             hidden[lo:hi] = h
@@ -186,15 +192,22 @@ def experts_forward(x, idx, w, w_gate_up, w_down, theta, dtype=torch.float32, re
     return (out, hidden) if return_hidden else out
 
 
-def moe_forward(x, w_router, bias, w_gate_up, w_down, theta, k, dtype=torch.float32, logits=None):
+def moe_forward(x, w_router, bias, w_gate_up, w_down, theta, k, dtype=torch.float32, logits=None, n_pos=0, n_neg=0):
     """Whole layer (moe.py:157-183, eval mode, no shared expert).  If `logits` is given the
     routing is computed from them (the parity protocol: same fp32 logits on both sides)."""
     if logits is None:
         logits = router_logits(x, w_router)
     b = bias.detach().float().numpy() if isinstance(bias, torch.Tensor) else bias
     idx, w, _ = route_from_logits(logits, b, k)
-    out = experts_forward(x, idx, w, w_gate_up, w_down, theta, dtype=dtype)
+    out = experts_forward(x, idx, w, w_gate_up, w_down, theta, dtype=dtype, n_pos=n_pos, n_neg=n_neg)
     return out, idx, w
+
+
+def shared_mlp(x, w_gate, w_up, w_down):
+    """The shared expert, BiBoMLP.forward (src/modeling/ffn/mlp.py:34-35) with hidden_act = silu:
+    down(silu(gate(x)) * up(x)); added to the routed output by the layer (moe.py:174-176).  fp32."""
+    xf = x.float()
+    return (F.silu(xf @ w_gate.float().t()) * (xf @ w_up.float().t())) @ w_down.float().t()
 
 
 # --------------------------------------------------------------------------------------

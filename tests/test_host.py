@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
     lib = L.lib()
     for name in declared:
         assert hasattr(lib, name)
-    assert lib.bibo_moe_abi_version() == 1
+    assert lib.bibo_moe_abi_version() == L.ABI_VERSION == 2
 
 
 def test_argument_errors_are_reported_without_a_gpu():
@@ -106,10 +106,30 @@ def test_state_dict_layout_matches_the_reference_layer():
 
 
 def test_unsupported_configurations_raise():
-    with pytest.raises(NotImplementedError, match="Identity"):
-        bibo_amd.BiBoMoELayer(make_config(special_expert_pairs=1))
-    with pytest.raises(NotImplementedError, match="shared"):
-        bibo_amd.BiBoMoELayer(make_config(use_shared_expert=True))
+    with pytest.raises(NotImplementedError, match="conv"):
+        bibo_amd.BiBoMoELayer(make_config(use_shared_expert=True, shared_expert_type="conv"))
+    with pytest.raises(NotImplementedError, match="hidden_act"):
+        bibo_amd.BiBoMoELayer(make_config(use_shared_expert=True, hidden_act="gelu"))
+    with pytest.raises(ValueError, match="GLU"):
+        make_config(num_routed_experts=4, num_pos_identity_experts=2, num_neg_identity_experts=2)
+
+
+def test_specials_and_shared_expert_follow_the_reference_layout():
+    """moe.py:19-44,118-127: the weight tensors hold only the GLU experts, the router has a row per routed expert
+    (specials included), the shared expert is a SwiGLU of width moe_intermediate_size * num_shared_experts."""
+    layer = bibo_amd.BiBoMoELayer(make_config(num_routed_experts=8, special_expert_pairs=1, use_shared_expert=True,
+                                              num_shared_experts=2))
+    e = layer.experts
+    assert (e.num_glu_experts, e.pos_start, e.pos_end, e.neg_start, e.neg_end) == (6, 6, 7, 7, 8)
+    sd = layer.state_dict()
+    assert sd["experts.gate_up_proj"].shape == (6, 192, 64) and sd["experts.down_proj"].shape == (6, 64, 96)
+    assert sd["experts.radial_theta"].shape == (6,) and sd["gate.gate_proj.weight"].shape == (8, 64)
+    assert sd["gate.bias"].shape == (8,) and sd["accumulated_tpe"].shape == (8,)
+    assert sd["shared_experts_list.0.gate_proj.weight"].shape == (192, 64)
+    assert sd["shared_experts_list.0.up_proj.weight"].shape == (192, 64)
+    assert sd["shared_experts_list.0.down_proj.weight"].shape == (64, 192)
+    asym = bibo_amd.BiBoMoELayer(make_config(num_routed_experts=8, num_pos_identity_experts=3, num_neg_identity_experts=0))
+    assert (asym.experts.num_glu_experts, asym.experts.pos_end, asym.experts.neg_end) == (5, 8, 8)
 
 
 def test_forward_refuses_to_drop_gradients():

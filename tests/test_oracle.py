@@ -289,3 +289,32 @@ def test_ffn_forward_is_residual_plus_block_of_the_normalised_input():
     out0, *_ = O.ffn_forward(p["x"], wgt, 1e-6, p["w_router"], p["bias"], p["w_gate_up"], torch.zeros_like(p["w_down"]),
                              p["theta"], 2)
     assert torch.equal(out0, p["x"])
+
+
+# ------------------------------------------------------------------ +/-Identity specials and the shared expert
+def test_identity_specials_add_and_subtract_the_weighted_input():
+    """moe.py:95-99.  A token routed only to a +Identity expert comes back as w*x, to a -Identity expert as -w*x;
+    mixed with a GLU expert the contributions add; a +/- pair with equal weights cancels."""
+    p = O.make_inputs(T=6, H=16, E=4, k=2, I=8, theta="normal", seed=2, dtype=torch.float32)
+    x, gu, dn, th = p["x"], p["w_gate_up"], p["w_down"], p["theta"]          # 4 GLU experts; ids 4,5 = +I, 6 = -I
+    w = np.full((6, 2), 0.25, np.float32)
+    w[:, 1] = 0.5
+    only_pos = O.experts_forward(x, np.tile([[4, 5]], (6, 1)), w, gu, dn, th, n_pos=2, n_neg=1)
+    assert torch.allclose(only_pos, 0.75 * x, atol=1e-6)
+    only_neg = O.experts_forward(x, np.tile([[6, 6]], (6, 1)), w, gu, dn, th, n_pos=2, n_neg=1)
+    assert torch.allclose(only_neg, -0.75 * x, atol=1e-6)
+    cancel = O.experts_forward(x, np.tile([[5, 6]], (6, 1)), np.full((6, 2), 0.3, np.float32), gu, dn, th, n_pos=2, n_neg=1)
+    assert torch.allclose(cancel, torch.zeros_like(x), atol=1e-6)
+    glu_only = O.experts_forward(x, np.tile([[1, 1]], (6, 1)), np.stack([w[:, 0], 0 * w[:, 1]], 1), gu, dn, th)
+    mixed = O.experts_forward(x, np.tile([[1, 6]], (6, 1)), w, gu, dn, th, n_pos=2, n_neg=1)
+    assert torch.allclose(mixed, glu_only - 0.5 * x, atol=1e-5)
+
+
+def test_shared_mlp_is_a_swiglu():
+    g = torch.Generator().manual_seed(3)
+    x, wg, wu, wd = (torch.randn(5, 12, generator=g), torch.randn(20, 12, generator=g), torch.randn(20, 12, generator=g),
+                     torch.randn(12, 20, generator=g))
+    got = O.shared_mlp(x, wg, wu, wd)
+    a = x.double() @ wg.double().t()
+    want = ((a / (1 + torch.exp(-a))) * (x.double() @ wu.double().t())) @ wd.double().t()
+    assert torch.allclose(got.double(), want, rtol=1e-4, atol=1e-4)
