@@ -110,3 +110,31 @@ def test_layer_with_default_style_config_specials_and_shared_expert():
         xf32 = x.float()
         xn = (xf32 * torch.rsqrt(xf32.pow(2).mean(-1, keepdim=True) + 1e-6)).bfloat16()
         assert rel_err(seam.cpu(), (x + layer(nw * xn)).cpu().float()) <= 1e-2
+
+
+def test_reference_tiny_config_six_glu_plus_identity_pair():
+    """The reference's own test configuration (tests/conftest.py:30-43 there): H=64, 8 routed experts = 6 GLU + one
+    +/-Identity pair, k=2.  Same checks as its tests/test_moe.py:81-126,138-145: router weights positive and
+    summing to one, indices in range, the layer equal to the oracle, and a bias that forces the specials gives
+    out = (w_pos - w_neg) * x."""
+    torch.manual_seed(0)
+    cfg = bibo_amd.BiBoMoEConfig(hidden_size=64, intermediate_size=96, moe_intermediate_size=96, num_routed_experts=8,
+                                 special_expert_pairs=1, num_experts_per_tok=2)
+    layer = bibo_amd.BiBoMoELayer(cfg).to(DEV).eval()                # fp32 module: generic kernels
+    x = torch.randn(2, 33, 64, device=DEV)
+    with torch.no_grad():
+        out = layer(x)
+        idx, w = layer.gate(x)
+    assert idx.dtype == torch.int64 and w.dtype == torch.float32 and idx.min() >= 0 and idx.max() < 8
+    assert (w > 0).all() and torch.allclose(w.sum(-1), torch.ones_like(w.sum(-1)), atol=1e-6)
+    sd = {k_: v.detach().cpu() for k_, v in layer.state_dict().items()}
+    ref = O.experts_forward(x.cpu().reshape(-1, 64), idx.cpu().reshape(-1, 2).numpy(), w.cpu().reshape(-1, 2).numpy(),
+                            sd["experts.gate_up_proj"], sd["experts.down_proj"], sd["experts.radial_theta"], n_pos=1,
+                            n_neg=1)
+    assert rel_err(out.cpu().reshape(-1, 64), ref) <= 1e-5
+    with torch.no_grad():
+        layer.gate.bias[6:] += 5.0                                  # selection only: both specials always win
+        out2 = layer(x)
+        idx2, w2 = layer.gate(x)
+    assert (idx2 == torch.tensor([6, 7], device=DEV)).all()
+    assert torch.allclose(out2, (w2[..., :1] - w2[..., 1:]) * x, atol=1e-6)
