@@ -74,8 +74,8 @@ Workspace carve(int T, int H, int E, int k, int I, int dtype) {
   ws.perm_slot = o;  o += align_up(S * sizeof(int32_t));
   ws.perm_token = o; o += align_up(S * sizeof(int32_t));
   ws.hidden = o;     o += align_up(S * (size_t)I * elt_size(dtype));
-  // fp32 gate/up pre-activations, only ever used when the streaming kernels are eligible
-  ws.gu = o;         o += align_up(stream_eligible(T, H, E, k, I, dtype) ? S * (size_t)2 * I * sizeof(float) : 0);
+  // bf16 gate/up pre-activations, only ever used when the streaming kernels are eligible
+  ws.gu = o;         o += align_up(stream_eligible(T, H, E, k, I, dtype) ? S * (size_t)2 * I * sizeof(bf16_t) : 0);
   ws.yw = o;         o += align_up(S * (size_t)H * sizeof(float));
   ws.total = o;
   return ws;
@@ -126,7 +126,7 @@ int experts_dispatch(const void* x, const void* wgu, const void* wd, const float
   if (algo == BIBO_ALGO_STREAM) {
     if (!aligned16(x) || !aligned16(wgu) || !aligned16(wd)) return BIBO_ERR_MISALIGNED;
     if (!stream_eligible(T, H, Eg + np + nn, k, I, dtype)) return BIBO_ERR_UNSUPPORTED;   // no pre-activation segment carved
-    float* gu = reinterpret_cast<float*>(base + ws.gu);
+    void* gu = base + ws.gu;
     hipError_t e = launch_gateup_stream(x, wgu, idx, T, H, Eg, k, I, gu, s);
     if (e != hipSuccess) return (int)e;
     e = launch_down_stream(gu, wd, theta, w, idx, T, H, Eg, k, I, base + ws.hidden, yw, s);

@@ -151,8 +151,8 @@ hipError_t launch_experts_fused(const void* x, const void* wgu, const void* wd, 
                                 int H, int E, int k, int I, void* yw, hipStream_t s);
 bool stream_supported(int H, int I, int dtype);
 hipError_t launch_gateup_stream(const void* x, const void* wgu, const int32_t* idx, int T, int H, int E, int k, int I,
-                                float* gu, hipStream_t s);
-hipError_t launch_down_stream(const float* gu, const void* wd, const float* theta, const float* w, const int32_t* idx,
+                                void* gu, hipStream_t s);
+hipError_t launch_down_stream(const void* gu, const void* wd, const float* theta, const float* w, const int32_t* idx,
                               int T, int H, int E, int k, int I, void* hidden, float* yw, hipStream_t s);
 
 }  // namespace bibo

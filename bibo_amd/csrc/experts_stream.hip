@@ -12,10 +12,18 @@
 // 32 contiguous bytes [32g, 32g+32) of every 128-byte line of weight row r, so four lanes consume a
 // whole line; the token operand, staged in LDS, is read with the same K permutation.
 //
-//   gateup_stream_kernel : raw gate/up pre-activations  gu[slot, 0..2I) fp32  (src/modeling/ffn/moe.py:84)
-//   activate_rows_kernel : hidden[slot] = r^p SiLU(g/r) up; needs the whole gate row, which no single
-//                          gate/up workgroup has, hence its own tiny launch    (moe.py:87-92)
-//   down_stream_kernel   : streams w_down and writes routing-weighted rows in slot order (moe.py:92-93)
+// Order of the memory requests.  A CU serves its vector loads first in, first out, and its share of the
+// HBM rate is about 23 GB/s, so a small load issued behind 64 KB of weight requests waits about 3 us for
+// them (and behind 192 KB about 8 us).  Every small load the multiplication depends on is therefore issued
+// AHEAD of the weights it would otherwise queue behind: the routing indices before the first weight
+// chunk, the operand rows before the second, and only as much weight data is requested in between as the
+// dependent work (finding the rows) takes to complete.
+//
+//   gateup_stream_kernel : raw gate/up pre-activations gu[slot, 0..2I) bf16        (src/modeling/ffn/moe.py:84)
+//   down_stream_kernel   : streams w_down and writes routing-weighted rows in slot order (moe.py:92-93);
+//                          for I <= 512 it also turns the expert's pre-activations into the operand rows,
+//                          hidden = r^p SiLU(g/r) up (moe.py:87-92), while the weights are on their way
+//   activate_rows_kernel : the same activation as a launch of its own, for wider I
 #include "common.h"
 
 namespace bibo {
@@ -25,26 +33,32 @@ constexpr int kRowsPerWave = 16;
 constexpr int kRowsPerWg = 64;     // weight rows per workgroup
 constexpr int kTok = 16;           // routed rows multiplied per pass
 constexpr int kLine = 64;          // bf16 elements per 128-byte line
-
 constexpr int kChunk = 4;          // 128-byte lines per register chunk (two chunks are alive: 64 VGPRs)
 constexpr int kScan = kStreamMaxSlots / 256;   // routing indices each thread inspects
+constexpr int kFusedActMaxI = 512; // widest I whose activation the down kernel computes itself
 
-// Slots routed to expert e, ascending, into rows_s; returns how many.  All 256 threads call it; slot
-// s = 256*q + tid, so slot order is (q, wave, lane).  Ends with a barrier.
-__device__ __forceinline__ int expert_rows(const int32_t* __restrict__ idx, int S, int e, unsigned short* rows_s,
-                                           int* cnt_s) {
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const unsigned long long lt = (1ull << lane) - 1ull;
+struct ScanRegs {
   int v[kScan];
+};
+
+// request this thread's routing indices: slot s = 256*q + tid, so slot order is (q, wave, lane)
+__device__ __forceinline__ void scan_issue(ScanRegs& r, const int32_t* __restrict__ idx, int S) {
 #pragma unroll
   for (int q = 0; q < kScan; ++q) {
-    const int s = q * 256 + tid;
-    v[q] = (s < S) ? idx[s] : -1;                               // all loads in flight together
+    const int s = q * 256 + threadIdx.x;
+    r.v[q] = (s < S) ? idx[s] : -1;                             // all loads in flight together
   }
+}
+
+// Slots routed to expert e, ascending, into rows_s; returns how many.  All 256 threads call it; ends with a
+// barrier.
+__device__ __forceinline__ int scan_finish(const ScanRegs& r, int e, unsigned short* rows_s, int* cnt_s) {
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const unsigned long long lt = (1ull << lane) - 1ull;
   int rank[kScan];
 #pragma unroll
   for (int q = 0; q < kScan; ++q) {
-    const unsigned long long b = __ballot(v[q] == e);
+    const unsigned long long b = __ballot(r.v[q] == e);
     rank[q] = __popcll(b & lt);
     if (lane == 0) cnt_s[q * 4 + wave] = __popcll(b);
   }
@@ -54,7 +68,7 @@ __device__ __forceinline__ int expert_rows(const int32_t* __restrict__ idx, int 
   for (int q = 0; q < kScan; ++q)
 #pragma unroll
     for (int ww = 0; ww < 4; ++ww) {
-      if (ww == wave && v[q] == e) rows_s[run + rank[q]] = (unsigned short)(q * 256 + tid);
+      if (ww == wave && r.v[q] == e) rows_s[run + rank[q]] = (unsigned short)(q * 256 + tid);
       run += cnt_s[q * 4 + ww];
     }
   __syncthreads();
@@ -65,46 +79,93 @@ struct WChunk {
   bf16x8 w0[kChunk], w1[kChunk];
 };
 
-// this lane's 32 bytes of lines l .. l+kChunk-1 of its weight row (lines past nlines are skipped)
+// this lane's 32 bytes of lines l .. l+kChunk-1 of its weight row.  kWhole: the row is a whole number of
+// chunks, and a chunk that starts past its end is skipped as a whole; otherwise line by line.
+template <bool kWhole>
 __device__ __forceinline__ void load_chunk(WChunk& c, const bf16_t* __restrict__ wp, int l, int nlines) {
+  if (kWhole && l >= nlines) return;
 #pragma unroll
   for (int u = 0; u < kChunk; ++u)
-    if (l + u < nlines) {
+    if (kWhole || l + u < nlines) {
       c.w0[u] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(wp + (l + u) * kLine));
       c.w1[u] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(wp + (l + u) * kLine + 8));
     }
 }
 
-// Stream kRowsPerWave weight rows (row stride K) against 16 token rows held in LDS `xs` (row stride K + 8
-// elements, so the 16 lanes of a fragment read hit distinct banks).  `first` already holds lines 0..kChunk-1
-// (loaded before the token rows were staged); each further chunk is requested one chunk ahead of its use.
-__device__ __forceinline__ floatx4 stream_rows(const bf16_t* __restrict__ wrow, const bf16_t* xs, int K, int lane,
-                                               const WChunk& first) {
-  const int g = lane >> 4;
-  const bf16_t* wp = wrow + g * 16;                            // this lane's 32 bytes of every line
-  const bf16_t* xp = xs + (lane & 15) * (K + 8) + g * 16;
+// Multiply kChunk lines (from line l) of the wave's weight rows, held in `c`, with the operand rows in LDS.
+template <bool kWhole>
+__device__ __forceinline__ void mul_chunk(floatx4& acc, const WChunk& c, const bf16_t* xp, int l, int nlines) {
+  if (kWhole && l >= nlines) return;
+#pragma unroll
+  for (int u = 0; u < kChunk; ++u)
+    if (kWhole || l + u < nlines) {
+      const bf16x8 x0 = *reinterpret_cast<const bf16x8*>(xp + (l + u) * kLine);
+      const bf16x8 x1 = *reinterpret_cast<const bf16x8*>(xp + (l + u) * kLine + 8);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(c.w0[u], x0, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(c.w1[u], x1, acc, 0, 0, 0);
+    }
+}
+
+// Stream kRowsPerWave weight rows (row stride K) against 16 operand rows held in LDS `xs` (row stride K + 8
+// elements, so the 16 lanes of a fragment read hit distinct banks).  On entry `a` and `b` hold lines
+// 0..kChunk-1 and kChunk..2*kChunk-1; each is refilled, two chunks ahead, as soon as it is consumed, so on
+// return they hold other lines.
+template <bool kWhole>
+__device__ __forceinline__ floatx4 stream_rows(const bf16_t* __restrict__ wp, const bf16_t* xs, int K, int lane,
+                                               WChunk& a, WChunk& b) {
+  const bf16_t* xp = xs + (lane & 15) * (K + 8) + (lane >> 4) * 16;
   floatx4 acc = {0.f, 0.f, 0.f, 0.f};
   const int nlines = K / kLine;
-  WChunk cur = first, nxt;
-  for (int l = 0; l < nlines; l += kChunk) {
-    if (l + kChunk < nlines) load_chunk(nxt, wp, l + kChunk, nlines);
-#pragma unroll
-    for (int u = 0; u < kChunk; ++u)
-      if (l + u < nlines) {
-        const bf16x8 x0 = *reinterpret_cast<const bf16x8*>(xp + (l + u) * kLine);
-        const bf16x8 x1 = *reinterpret_cast<const bf16x8*>(xp + (l + u) * kLine + 8);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.w0[u], x0, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.w1[u], x1, acc, 0, 0, 0);
-      }
-    cur = nxt;
+  for (int l = 0; l < nlines; l += 2 * kChunk) {
+    mul_chunk<kWhole>(acc, a, xp, l, nlines);
+    load_chunk<kWhole>(a, wp, l + 2 * kChunk, nlines);
+    mul_chunk<kWhole>(acc, b, xp, l + kChunk, nlines);
+    load_chunk<kWhole>(b, wp, l + 3 * kChunk, nlines);
   }
   return acc;
 }
 
-// grid = (2I / 64, E).  gu[slot, c] = x[slot / k] . w_gate_up[e, c, :]
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void gateup_stream_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wgu,
-                                                            const int32_t* __restrict__ idx, int S, int k, int H, int I,
-                                                            float* __restrict__ gu) {
+typedef __attribute__((address_space(3))) void stream_lds_void;
+typedef const __attribute__((address_space(1))) void stream_gbl_void;
+
+// wait until at most the kChunk lines of weights requested last are still on their way (loads complete in order)
+__device__ __forceinline__ void wait_all_but_chunk(bool chunk_requested) {
+  if (chunk_requested) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  static_assert(2 * kChunk == 8, "the wait above counts the two loads per line of one chunk");
+}
+
+// Operand rows of slots rows_s[r0 .. r0+nrow), row (slot / div) of `src` (row length K), into xs[t][0..K) (row
+// stride K + 8), by LDS-DMA: one wave instruction moves 1 KB of one row (lane L's 16 bytes land at base + 16 L),
+// no registers hold the data.  The rows are requested, then chunk `b` of the weights (lines kChunk..), and the
+// wave then waits for its rows only.  Rows past nrow keep whatever LDS held: they only feed accumulator
+// columns nobody stores.  The caller's barrier makes the rows visible to the other waves.
+template <bool kWhole>
+__device__ __forceinline__ void stage_rows(const bf16_t* __restrict__ src, const unsigned short* rows_s, int r0,
+                                           int nrow, int div, int K, bf16_t* xs, WChunk& b,
+                                           const bf16_t* __restrict__ wp, int nlines) {
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int gran = K / 8;                                      // 16-byte granules per row
+  const int segs = (gran + 63) >> 6;                           // 1 KB pieces per row
+  const int items = nrow * segs;
+  for (int it = wave; it < items; it += 4) {
+    const int t = it / segs, sg = it - t * segs;
+    const int row = __builtin_amdgcn_readfirstlane((int)rows_s[r0 + t]) / div;                 // moe.py:81
+    const int c = sg * 64 + lane;
+    if (c < gran)
+      __builtin_amdgcn_global_load_lds((stream_gbl_void*)(src + (size_t)row * K + c * 8),
+                                       (stream_lds_void*)(xs + t * (K + 8) + sg * 512), 16, 0, 0);
+  }
+  load_chunk<kWhole>(b, wp, kChunk, nlines);
+  wait_all_but_chunk(kWhole && nlines > kChunk);
+}
+
+// grid = (2I / 64, E).  gu[slot, c] = x[slot / k] . w_gate_up[e, c, :].  kWhole: H is a whole number of chunks.
+template <bool kWhole>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4)))
+void gateup_stream_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wgu, const int32_t* __restrict__ idx,
+                          int S, int k, int H, int I, bf16_t* __restrict__ gu) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   __shared__ unsigned short rows_s[kStreamMaxSlots];   // 16-bit slot ids keep four workgroups within a CU's LDS
   __shared__ int cnt_s[kScan * 4];
@@ -112,32 +173,34 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
   const int e = blockIdx.y;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int c0 = blockIdx.x * kRowsPerWg + wave * kRowsPerWave;  // first weight row of this wave
-  const bf16_t* wrow = wgu + ((size_t)e * 2 * I + c0 + (lane & 15)) * H;
-  WChunk first;
-  load_chunk(first, wrow + (lane >> 4) * 16, 0, H / kLine);    // in flight while the rows are found and staged
-  const int n = expert_rows(idx, S, e, rows_s, cnt_s);
-  if (n == 0) return;                                          // idle expert
-  const int gran_per_row = H / 8;
+  // this lane's 32 bytes of every line of its weight row
+  const bf16_t* wp = wgu + ((size_t)e * 2 * I + c0 + (lane & 15)) * H + (lane >> 4) * 16;
+  const int nlines = H / kLine;
+  ScanRegs sr;
+  scan_issue(sr, idx, S);
+  WChunk ca, cb;
+  load_chunk<kWhole>(ca, wp, 0, nlines);                       // keeps HBM busy while the rows are found
+  const int n = scan_finish(sr, e, rows_s, cnt_s);
   for (int r0 = 0; r0 < n; r0 += kTok) {
     const int nrow = min(kTok, n - r0);
-    __syncthreads();                                           // previous pass is done with xs
-    for (int i = tid; i < kTok * gran_per_row; i += 256) {
-      const int t = i / gran_per_row, c = i - t * gran_per_row;
-      u32x4 v = {0u, 0u, 0u, 0u};
-      if (t < nrow) v = *reinterpret_cast<const u32x4*>(x + (size_t)(rows_s[r0 + t] / k) * H + c * 8);   // moe.py:81
-      *reinterpret_cast<u32x4*>(xs + t * (H + 8) + c * 8) = v;
+    if (r0 > 0) {                                              // a further pass starts the weight rows again
+      __syncthreads();                                         // the pass before is done with xs
+      load_chunk<kWhole>(ca, wp, 0, nlines);
     }
+    stage_rows<kWhole>(x, rows_s, r0, nrow, k, H, xs, cb, wp, nlines);
     __syncthreads();
-    const floatx4 acc = stream_rows(wrow, xs, H, lane, first);
+    const floatx4 acc = stream_rows<kWhole>(wp, xs, H, lane, ca, cb);
     // accumulator: lane holds row lane%16 of the pass, weight rows 4*(lane/16) + i
     const int t = lane & 15;
-    if (t < nrow)
-      *reinterpret_cast<floatx4*>(gu + (size_t)rows_s[r0 + t] * 2 * I + c0 + 4 * (lane >> 4)) = acc;
+    if (t < nrow) {
+      bf16x4 o = {(bf16_t)acc[0], (bf16_t)acc[1], (bf16_t)acc[2], (bf16_t)acc[3]};
+      *reinterpret_cast<bf16x4*>(gu + (size_t)rows_s[r0 + t] * 2 * I + c0 + 4 * (lane >> 4)) = o;
+    }
   }
 }
 
-// One workgroup per slot: hidden[slot] = r^p SiLU(g/r) up from the fp32 pre-activations (moe.py:87-92).
-__global__ __launch_bounds__(256) void activate_rows_kernel(const float* __restrict__ gu, const float* __restrict__ theta,
+// One workgroup per slot: hidden[slot] = r^p SiLU(g/r) up from the bf16 pre-activations (moe.py:87-92).
+__global__ __launch_bounds__(256) void activate_rows_kernel(const bf16_t* __restrict__ gu, const float* __restrict__ theta,
                                                             const int32_t* __restrict__ idx, int E, int I,
                                                             bf16_t* __restrict__ hidden) {
   __shared__ float red[4];
@@ -145,9 +208,9 @@ __global__ __launch_bounds__(256) void activate_rows_kernel(const float* __restr
   const int e = idx[slot];
   if ((unsigned)e >= (unsigned)E) return;                      // no expert: the slot has no row
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const float* grow = gu + (size_t)slot * 2 * I;
+  const bf16_t* grow = gu + (size_t)slot * 2 * I;
   float ss = 0.f;
-  for (int i = tid; i < I; i += 256) ss = fmaf(grow[i], grow[i], ss);
+  for (int i = tid; i < I; i += 256) ss = fmaf((float)grow[i], (float)grow[i], ss);
   ss = wave_sum(ss);
   if (lane == 0) red[wave] = ss;
   __syncthreads();
@@ -155,39 +218,104 @@ __global__ __launch_bounds__(256) void activate_rows_kernel(const float* __restr
   const float p = 1.f / (1.f + __expf(-theta[e]));                                        // moe.py:89
   const float rinv = rsqrtf(r2), gain = __expf(0.5f * p * __logf(r2));                     // 1/r, r^p
   for (int i = tid; i < I; i += 256) {
-    const float z = grow[i] * rinv;
-    hidden[(size_t)slot * I + i] = (bf16_t)(z / (1.f + __expf(-z)) * gain * grow[I + i]);
+    const float z = (float)grow[i] * rinv;
+    hidden[(size_t)slot * I + i] = (bf16_t)(z / (1.f + __expf(-z)) * gain * (float)grow[I + i]);
   }
 }
 
-// grid = (H / 64, E).  yw[slot, c] = w[slot] * (hidden[slot] . w_down[e, c, :])
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void down_stream_kernel(const bf16_t* __restrict__ hidden, const bf16_t* __restrict__ wd,
-                                                          const float* __restrict__ w, const int32_t* __restrict__ idx,
-                                                          int S, int H, int I, float* __restrict__ yw) {
+// Operand rows of the down projection computed in place of a copy: hidden rows of slots rows_s[r0 .. r0+nrow)
+// from the bf16 pre-activations, r = sqrt(mean(g^2) + eps), hidden = r^p SiLU(g/r) up, p = sigmoid(theta)
+// (moe.py:87-92), into hs[t][0..I) (row stride I + 8).  tpr = 32 or 64 threads share a row, so the workgroup
+// covers 8 (or 4) rows per round; a thread owns granules part, part + tpr of the gate and of the up half.  The
+// first round's loads are requested ahead of chunk `b` of the weights, like the rows in stage_rows.
+// I <= kFusedActMaxI.
+template <bool kWhole>
+__device__ __forceinline__ void stage_activated(const bf16_t* __restrict__ gu, float theta_e,
+                                                const unsigned short* rows_s, int r0, int nrow, int I, bf16_t* hs,
+                                                WChunk& b, const bf16_t* __restrict__ wp, int nlines) {
+  constexpr int kPer = kFusedActMaxI / 8 / 32;                 // granules per thread and half at 32 threads per row
+  const int tid = threadIdx.x;
+  const int tpr = nrow <= 4 ? 64 : 32;
+  const int row_in = tid / tpr, part = tid - row_in * tpr;
+  const int gran = I / 8;
+  const float p = 1.f / (1.f + __expf(-theta_e));                                          // moe.py:89
+  for (int rb = 0; rb < nrow; rb += 256 / tpr) {
+    const int row = rb + row_in;
+    const bool live = row < nrow;                              // whole groups of tpr lanes are live or not
+    const bf16_t* grow = gu + (size_t)rows_s[r0 + (live ? row : 0)] * 2 * I;
+    bf16x8 g[kPer], u[kPer];
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+      const int c = part + j * tpr;
+      if (live && c < gran) {
+        g[j] = *reinterpret_cast<const bf16x8*>(grow + c * 8);
+        u[j] = *reinterpret_cast<const bf16x8*>(grow + I + c * 8);
+      }
+    }
+    if (rb == 0) load_chunk<kWhole>(b, wp, kChunk, nlines);
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < kPer; ++j)
+      if (live && part + j * tpr < gran) {
+#pragma unroll
+        for (int q = 0; q < 8; ++q) ss = fmaf((float)g[j][q], (float)g[j][q], ss);
+      }
+    for (int o = tpr >> 1; o > 0; o >>= 1) ss += __shfl_xor(ss, o, kWave);   // the row's threads are adjacent lanes
+    const float r2 = ss / (float)I + kNormSiluEps;                                        // moe.py:88
+    const float rinv = rsqrtf(r2), gain = __expf(0.5f * p * __logf(r2));                   // 1/r, r^p
+    const float nrl = -1.4426950408889634f * rinv, rg = rinv * gain;
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+      const int c = part + j * tpr;
+      if (live && c < gran) {
+        bf16x8 h;
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+          // z / (1 + exp(-z)) * gain * up with z = g / r, constants folded per row
+          const float gq = (float)g[j][q];
+          const float sig = __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(gq * nrl));
+          h[q] = (bf16_t)(gq * rg * sig * (float)u[j][q]);
+          if (q & 1) __builtin_amdgcn_sched_barrier(0);        // two elements at a time: few temporaries alive
+        }
+        *reinterpret_cast<bf16x8*>(hs + row * (I + 8) + c * 8) = h;
+      }
+    }
+  }
+}
+
+// grid = (H / 64, E).  yw[slot, c] = w[slot] * (hidden[slot] . w_down[e, c, :]).  kFusedAct: `act` holds the bf16
+// gate/up pre-activations [slot, 2I] and the activation happens here; otherwise it holds hidden [slot, I].
+// kWhole: I is a whole number of chunks.
+template <bool kFusedAct, bool kWhole>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4)))
+void down_stream_kernel(const bf16_t* __restrict__ act, const bf16_t* __restrict__ wd, const float* __restrict__ theta,
+                        const float* __restrict__ w, const int32_t* __restrict__ idx, int S, int H, int I,
+                        float* __restrict__ yw) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  __shared__ unsigned short rows_s[kStreamMaxSlots];   // 16-bit slot ids keep four workgroups within a CU's LDS
+  __shared__ unsigned short rows_s[kStreamMaxSlots];
   __shared__ int cnt_s[kScan * 4];
-  bf16_t* hs = reinterpret_cast<bf16_t*>(smem_raw);            // [kTok][I + 8] activations of this pass
+  bf16_t* hs = reinterpret_cast<bf16_t*>(smem_raw);            // [kTok][I + 8] operand rows of this pass
   const int e = blockIdx.y;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int c0 = blockIdx.x * kRowsPerWg + wave * kRowsPerWave;
-  const bf16_t* wrow = wd + ((size_t)e * H + c0 + (lane & 15)) * I;
-  WChunk first;
-  load_chunk(first, wrow + (lane >> 4) * 16, 0, I / kLine);
-  const int n = expert_rows(idx, S, e, rows_s, cnt_s);
-  if (n == 0) return;
-  const int gran_per_row = I / 8;
+  const bf16_t* wp = wd + ((size_t)e * H + c0 + (lane & 15)) * I + (lane >> 4) * 16;
+  const int nlines = I / kLine;
+  ScanRegs sr;
+  scan_issue(sr, idx, S);
+  const float theta_e = kFusedAct ? theta[e] : 0.f;
+  WChunk ca, cb;
+  load_chunk<kWhole>(ca, wp, 0, nlines);
+  const int n = scan_finish(sr, e, rows_s, cnt_s);
   for (int r0 = 0; r0 < n; r0 += kTok) {
     const int nrow = min(kTok, n - r0);
-    __syncthreads();
-    for (int i = tid; i < kTok * gran_per_row; i += 256) {
-      const int t = i / gran_per_row, c = i - t * gran_per_row;
-      u32x4 v = {0u, 0u, 0u, 0u};
-      if (t < nrow) v = *reinterpret_cast<const u32x4*>(hidden + (size_t)rows_s[r0 + t] * I + c * 8);
-      *reinterpret_cast<u32x4*>(hs + t * (I + 8) + c * 8) = v;
+    if (r0 > 0) {
+      __syncthreads();
+      load_chunk<kWhole>(ca, wp, 0, nlines);
     }
+    if (kFusedAct) stage_activated<kWhole>(act, theta_e, rows_s, r0, nrow, I, hs, cb, wp, nlines);
+    else stage_rows<kWhole>(act, rows_s, r0, nrow, 1, I, hs, cb, wp, nlines);
     __syncthreads();
-    const floatx4 acc = stream_rows(wrow, hs, I, lane, first);
+    const floatx4 acc = stream_rows<kWhole>(wp, hs, I, lane, ca, cb);
     const int t = lane & 15;
     if (t < nrow) {
       const int slot = rows_s[r0 + t];
@@ -201,32 +329,44 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 }  // namespace
 
 bool stream_supported(int H, int I, int dtype) {
-  // LDS: 16 rows of (max(H, I) + 8) bf16 within 56 KB (next to the 8 KB row list); every K extent must be whole
+  // LDS: 16 rows of (max(H, I) + 8) bf16 within 56 KB (next to the 4 KB row list); every K extent must be whole
   // 128-byte lines
   return dtype == BIBO_DTYPE_BF16 && (H % 64) == 0 && (I % 64) == 0 && H <= 1728 && I <= 1728;
 }
 
-size_t stream_gu_bytes(int T, int k, int I) { return (size_t)T * k * 2 * I * sizeof(float); }
-
 hipError_t launch_gateup_stream(const void* x, const void* wgu, const int32_t* idx, int T, int H, int E, int k, int I,
-                                float* gu, hipStream_t s) {
+                                void* gu, hipStream_t s) {
   if (T * k == 0) return hipSuccess;
   if (T * k > kStreamMaxSlots) return hipErrorInvalidValue;
   const size_t shm = (size_t)kTok * (H + 8) * sizeof(bf16_t);
-  hipLaunchKernelGGL(gateup_stream_kernel, dim3(2 * I / kRowsPerWg, E), dim3(256), shm, s,
-                     static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(wgu), idx, T * k, k, H, I, gu);
+  const dim3 grid(2 * I / kRowsPerWg, E);
+  if (H % (kChunk * kLine) == 0)
+    hipLaunchKernelGGL(gateup_stream_kernel<true>, grid, dim3(256), shm, s, static_cast<const bf16_t*>(x),
+                       static_cast<const bf16_t*>(wgu), idx, T * k, k, H, I, static_cast<bf16_t*>(gu));
+  else
+    hipLaunchKernelGGL(gateup_stream_kernel<false>, grid, dim3(256), shm, s, static_cast<const bf16_t*>(x),
+                       static_cast<const bf16_t*>(wgu), idx, T * k, k, H, I, static_cast<bf16_t*>(gu));
   return hipGetLastError();
 }
 
-hipError_t launch_down_stream(const float* gu, const void* wd, const float* theta, const float* w, const int32_t* idx,
+hipError_t launch_down_stream(const void* gu, const void* wd, const float* theta, const float* w, const int32_t* idx,
                               int T, int H, int E, int k, int I, void* hidden, float* yw, hipStream_t s) {
   if (T * k == 0) return hipSuccess;
   if (T * k > kStreamMaxSlots) return hipErrorInvalidValue;
-  bf16_t* hp = static_cast<bf16_t*>(hidden);
-  hipLaunchKernelGGL(activate_rows_kernel, dim3(T * k), dim3(256), 0, s, gu, theta, idx, E, I, hp);
   const size_t shm = (size_t)kTok * (I + 8) * sizeof(bf16_t);
-  hipLaunchKernelGGL(down_stream_kernel, dim3(H / kRowsPerWg, E), dim3(256), shm, s, hp,
-                     static_cast<const bf16_t*>(wd), w, idx, T * k, H, I, yw);
+  const dim3 grid(H / kRowsPerWg, E);
+  const bf16_t* g = static_cast<const bf16_t*>(gu);
+  const bf16_t* wdp = static_cast<const bf16_t*>(wd);
+  const bool whole = I % (kChunk * kLine) == 0;
+  if (I <= kFusedActMaxI) {
+    if (whole) hipLaunchKernelGGL((down_stream_kernel<true, true>), grid, dim3(256), shm, s, g, wdp, theta, w, idx, T * k, H, I, yw);
+    else hipLaunchKernelGGL((down_stream_kernel<true, false>), grid, dim3(256), shm, s, g, wdp, theta, w, idx, T * k, H, I, yw);
+  } else {
+    bf16_t* hp = static_cast<bf16_t*>(hidden);
+    hipLaunchKernelGGL(activate_rows_kernel, dim3(T * k), dim3(256), 0, s, g, theta, idx, E, I, hp);
+    if (whole) hipLaunchKernelGGL((down_stream_kernel<false, true>), grid, dim3(256), shm, s, hp, wdp, theta, w, idx, T * k, H, I, yw);
+    else hipLaunchKernelGGL((down_stream_kernel<false, false>), grid, dim3(256), shm, s, hp, wdp, theta, w, idx, T * k, H, I, yw);
+  }
   return hipGetLastError();
 }
 
