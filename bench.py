@@ -86,7 +86,11 @@ class Layer:
         }
         # the expert stages the composite call runs for this shape: one fused launch + combine where the
         # fused kernel applies (and no other family was asked for), else one kernel per projection
-        self.fused = (algo in ("auto", "fused") and self.S > 32 * E and H % 128 == 0 and I in (128, 256, 384))
+        # (the library's own rule: streaming kernels up to 40 / 32 / 24 rows per expert by row width)
+        stream_rows = 40 if (H <= 512 and I <= 512) else (32 if H <= 768 else 24)
+        streams = H % 64 == 0 and I % 64 == 0 and self.S <= min(stream_rows * E, 4096) and T <= 2048
+        self.fused = (algo in ("auto", "fused") and not (algo == "auto" and streams) and H % 128 == 0
+                      and I in (128, 256, 384))
         if self.fused:
             self._stages.update({
                 "gateup_down": (self.lib.bibo_moe_gateup_down_fwd,

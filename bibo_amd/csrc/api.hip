@@ -19,12 +19,18 @@ int check_dims(int T, int H, int E, int k, int I, int dtype, int n_pos = 0, int 
   return BIBO_OK;
 }
 
-// rows per expert at or below which the weight-streaming kernels are preferred
-constexpr long long kStreamRowsPerExpert = 32;
+// Rows per expert at or below which the weight-streaming kernels are preferred (measured against the MFMA tile
+// kernels at E = 64, k = 6).  With H and I up to 512 a wave's 16 weight rows stay in registers for all of the
+// expert's rows and a further 16-row pass only costs its staging (crossover near 40 rows); wider rows are
+// streamed again, from L2, for every pass (crossover near 32 rows at H = 768, near 24 at H = 1024).
+inline long long stream_rows_per_expert(int H, int I) {
+  if (H <= 512 && I <= 512) return 40;
+  return H <= 768 ? 32 : 24;
+}
 
 inline bool stream_eligible(int T, int H, int E, int k, int I, int dtype) {
-  return stream_supported(H, I, dtype) && (long long)T * k <= kStreamRowsPerExpert * E &&
-         (long long)T * k <= kStreamMaxSlots;
+  return stream_supported(H, I, dtype) && (long long)T * k <= stream_rows_per_expert(H, I) * E &&
+         (long long)T * k <= kStreamMaxSlots && T <= kStreamMaxRows;
 }
 
 // `composite`: the caller is bibo_moe_experts_fwd / bibo_moe_forward, the only entry points that can run

@@ -16,7 +16,8 @@ constexpr float kSumNormEps = 1e-20f;   // src/modeling/ffn/router.py:45
 
 // tokens handled by one workgroup of the histogram / permutation kernels
 constexpr int kPermTokens = 128;   // tokens per permutation workgroup (256 and 64 measured slower)
-constexpr int kStreamMaxSlots = 2048;   // routed slots the weight-streaming kernels can scan per workgroup
+constexpr int kStreamMaxSlots = 4096;   // routed slots the weight-streaming kernels can scan per workgroup
+constexpr int kStreamMaxRows = 2048;    // rows (= tokens) one expert can get in them
 
 typedef __bf16 bf16_t;
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));

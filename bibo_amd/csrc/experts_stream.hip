@@ -51,25 +51,29 @@ __device__ __forceinline__ void scan_issue(ScanRegs& r, const int32_t* __restric
 }
 
 // Slots routed to expert e, ascending, into rows_s; returns how many.  All 256 threads call it; ends with a
-// barrier.
-__device__ __forceinline__ int scan_finish(const ScanRegs& r, int e, unsigned short* rows_s, int* cnt_s) {
+// barrier.  Only the ceil(S / 256) index groups that hold slots are looked at.
+__device__ __forceinline__ int scan_finish(const ScanRegs& r, int S, int e, unsigned short* rows_s, int* cnt_s) {
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const unsigned long long lt = (1ull << lane) - 1ull;
+  const int nq = (S + 255) >> 8;
   int rank[kScan];
 #pragma unroll
-  for (int q = 0; q < kScan; ++q) {
-    const unsigned long long b = __ballot(r.v[q] == e);
-    rank[q] = __popcll(b & lt);
-    if (lane == 0) cnt_s[q * 4 + wave] = __popcll(b);
-  }
+  for (int q = 0; q < kScan; ++q)
+    if (q < nq) {
+      const unsigned long long b = __ballot(r.v[q] == e);
+      rank[q] = __popcll(b & lt);
+      if (lane == 0) cnt_s[q * 4 + wave] = __popcll(b);
+    }
   __syncthreads();
   int run = 0;                                                  // exclusive prefix over the (q, wave) cells in slot order
 #pragma unroll
   for (int q = 0; q < kScan; ++q)
+    if (q < nq) {
 #pragma unroll
-    for (int ww = 0; ww < 4; ++ww) {
-      if (ww == wave && r.v[q] == e) rows_s[run + rank[q]] = (unsigned short)(q * 256 + tid);
-      run += cnt_s[q * 4 + ww];
+      for (int ww = 0; ww < 4; ++ww) {
+        if (ww == wave && r.v[q] == e) rows_s[run + rank[q]] = (unsigned short)(q * 256 + tid);
+        run += cnt_s[q * 4 + ww];
+      }
     }
   __syncthreads();
   return run;
@@ -143,7 +147,7 @@ __device__ __forceinline__ void wait_all_but_chunk(bool chunk_requested) {
 template <bool kWhole>
 __device__ __forceinline__ void stage_rows(const bf16_t* __restrict__ src, const unsigned short* rows_s, int r0,
                                            int nrow, int div, int K, bf16_t* xs, WChunk& b,
-                                           const bf16_t* __restrict__ wp, int nlines) {
+                                           const bf16_t* __restrict__ wp, int nlines, bool load_b) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int gran = K / 8;                                      // 16-byte granules per row
@@ -157,8 +161,8 @@ __device__ __forceinline__ void stage_rows(const bf16_t* __restrict__ src, const
       __builtin_amdgcn_global_load_lds((stream_gbl_void*)(src + (size_t)row * K + c * 8),
                                        (stream_lds_void*)(xs + t * (K + 8) + sg * 512), 16, 0, 0);
   }
-  load_chunk<kWhole>(b, wp, kChunk, nlines);
-  wait_all_but_chunk(kWhole && nlines > kChunk);
+  if (load_b) load_chunk<kWhole>(b, wp, kChunk, nlines);
+  wait_all_but_chunk(load_b && kWhole && nlines > kChunk);
 }
 
 // grid = (2I / 64, E).  gu[slot, c] = x[slot / k] . w_gate_up[e, c, :].  kWhole: H is a whole number of chunks.
@@ -167,7 +171,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4)))
 void gateup_stream_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wgu, const int32_t* __restrict__ idx,
                           int S, int k, int H, int I, bf16_t* __restrict__ gu) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  __shared__ unsigned short rows_s[kStreamMaxSlots];   // 16-bit slot ids keep four workgroups within a CU's LDS
+  __shared__ unsigned short rows_s[kStreamMaxRows];    // 16-bit slot ids keep four workgroups within a CU's LDS
   __shared__ int cnt_s[kScan * 4];
   bf16_t* xs = reinterpret_cast<bf16_t*>(smem_raw);            // [kTok][H + 8]
   const int e = blockIdx.y;
@@ -176,18 +180,20 @@ void gateup_stream_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict
   // this lane's 32 bytes of every line of its weight row
   const bf16_t* wp = wgu + ((size_t)e * 2 * I + c0 + (lane & 15)) * H + (lane >> 4) * 16;
   const int nlines = H / kLine;
+  const bool resident = nlines <= 2 * kChunk;                  // the two chunks hold the whole row: passes share them
   ScanRegs sr;
   scan_issue(sr, idx, S);
   WChunk ca, cb;
   load_chunk<kWhole>(ca, wp, 0, nlines);                       // keeps HBM busy while the rows are found
-  const int n = scan_finish(sr, e, rows_s, cnt_s);
+  const int n = scan_finish(sr, S, e, rows_s, cnt_s);
   for (int r0 = 0; r0 < n; r0 += kTok) {
     const int nrow = min(kTok, n - r0);
-    if (r0 > 0) {                                              // a further pass starts the weight rows again
+    const bool reload = r0 == 0 || !resident;
+    if (r0 > 0) {
       __syncthreads();                                         // the pass before is done with xs
-      load_chunk<kWhole>(ca, wp, 0, nlines);
+      if (reload) load_chunk<kWhole>(ca, wp, 0, nlines);       // a further pass starts the weight rows again
     }
-    stage_rows<kWhole>(x, rows_s, r0, nrow, k, H, xs, cb, wp, nlines);
+    stage_rows<kWhole>(x, rows_s, r0, nrow, k, H, xs, cb, wp, nlines, reload);
     __syncthreads();
     const floatx4 acc = stream_rows<kWhole>(wp, xs, H, lane, ca, cb);
     // accumulator: lane holds row lane%16 of the pass, weight rows 4*(lane/16) + i
@@ -232,7 +238,7 @@ __global__ __launch_bounds__(256) void activate_rows_kernel(const bf16_t* __rest
 template <bool kWhole>
 __device__ __forceinline__ void stage_activated(const bf16_t* __restrict__ gu, float theta_e,
                                                 const unsigned short* rows_s, int r0, int nrow, int I, bf16_t* hs,
-                                                WChunk& b, const bf16_t* __restrict__ wp, int nlines) {
+                                                WChunk& b, const bf16_t* __restrict__ wp, int nlines, bool load_b) {
   constexpr int kPer = kFusedActMaxI / 8 / 32;                 // granules per thread and half at 32 threads per row
   const int tid = threadIdx.x;
   const int tpr = nrow <= 4 ? 64 : 32;
@@ -252,7 +258,7 @@ __device__ __forceinline__ void stage_activated(const bf16_t* __restrict__ gu, f
         u[j] = *reinterpret_cast<const bf16x8*>(grow + I + c * 8);
       }
     }
-    if (rb == 0) load_chunk<kWhole>(b, wp, kChunk, nlines);
+    if (rb == 0 && load_b) load_chunk<kWhole>(b, wp, kChunk, nlines);
     float ss = 0.f;
 #pragma unroll
     for (int j = 0; j < kPer; ++j)
@@ -292,7 +298,7 @@ void down_stream_kernel(const bf16_t* __restrict__ act, const bf16_t* __restrict
                         const float* __restrict__ w, const int32_t* __restrict__ idx, int S, int H, int I,
                         float* __restrict__ yw) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  __shared__ unsigned short rows_s[kStreamMaxSlots];
+  __shared__ unsigned short rows_s[kStreamMaxRows];
   __shared__ int cnt_s[kScan * 4];
   bf16_t* hs = reinterpret_cast<bf16_t*>(smem_raw);            // [kTok][I + 8] operand rows of this pass
   const int e = blockIdx.y;
@@ -300,20 +306,22 @@ void down_stream_kernel(const bf16_t* __restrict__ act, const bf16_t* __restrict
   const int c0 = blockIdx.x * kRowsPerWg + wave * kRowsPerWave;
   const bf16_t* wp = wd + ((size_t)e * H + c0 + (lane & 15)) * I + (lane >> 4) * 16;
   const int nlines = I / kLine;
+  const bool resident = nlines <= 2 * kChunk;
   ScanRegs sr;
   scan_issue(sr, idx, S);
   const float theta_e = kFusedAct ? theta[e] : 0.f;
   WChunk ca, cb;
   load_chunk<kWhole>(ca, wp, 0, nlines);
-  const int n = scan_finish(sr, e, rows_s, cnt_s);
+  const int n = scan_finish(sr, S, e, rows_s, cnt_s);
   for (int r0 = 0; r0 < n; r0 += kTok) {
     const int nrow = min(kTok, n - r0);
+    const bool reload = r0 == 0 || !resident;
     if (r0 > 0) {
       __syncthreads();
-      load_chunk<kWhole>(ca, wp, 0, nlines);
+      if (reload) load_chunk<kWhole>(ca, wp, 0, nlines);
     }
-    if (kFusedAct) stage_activated<kWhole>(act, theta_e, rows_s, r0, nrow, I, hs, cb, wp, nlines);
-    else stage_rows<kWhole>(act, rows_s, r0, nrow, 1, I, hs, cb, wp, nlines);
+    if (kFusedAct) stage_activated<kWhole>(act, theta_e, rows_s, r0, nrow, I, hs, cb, wp, nlines, reload);
+    else stage_rows<kWhole>(act, rows_s, r0, nrow, 1, I, hs, cb, wp, nlines, reload);
     __syncthreads();
     const floatx4 acc = stream_rows<kWhole>(wp, hs, I, lane, ca, cb);
     const int t = lane & 15;
@@ -337,7 +345,7 @@ bool stream_supported(int H, int I, int dtype) {
 hipError_t launch_gateup_stream(const void* x, const void* wgu, const int32_t* idx, int T, int H, int E, int k, int I,
                                 void* gu, hipStream_t s) {
   if (T * k == 0) return hipSuccess;
-  if (T * k > kStreamMaxSlots) return hipErrorInvalidValue;
+  if (T * k > kStreamMaxSlots || T > kStreamMaxRows) return hipErrorInvalidValue;
   const size_t shm = (size_t)kTok * (H + 8) * sizeof(bf16_t);
   const dim3 grid(2 * I / kRowsPerWg, E);
   if (H % (kChunk * kLine) == 0)
@@ -352,7 +360,7 @@ hipError_t launch_gateup_stream(const void* x, const void* wgu, const int32_t* i
 hipError_t launch_down_stream(const void* gu, const void* wd, const float* theta, const float* w, const int32_t* idx,
                               int T, int H, int E, int k, int I, void* hidden, float* yw, hipStream_t s) {
   if (T * k == 0) return hipSuccess;
-  if (T * k > kStreamMaxSlots) return hipErrorInvalidValue;
+  if (T * k > kStreamMaxSlots || T > kStreamMaxRows) return hipErrorInvalidValue;
   const size_t shm = (size_t)kTok * (I + 8) * sizeof(bf16_t);
   const dim3 grid(H / kRowsPerWg, E);
   const bf16_t* g = static_cast<const bf16_t*>(gu);

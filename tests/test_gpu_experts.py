@@ -122,7 +122,7 @@ def test_bf16_experts_reduced_prefill_and_ragged_shapes(T, H, I, bias, theta, al
 
 @pytest.mark.parametrize("T,H,I,k,theta", [(64, 1024, 512, 6, "zero"), (7, 1024, 512, 6, "normal"), (1, 768, 384, 6, "normal"),
                                            (200, 256, 128, 6, "normal"), (130, 128, 256, 2, "normal"),
-                                           (40, 64, 64, 1, "normal")])
+                                           (40, 64, 64, 1, "normal"), (400, 512, 256, 6, "normal")])
 def test_streaming_kernels_match_oracle(T, H, I, k, theta):
     """Weight-streaming (decode) kernels: few rows per expert, several 16-row passes, idle experts."""
     p = O.make_inputs(T=T, H=H, E=64, k=k, I=I, bias="uniform", theta=theta, seed=T + I)
