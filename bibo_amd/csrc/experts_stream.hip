@@ -366,7 +366,9 @@ hipError_t launch_down_stream(const void* gu, const void* wd, const float* theta
   const bf16_t* g = static_cast<const bf16_t*>(gu);
   const bf16_t* wdp = static_cast<const bf16_t*>(wd);
   const bool whole = I % (kChunk * kLine) == 0;
-  if (I <= kFusedActMaxI) {
+  // The fused activation is computed by every one of the H/64 workgroups of an expert, once per 16-row pass:
+  // cheap next to a launch for one pass, not for several
+  if (I <= kFusedActMaxI && T * k <= kTok * E) {
     if (whole) hipLaunchKernelGGL((down_stream_kernel<true, true>), grid, dim3(256), shm, s, g, wdp, theta, w, idx, T * k, H, I, yw);
     else hipLaunchKernelGGL((down_stream_kernel<true, false>), grid, dim3(256), shm, s, g, wdp, theta, w, idx, T * k, H, I, yw);
   } else {
