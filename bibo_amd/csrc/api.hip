@@ -34,7 +34,7 @@ inline bool stream_eligible(int T, int H, int E, int k, int I, int dtype) {
 }
 
 // `composite`: the caller is bibo_moe_experts_fwd / bibo_moe_forward, the only entry points that can run
-// the streaming kernels (they hand fp32 pre-activations, not `hidden`, from one kernel to the next) and
+// the streaming kernels (they hand bf16 pre-activations, not `hidden`, from one kernel to the next) and
 // the fused kernel (its activations never reach memory).
 int resolve_algo(int algo, int T, int H, int E, int k, int I, int dtype, bool composite, int* out) {
   switch (algo) {
