@@ -36,6 +36,7 @@ constexpr int kLine = 64;          // bf16 elements per 128-byte line
 constexpr int kChunk = 4;          // 128-byte lines per register chunk (two chunks are alive: 64 VGPRs)
 constexpr int kScan = kStreamMaxSlots / 256;   // routing indices each thread inspects
 constexpr int kFusedActMaxI = 512; // widest I whose activation the down kernel computes itself
+static_assert(kFusedActMaxI == 2 * kChunk * kLine, "the fused-activation down kernel assumes two chunks hold a row");
 
 struct ScanRegs {
   int v[kScan];
@@ -114,12 +115,19 @@ __device__ __forceinline__ void mul_chunk(floatx4& acc, const WChunk& c, const b
 // elements, so the 16 lanes of a fragment read hit distinct banks).  On entry `a` and `b` hold lines
 // 0..kChunk-1 and kChunk..2*kChunk-1; each is refilled, two chunks ahead, as soon as it is consumed, so on
 // return they hold other lines.
-template <bool kWhole>
+// kTwoChunks: the caller knows that the row is no longer than the two chunks (nothing is ever refilled, and the
+// weight pointer is dead once they are requested).
+template <bool kWhole, bool kTwoChunks = false>
 __device__ __forceinline__ floatx4 stream_rows(const bf16_t* __restrict__ wp, const bf16_t* xs, int K, int lane,
                                                WChunk& a, WChunk& b) {
   const bf16_t* xp = xs + (lane & 15) * (K + 8) + (lane >> 4) * 16;
   floatx4 acc = {0.f, 0.f, 0.f, 0.f};
   const int nlines = K / kLine;
+  if (kTwoChunks) {
+    mul_chunk<kWhole>(acc, a, xp, 0, nlines);
+    mul_chunk<kWhole>(acc, b, xp, kChunk, nlines);
+    return acc;
+  }
   for (int l = 0; l < nlines; l += 2 * kChunk) {
     mul_chunk<kWhole>(acc, a, xp, l, nlines);
     load_chunk<kWhole>(a, wp, l + 2 * kChunk, nlines);
@@ -323,7 +331,8 @@ void down_stream_kernel(const bf16_t* __restrict__ act, const bf16_t* __restrict
     if (kFusedAct) stage_activated<kWhole>(act, theta_e, rows_s, r0, nrow, I, hs, cb, wp, nlines, reload);
     else stage_rows<kWhole>(act, rows_s, r0, nrow, 1, I, hs, cb, wp, nlines, reload);
     __syncthreads();
-    const floatx4 acc = stream_rows<kWhole>(wp, hs, I, lane, ca, cb);
+    // the fused activation is only used up to I = kFusedActMaxI = two chunks
+    const floatx4 acc = stream_rows<kWhole, kFusedAct>(wp, hs, I, lane, ca, cb);
     const int t = lane & 15;
     if (t < nrow) {
       const int slot = rows_s[r0 + t];
