@@ -24,7 +24,8 @@ PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
 # WRITE_SIZE (KiB per dispatch), scaled by what the same counters read for a 256 MiB device copy
 # (FETCH_SIZE x2.0, WRITE_SIZE x1.0).  Fused kernel: 208.0 MB fetched + 76.4 MB written; gate/up kernel of the
 # two-kernel family: 158.4 MB + 37.7 MB.
-MEASURED_TRAFFIC_BYTES = {("c2", "gateup_down"): 284.4e6, ("c2", "gateup"): 196.1e6}
+MEASURED_TRAFFIC_BYTES = {("c2", "gateup_down"): 284.4e6, ("c2", "gateup"): 196.1e6,
+                          ("c3", "stream"): 137.0e6 + 0.8e6 + 73.7e6 + 1.6e6}   # both streaming kernels, fetch + write
 
 
 def flops_layer(T, H, E, k, I):
@@ -84,13 +85,10 @@ class Layer:
                         (P(self.idx), T, E, k, P(self.counts), P(self.offsets), P(self.perm_slot), P(self.perm_token),
                          P(self.ws), self.ws.numel(), self.stream)),
         }
-        # the expert stages the composite call runs for this shape: one fused launch + combine where the
-        # fused kernel applies (and no other family was asked for), else one kernel per projection
-        # (the library's own rule: streaming kernels up to 40 / 32 / 24 rows per expert by row width)
-        stream_rows = 40 if (H <= 512 and I <= 512) else (32 if H <= 768 else 24)
-        streams = H % 64 == 0 and I % 64 == 0 and self.S <= min(stream_rows * E, 4096) and T <= 2048
-        self.fused = (algo in ("auto", "fused") and not (algo == "auto" and streams) and H % 128 == 0
-                      and I in (128, 256, 384))
+        # the expert stages the composite call runs for this shape: one fused launch + combine where the library
+        # picks the fused kernel, else one kernel per projection (the streaming kernels have no stage entry points)
+        self.family = ops.select_algo(T, H, E, k, I, L.DTYPE_BF16, algo)
+        self.fused = self.family == "fused"
         if self.fused:
             self._stages.update({
                 "gateup_down": (self.lib.bibo_moe_gateup_down_fwd,
@@ -260,6 +258,15 @@ def main():
                      "frac": dom_flops / stages[dom] / 1e12 / PEAK_BF16_TFLOPS,
                      "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, dom))},
     }
+    if layer.family == "stream":
+        # The streaming kernels only exist behind the composite call (the stage entry points time the tile kernels):
+        # the roofline of this workload is the HBM one, algorithmic bytes of the layer over the whole step.
+        nbytes = bytes_layer(T, H, E, k, I, e_active)
+        out["roofline"] = {"kernel": "gateup_stream_kernel + down_stream_kernel (whole bibo_moe_forward step)", "bound": "hbm",
+                           "achieved": nbytes / sec / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                           "frac": nbytes / sec / 1e9 / PEAK_HBM_GBS,
+                           "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, "stream"))}
+        out["stage_us"] = {n: v for n, v in out["stage_us"].items() if n in ("router", "permute")}
     ffn_sec = layer.time_ffn_seam(args.steps, args.warmup)
     out["ffn_seam"] = {"entry": "bibo_moe_ffn_forward: out = h + moe(rmsnorm(h))", "us_per_step": ffn_sec * 1e6,
                        "extra_us_over_layer": (ffn_sec - sec) * 1e6}

@@ -17,7 +17,7 @@ ABI_VERSION = 2
 
 # every symbol include/bibo_moe.h declares
 SYMBOLS = (
-    "bibo_moe_abi_version", "bibo_moe_strerror", "bibo_moe_workspace_bytes", "bibo_moe_router_fwd",
+    "bibo_moe_abi_version", "bibo_moe_strerror", "bibo_moe_workspace_bytes", "bibo_moe_select_algo", "bibo_moe_router_fwd",
     "bibo_moe_permute", "bibo_moe_gateup_fwd", "bibo_moe_down_combine_fwd", "bibo_moe_gateup_down_fwd",
     "bibo_moe_combine_fwd", "bibo_moe_combine_ex_fwd", "bibo_moe_experts_fwd", "bibo_moe_forward", "bibo_moe_rmsnorm_fwd",
     "bibo_moe_ffn_workspace_bytes", "bibo_moe_ffn_forward",
@@ -41,6 +41,8 @@ def _declare(l):
     l.bibo_moe_strerror.argtypes = [ci]
     l.bibo_moe_workspace_bytes.restype = ci
     l.bibo_moe_workspace_bytes.argtypes = [ctypes.POINTER(Shape), ctypes.POINTER(sz)]
+    l.bibo_moe_select_algo.restype = ci
+    l.bibo_moe_select_algo.argtypes = [ctypes.POINTER(Shape), ci, ctypes.POINTER(ci)]
     l.bibo_moe_router_fwd.restype = ci
     l.bibo_moe_router_fwd.argtypes = [vp, vp, vp, ci, ci, ci, ci, ci, ci, vp, vp, vp, vp, vp]
     l.bibo_moe_permute.restype = ci

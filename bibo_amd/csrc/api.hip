@@ -228,6 +228,13 @@ int bibo_moe_workspace_bytes(const bibo_moe_shape* sh, size_t* bytes) {
   return BIBO_OK;
 }
 
+int bibo_moe_select_algo(const bibo_moe_shape* sh, int algo, int* selected) {
+  if (sh == nullptr || selected == nullptr) return BIBO_ERR_NULL_POINTER;
+  const int rc = check_dims(sh->T, sh->H, sh->E, sh->k, sh->I, sh->dtype, sh->n_pos, sh->n_neg);
+  if (rc != BIBO_OK) return rc;
+  return resolve_algo(algo, sh->T, sh->H, sh->E, sh->k, sh->I, sh->dtype, true, selected);
+}
+
 int bibo_moe_router_fwd(const void* x, const void* w_router, const float* bias, int T, int H, int E, int k, int dtype,
                         int norm_mode, float* logits, int32_t* idx, float* w, float* gap, void* stream) {
   const int rc = check_dims(T, H, E, k, 1, dtype);

@@ -25,6 +25,14 @@ def algo_code(v) -> int:
     return _ALGO[v]
 
 
+def select_algo(T, H, E, k, I, dtype_code=L.DTYPE_BF16, algo="auto", n_pos=0, n_neg=0) -> str:
+    """Name of the kernel family the composite calls run for this shape (bibo_moe_select_algo)."""
+    sh = L.Shape(T, H, E, k, I, dtype_code, n_pos, n_neg)
+    out = ctypes.c_int(0)
+    L.check(L.lib().bibo_moe_select_algo(ctypes.byref(sh), algo_code(algo), ctypes.byref(out)), "bibo_moe_select_algo")
+    return {v: n for n, v in _ALGO.items()}[out.value]
+
+
 def _dtype_code(t: torch.Tensor) -> int:
     if t.dtype == torch.bfloat16:
         return L.DTYPE_BF16

@@ -88,6 +88,15 @@ const char* bibo_moe_strerror(int code);
 int bibo_moe_workspace_bytes(const bibo_moe_shape* shape, size_t* bytes);
 
 /*
+ * The kernel family the composite entry points (bibo_moe_experts_fwd, bibo_moe_forward, bibo_moe_ffn_forward) run
+ * for this shape when asked for `algo`: *selected is one of BIBO_ALGO_GENERIC / MFMA / STREAM / FUSED (never AUTO).
+ * Returns BIBO_ERR_UNSUPPORTED when `algo` names a family that cannot run the shape.  Host-side only; no
+ * counterpart in the reference (its choice between eager and patched paths is made by the caller,
+ * ablate/common/patches.py:402-417).
+ */
+int bibo_moe_select_algo(const bibo_moe_shape* shape, int algo, int* selected);
+
+/*
  * Router: fp32 logits, sigmoid scores, selection on scores+bias, gather of the unbiased scores and
  * normalisation.  Replaces BiBoMoERouter.forward (src/modeling/ffn/router.py:28-51) and the external
  * fused router the reference once bound (legacy/bench/exp_kappa.py:142-155).

@@ -65,6 +65,25 @@ def test_argument_errors_are_reported_without_a_gpu():
         L.check(-4, "x")
 
 
+def test_kernel_family_selection_is_exported():
+    """bibo_moe_select_algo: what the composite calls run per workload, and which requests cannot be met."""
+    from bibo_amd import ops
+    assert ops.select_algo(8192, 768, 64, 6, 384) == "fused"            # prefill workload
+    assert ops.select_algo(16384, 768, 64, 6, 384) == "fused"
+    assert ops.select_algo(64, 1024, 64, 6, 512) == "stream"            # decode workload: 6 rows per expert
+    assert ops.select_algo(512, 512, 64, 6, 256) == "fused"             # 48 rows per expert: past the streaming limit
+    assert ops.select_algo(400, 512, 64, 6, 256) == "stream"            # 37.5 rows, register-resident weight rows
+    assert ops.select_algo(341, 1024, 64, 6, 512) == "mfma"             # 32 rows of 2 KB: tiles win, I = 512 is not fused
+    assert ops.select_algo(8192, 768, 64, 6, 384, L.DTYPE_F32) == "generic"
+    assert ops.select_algo(8192, 768, 64, 6, 384, algo="mfma") == "mfma"
+    with pytest.raises(RuntimeError, match="does not support"):
+        ops.select_algo(8192, 768, 64, 6, 384, L.DTYPE_F32, algo="fused")
+    with pytest.raises(RuntimeError, match="does not support"):
+        ops.select_algo(64, 1000, 64, 6, 500, algo="stream")
+    out = ctypes.c_int(0)
+    assert L.lib().bibo_moe_select_algo(None, 0, ctypes.byref(out)) == -1
+
+
 def test_cpu_tensors_are_refused_loudly():
     x = torch.zeros(4, 64, dtype=torch.bfloat16)
     with pytest.raises(RuntimeError, match="GPU"):
