@@ -47,17 +47,25 @@ __global__ __launch_bounds__(256) void scatter_kernel(const int32_t* __restrict_
   constexpr int kPerWg = kPermTokens / HT;          // histograms that cover this workgroup's tokens
   const int h0 = b * kPerWg;                        // the first of them
 
+  // this wave's slots, requested before anything else: their latency passes behind the histogram sums
+  constexpr int kSlotIters = (kPermTokens / 4) * kMaxK / kWave;   // 32 tokens x at most 8 slots / 64 lanes
+  int ev[kSlotIters];
+#pragma unroll
+  for (int it = 0; it < kSlotIters; ++it) {
+    const int s = s0 + it * kWave + lane;
+    ev[it] = (s < s1) ? idx[s] : -1;
+  }
+
   int mycnt = 0;                                  // slots of expert `lane` among this wave's tokens
   if constexpr (HT == kPermTokens) {
-    for (int base = s0; base < s1; base += kWave) {
-      const int s = base + lane;
-      int e = 0;
-      bool valid = s < s1;
-      if (valid) { e = idx[s]; valid = (unsigned)e < (unsigned)E; }
-      if (!valid) e = 0;
-      unsigned long long peers, mine;
-      match64(e, valid, lane, peers, mine);
-      mycnt += __popcll(mine);
+#pragma unroll
+    for (int it = 0; it < kSlotIters; ++it) {
+      if (s0 + it * kWave < s1) {
+        const bool valid = s0 + it * kWave + lane < s1 && (unsigned)ev[it] < (unsigned)E;
+        unsigned long long peers, mine;
+        match64(valid ? ev[it] : 0, valid, lane, peers, mine);
+        mycnt += __popcll(mine);
+      }
     }
   } else {
 #pragma unroll
@@ -97,17 +105,19 @@ __global__ __launch_bounds__(256) void scatter_kernel(const int32_t* __restrict_
   int cnt = excl + before;                        // next free row of expert `lane` for this wave
   for (int ww = 0; ww < wave; ++ww) cnt += wave_cnt[ww][lane];
 
-  for (int base = s0; base < s1; base += kWave) {
-    const int s = base + lane;
-    int e = 0;
-    bool valid = s < s1;
-    if (valid) { e = idx[s]; valid = (unsigned)e < (unsigned)E; }
-    if (!valid) e = 0;
-    unsigned long long peers, mine;
-    match64(e, valid, lane, peers, mine);
-    const int pos = __shfl(cnt, e, kWave) + __popcll(peers & lt);
-    if (valid) { perm_slot[pos] = s; perm_token[pos] = s / k; }
-    cnt += __popcll(mine);
+#pragma unroll
+  for (int it = 0; it < kSlotIters; ++it) {
+    const int base = s0 + it * kWave;
+    if (base < s1) {
+      const int s = base + lane;
+      const bool valid = s < s1 && (unsigned)ev[it] < (unsigned)E;
+      const int e = valid ? ev[it] : 0;
+      unsigned long long peers, mine;
+      match64(e, valid, lane, peers, mine);
+      const int pos = __shfl(cnt, e, kWave) + __popcll(peers & lt);
+      if (valid) { perm_slot[pos] = s; perm_token[pos] = s / k; }
+      cnt += __popcll(mine);
+    }
   }
 }
 
