@@ -135,6 +135,23 @@ def test_streaming_kernels_match_oracle(T, H, I, k, theta):
     assert rel_err(out, gen) <= 1e-2
 
 
+@pytest.mark.parametrize("T,H,I,E,k", [(69, 1536, 512, 64, 8), (36, 1024, 576, 4, 1), (56, 1088, 128, 64, 1),
+                                       (61, 192, 1024, 8, 2), (5, 768, 64, 4, 2), (19, 64, 384, 64, 6),
+                                       (77, 512, 1024, 64, 6), (39, 64, 512, 8, 6), (18, 1536, 1024, 8, 2),
+                                       (15, 256, 576, 4, 4)])
+def test_streaming_kernels_over_odd_shapes(T, H, I, E, k):
+    """Rows that are not whole 256-element chunks, I above the fused-activation width (activation as its own launch),
+    rows longer than the two register chunks (refilled every pass), few experts with many rows each."""
+    p = O.make_inputs(T=T, H=H, E=E, k=k, I=I, bias="uniform", theta="normal", seed=T * 7 + H)
+    idx, w = _route(p)
+    ref = O.experts_forward(p["x"], idx, w, p["w_gate_up"], p["w_down"], p["theta"])
+    out, counts = _gpu_experts(p, idx, w, "stream")
+    assert rel_err(out, ref) <= BF16_TOL
+    assert np.array_equal(counts, O.permute(idx, E)[0])
+    gen, _ = _gpu_experts(p, idx, w, "generic")
+    assert rel_err(out, gen) <= 1e-2
+
+
 def test_streaming_kernels_without_the_permutation_pass():
     """Without a counts request the composite call launches no permutation: the streaming kernels scan the
     routing indices themselves.  Same bits either way."""
