@@ -49,7 +49,8 @@ int resolve_algo(int algo, int T, int H, int E, int k, int I, int dtype, bool co
       *out = BIBO_ALGO_MFMA;
       break;
     case BIBO_ALGO_STREAM:
-      if (!composite || !stream_supported(H, I, dtype)) return BIBO_ERR_UNSUPPORTED;
+      // more rows per expert than the limit: refused here, before anything is launched
+      if (!composite || !stream_eligible(T, H, E, k, I, dtype)) return BIBO_ERR_UNSUPPORTED;
       *out = BIBO_ALGO_STREAM;
       break;
     case BIBO_ALGO_FUSED:
