@@ -21,9 +21,10 @@
 //
 //   gateup_stream_kernel : raw gate/up pre-activations gu[slot, 0..2I) bf16        (src/modeling/ffn/moe.py:84)
 //   down_stream_kernel   : streams w_down and writes routing-weighted rows in slot order (moe.py:92-93);
-//                          for I <= 512 it also turns the expert's pre-activations into the operand rows,
-//                          hidden = r^p SiLU(g/r) up (moe.py:87-92), while the weights are on their way
-//   activate_rows_kernel : the same activation as a launch of its own, for wider I
+//                          for I <= 512 and at most 16 rows per expert on average it also turns the expert's
+//                          pre-activations into the operand rows, hidden = r^p SiLU(g/r) up (moe.py:87-92),
+//                          while the weights are on their way
+//   activate_rows_kernel : the same activation as a launch of its own, for wider I or more rows
 #include "common.h"
 
 namespace bibo {
