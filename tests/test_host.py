@@ -84,6 +84,12 @@ def test_kernel_family_selection_is_exported():
     assert L.lib().bibo_moe_select_algo(None, 0, ctypes.byref(out)) == -1
 
 
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess, sys
+    r = subprocess.run([sys.executable, str(ROOT / "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0 and "one GPU" in (r.stderr + r.stdout)
+
+
 def test_cpu_tensors_are_refused_loudly():
     x = torch.zeros(4, 64, dtype=torch.bfloat16)
     with pytest.raises(RuntimeError, match="GPU"):
