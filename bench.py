@@ -93,8 +93,8 @@ class Layer:
             self._stages.update({
                 "gateup_down": (self.lib.bibo_moe_gateup_down_fwd,
                                 (P(self.x), P(self.wgu), P(self.wd), P(self.theta), P(self.w), P(self.offsets),
-                                 P(self.perm_slot), P(self.perm_token), T, H, E, k, I, L.DTYPE_BF16, P(self.yw),
-                                 self.stream)),
+                                 P(self.perm_slot), P(self.perm_token), T, H, E, k, I, L.DTYPE_BF16,
+                                 L.ACT_RADIAL_SIGMOID, P(self.yw), self.stream)),
                 "combine": (self.lib.bibo_moe_combine_fwd, (P(self.yw), 1, T, H, k, L.DTYPE_BF16, P(self.out), self.stream)),
             })
         else:
@@ -102,7 +102,7 @@ class Layer:
             self._stages.update({
                 "gateup": (self.lib.bibo_moe_gateup_fwd,
                            (P(self.x), P(self.wgu), P(self.theta), P(self.offsets), P(self.perm_token), T, H, E, k, I,
-                            L.DTYPE_BF16, stage_algo, P(self.hidden), self.stream)),
+                            L.DTYPE_BF16, stage_algo, L.ACT_RADIAL_SIGMOID, P(self.hidden), self.stream)),
                 "down_combine": (self.lib.bibo_moe_down_combine_fwd,
                                  (P(self.hidden), P(self.wd), P(self.w), P(self.offsets), P(self.perm_slot), T, H, E, k, I,
                                   L.DTYPE_BF16, stage_algo, P(self.out), P(self.ws), self.ws.numel(), self.stream)),

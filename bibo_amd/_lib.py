@@ -13,7 +13,9 @@ DTYPE_BF16, DTYPE_F32 = 0, 1
 NORM_NONE, NORM_SUM, NORM_SOFTMAX = 0, 1, 2
 ALGO_AUTO, ALGO_GENERIC, ALGO_MFMA, ALGO_STREAM, ALGO_FUSED = 0, 1, 2, 3, 4
 MAX_EXPERTS, MAX_TOPK = 64, 8
-ABI_VERSION = 2
+ACT_RADIAL_SIGMOID, ACT_RADIAL_TANH, ACT_SILU = 0, 1, 2
+FLAG_ROUND_BLOCK_OUT = 1
+ABI_VERSION = 3
 
 # every symbol include/bibo_moe.h declares
 SYMBOLS = (
@@ -26,7 +28,8 @@ SYMBOLS = (
 
 class Shape(ctypes.Structure):
     _fields_ = [("T", ctypes.c_int32), ("H", ctypes.c_int32), ("E", ctypes.c_int32), ("k", ctypes.c_int32),
-                ("I", ctypes.c_int32), ("dtype", ctypes.c_int32), ("n_pos", ctypes.c_int32), ("n_neg", ctypes.c_int32)]
+                ("I", ctypes.c_int32), ("dtype", ctypes.c_int32), ("n_pos", ctypes.c_int32), ("n_neg", ctypes.c_int32),
+                ("act", ctypes.c_int32), ("flags", ctypes.c_int32)]
 
 
 _lock = threading.Lock()
@@ -48,11 +51,11 @@ def _declare(l):
     l.bibo_moe_permute.restype = ci
     l.bibo_moe_permute.argtypes = [vp, ci, ci, ci, vp, vp, vp, vp, vp, sz, vp]
     l.bibo_moe_gateup_fwd.restype = ci
-    l.bibo_moe_gateup_fwd.argtypes = [vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, vp, vp]
+    l.bibo_moe_gateup_fwd.argtypes = [vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, ci, vp, vp]
     l.bibo_moe_down_combine_fwd.restype = ci
     l.bibo_moe_down_combine_fwd.argtypes = [vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, vp, vp, sz, vp]
     l.bibo_moe_gateup_down_fwd.restype = ci
-    l.bibo_moe_gateup_down_fwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, vp, vp]
+    l.bibo_moe_gateup_down_fwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, vp, vp]
     l.bibo_moe_combine_fwd.restype = ci
     l.bibo_moe_combine_fwd.argtypes = [vp, ci, ci, ci, ci, ci, vp, vp]
     l.bibo_moe_combine_ex_fwd.restype = ci

@@ -11,7 +11,8 @@ class BiBoMoEConfig:
                  num_routed_experts=6, special_expert_pairs=1, pos_identity_expert=True, neg_identity_expert=True,
                  num_pos_identity_experts=None, num_neg_identity_experts=None, use_shared_expert=False,
                  shared_expert_type="mlp", num_shared_experts=1, norm_topk_prob="sum", bias_update_factor=None,
-                 bias_update_threshold=8000, initializer_range=0.02, hidden_act="silu", **unused):
+                 bias_update_threshold=8000, initializer_range=0.02, hidden_act="silu", kernel_size=3,
+                 radial_p="sigmoid", expert_act="radial", **unused):
         self.hidden_size = hidden_size
         self.intermediate_size = intermediate_size
         self.num_experts_per_tok = num_experts_per_tok
@@ -37,6 +38,11 @@ class BiBoMoEConfig:
         self.bias_update_threshold = 8000 if bias_update_threshold is None else bias_update_threshold
         self.initializer_range = initializer_range
         self.hidden_act = hidden_act
+        self.kernel_size = kernel_size          # causal Conv1d of the conv shared expert (configuration_bibo.py:56,124)
+        # not fields of the reference's config: its harness keeps them in two module globals
+        # (RADIAL_P / EXPERT_ACT, ablate/common/patches.py:53-69)
+        self.radial_p = radial_p
+        self.expert_act = expert_act
         if not 1 <= num_experts_per_tok <= num_routed_experts:
             raise ValueError(f"num_experts_per_tok ({num_experts_per_tok}) must be in "
                              f"[1, num_routed_experts={num_routed_experts}]")

@@ -10,6 +10,9 @@ constexpr size_t kAlign = 256;
 inline size_t align_up(size_t v) { return (v + kAlign - 1) & ~(kAlign - 1); }
 inline size_t elt_size(int dtype) { return dtype == BIBO_DTYPE_BF16 ? 2 : 4; }
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+inline bool aligned_ws(const void* p) { return (reinterpret_cast<uintptr_t>(p) & (kAlign - 1)) == 0; }
+
+inline bool act_ok(int act) { return act >= BIBO_ACT_RADIAL_SIGMOID && act <= BIBO_ACT_SILU; }
 
 int check_dims(int T, int H, int E, int k, int I, int dtype, int n_pos = 0, int n_neg = 0) {
   if (n_pos < 0 || n_neg < 0 || n_pos + n_neg >= E) return BIBO_ERR_BAD_SHAPE;     // at least one GLU expert
@@ -28,18 +31,21 @@ inline long long stream_rows_per_expert(int H, int I) {
   return H <= 768 ? 32 : 24;
 }
 
-inline bool stream_eligible(int T, int H, int E, int k, int I, int dtype) {
+// `distinct`: the k experts of a token are known to differ (indices that come straight from the router kernel), so
+// one expert gets at most T rows.  A caller's indices may name an expert several times per token, up to all T*k
+// slots on one expert, and the row list of a streaming workgroup holds kStreamMaxRows entries.
+inline bool stream_eligible(int T, int H, int E, int k, int I, int dtype, bool distinct) {
   return stream_supported(H, I, dtype) && (long long)T * k <= stream_rows_per_expert(H, I) * E &&
-         (long long)T * k <= kStreamMaxSlots && T <= kStreamMaxRows;
+         (long long)T * k <= kStreamMaxSlots && (distinct ? T : (long long)T * k) <= kStreamMaxRows;
 }
 
 // `composite`: the caller is bibo_moe_experts_fwd / bibo_moe_forward, the only entry points that can run
 // the streaming kernels (they hand bf16 pre-activations, not `hidden`, from one kernel to the next) and
 // the fused kernel (its activations never reach memory).
-int resolve_algo(int algo, int T, int H, int E, int k, int I, int dtype, bool composite, int* out) {
+int resolve_algo(int algo, int T, int H, int E, int k, int I, int dtype, bool composite, bool distinct, int* out) {
   switch (algo) {
     case BIBO_ALGO_AUTO:
-      if (composite && stream_eligible(T, H, E, k, I, dtype)) *out = BIBO_ALGO_STREAM;
+      if (composite && stream_eligible(T, H, E, k, I, dtype, distinct)) *out = BIBO_ALGO_STREAM;
       else if (composite && fused_supported(H, I, dtype)) *out = BIBO_ALGO_FUSED;
       else *out = mfma_supported(H, I, dtype) ? BIBO_ALGO_MFMA : BIBO_ALGO_GENERIC;
       break;
@@ -50,7 +56,7 @@ int resolve_algo(int algo, int T, int H, int E, int k, int I, int dtype, bool co
       break;
     case BIBO_ALGO_STREAM:
       // more rows per expert than the limit: refused here, before anything is launched
-      if (!composite || !stream_eligible(T, H, E, k, I, dtype)) return BIBO_ERR_UNSUPPORTED;
+      if (!composite || !stream_eligible(T, H, E, k, I, dtype, distinct)) return BIBO_ERR_UNSUPPORTED;
       *out = BIBO_ALGO_STREAM;
       break;
     case BIBO_ALGO_FUSED:
@@ -82,7 +88,7 @@ Workspace carve(int T, int H, int E, int k, int I, int dtype) {
   ws.perm_token = o; o += align_up(S * sizeof(int32_t));
   ws.hidden = o;     o += align_up(S * (size_t)I * elt_size(dtype));
   // bf16 gate/up pre-activations, only ever used when the streaming kernels are eligible
-  ws.gu = o;         o += align_up(stream_eligible(T, H, E, k, I, dtype) ? S * (size_t)2 * I * sizeof(bf16_t) : 0);
+  ws.gu = o;         o += align_up(stream_eligible(T, H, E, k, I, dtype, true) ? S * (size_t)2 * I * sizeof(bf16_t) : 0);
   ws.yw = o;         o += align_up(S * (size_t)H * sizeof(float));
   ws.total = o;
   return ws;
@@ -91,13 +97,13 @@ Workspace carve(int T, int H, int E, int k, int I, int dtype) {
 inline int hip_rc(hipError_t e) { return e == hipSuccess ? BIBO_OK : (int)e; }
 
 int gateup_dispatch(const void* x, const void* wgu, const float* theta, const int32_t* offsets,
-                    const int32_t* perm_token, int T, int H, int E, int k, int I, int dtype, int algo, void* hidden,
-                    hipStream_t s) {
+                    const int32_t* perm_token, int T, int H, int E, int k, int I, int dtype, int algo, int act,
+                    void* hidden, hipStream_t s) {
   if (algo == BIBO_ALGO_MFMA) {
     if (!aligned16(x) || !aligned16(wgu) || !aligned16(hidden)) return BIBO_ERR_MISALIGNED;
-    return hip_rc(launch_gateup_mfma(x, wgu, theta, offsets, perm_token, T, H, E, k, I, hidden, s));
+    return hip_rc(launch_gateup_mfma(x, wgu, theta, offsets, perm_token, T, H, E, k, I, act, hidden, s));
   }
-  return hip_rc(launch_gateup_generic(x, wgu, theta, offsets, perm_token, T, H, E, k, I, dtype, hidden, s));
+  return hip_rc(launch_gateup_generic(x, wgu, theta, offsets, perm_token, T, H, E, k, I, dtype, act, hidden, s));
 }
 
 // E here and in gateup_dispatch counts the GLU experts (those that have weights)
@@ -123,30 +129,31 @@ int down_dispatch(const void* hidden, const void* wd, const float* w, const int3
 int experts_dispatch(const void* x, const void* wgu, const void* wd, const float* theta, const int32_t* idx,
                      const float* w, const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token,
                      const void* residual, bool idx_trusted, int T, int H, int Eg, int np, int nn, int k, int I, int dtype,
-                     int algo, void* out, char* base, const Workspace& ws, hipStream_t s) {
+                     int algo, int act, int flags, void* out, char* base, const Workspace& ws, hipStream_t s) {
   float* yw = reinterpret_cast<float*>(base + ws.yw);
   CombineArgs ca;
   ca.residual = residual;
+  ca.round_block = (residual != nullptr && (flags & BIBO_FLAG_ROUND_BLOCK_OUT)) ? 1 : 0;   // layers.py:62-63
   // indices that come straight from the router kernel are in range; a caller's may hold padding values, whose
   // slots the combine has to skip; specials are the combine's work either way (moe.py:95-99)
   if (!idx_trusted || np + nn > 0) { ca.idx = idx; ca.w = w; ca.x = x; ca.E_glu = Eg; ca.n_pos = np; ca.n_neg = nn; }
   if (algo == BIBO_ALGO_STREAM) {
     if (!aligned16(x) || !aligned16(wgu) || !aligned16(wd)) return BIBO_ERR_MISALIGNED;
-    if (!stream_eligible(T, H, Eg + np + nn, k, I, dtype)) return BIBO_ERR_UNSUPPORTED;   // no pre-activation segment carved
+    if (!stream_eligible(T, H, Eg + np + nn, k, I, dtype, idx_trusted)) return BIBO_ERR_UNSUPPORTED;   // no pre-activation segment carved, or more rows than a row list holds
     void* gu = base + ws.gu;
     hipError_t e = launch_gateup_stream(x, wgu, idx, T, H, Eg, k, I, gu, s);
     if (e != hipSuccess) return (int)e;
-    e = launch_down_stream(gu, wd, theta, w, idx, T, H, Eg, k, I, base + ws.hidden, yw, s);
+    e = launch_down_stream(gu, wd, theta, w, idx, T, H, Eg, k, I, act, base + ws.hidden, yw, s);
     if (e != hipSuccess) return (int)e;
     return hip_rc(launch_combine(yw, 0, ca, T, H, k, dtype, out, s));
   }
   if (algo == BIBO_ALGO_FUSED) {
     if (!aligned16(x) || !aligned16(wgu) || !aligned16(wd)) return BIBO_ERR_MISALIGNED;
-    hipError_t e = launch_experts_fused(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, T, H, Eg, k, I, yw, s);
+    hipError_t e = launch_experts_fused(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, T, H, Eg, k, I, act, yw, s);
     if (e != hipSuccess) return (int)e;
     return hip_rc(launch_combine(yw, 1, ca, T, H, k, dtype, out, s));
   }
-  const int rc = gateup_dispatch(x, wgu, theta, offsets, perm_token, T, H, Eg, k, I, dtype, algo, base + ws.hidden, s);
+  const int rc = gateup_dispatch(x, wgu, theta, offsets, perm_token, T, H, Eg, k, I, dtype, algo, act, base + ws.hidden, s);
   if (rc != BIBO_OK) return rc;
   return down_dispatch(base + ws.hidden, wd, w, offsets, perm_slot, ca, T, H, Eg, k, I, dtype, algo, out, yw, s);
 }
@@ -161,11 +168,13 @@ int forward_impl(const void* x, const void* w_router, const float* bias, const v
   int rc = check_dims(T, H, E, k, I, dtype, sh->n_pos, sh->n_neg);
   if (rc != BIBO_OK) return rc;
   const int Eg = E - sh->n_pos - sh->n_neg;
-  if (norm_mode < BIBO_NORM_NONE || norm_mode > BIBO_NORM_SOFTMAX) return BIBO_ERR_UNSUPPORTED;
+  if (norm_mode < BIBO_NORM_NONE || norm_mode > BIBO_NORM_SOFTMAX || !act_ok(sh->act)) return BIBO_ERR_UNSUPPORTED;
   int a;
-  if ((rc = resolve_algo(algo, T, H, E, k, I, dtype, true, &a)) != BIBO_OK) return rc;
+  if ((rc = resolve_algo(algo, T, H, E, k, I, dtype, true, true, &a)) != BIBO_OK) return rc;
   if (!workspace) return BIBO_ERR_NULL_POINTER;
-  if (T > 0 && (!x || !w_router || !bias || !w_gate_up || !w_down || !theta || !out)) return BIBO_ERR_NULL_POINTER;
+  if (!aligned_ws(workspace)) return BIBO_ERR_MISALIGNED;
+  if (T > 0 && (!x || !w_router || !bias || !w_gate_up || !w_down || !out)) return BIBO_ERR_NULL_POINTER;
+  if (T > 0 && !theta && sh->act != BIBO_ACT_SILU) return BIBO_ERR_NULL_POINTER;
   const Workspace ws = carve(T, H, E, k, I, dtype);
   if (workspace_bytes < ws.total) return BIBO_ERR_WORKSPACE_TOO_SMALL;
   char* base = static_cast<char*>(workspace);
@@ -195,7 +204,7 @@ int forward_impl(const void* x, const void* w_router, const float* bias, const v
   }
   if (T == 0) return BIBO_OK;
   return experts_dispatch(x, w_gate_up, w_down, theta, idx, w, offsets, perm_slot, perm_token, residual, true, T, H, Eg,
-                          sh->n_pos, sh->n_neg, k, I, dtype, a, out, base, ws, s);
+                          sh->n_pos, sh->n_neg, k, I, dtype, a, sh->act, sh->flags, out, base, ws, s);
 }
 
 
@@ -213,7 +222,7 @@ const char* bibo_moe_strerror(int code) {
       return "bad shape: need T >= 0, H, I >= 1, 1 <= E <= 64, 1 <= k <= min(E, 8), n_pos, n_neg >= 0, n_pos + n_neg < E";
     case BIBO_ERR_BAD_DTYPE: return "dtype must be BIBO_DTYPE_BF16 or BIBO_DTYPE_F32";
     case BIBO_ERR_WORKSPACE_TOO_SMALL: return "workspace smaller than bibo_moe_workspace_bytes() for this shape";
-    case BIBO_ERR_MISALIGNED: return "tensor base pointers must be 16-byte aligned";
+    case BIBO_ERR_MISALIGNED: return "tensor base pointers must be 16-byte aligned and the workspace 256-byte aligned";
     case BIBO_ERR_UNSUPPORTED: return "requested kernel family does not support this shape or dtype";
     default: break;
   }
@@ -233,7 +242,7 @@ int bibo_moe_select_algo(const bibo_moe_shape* sh, int algo, int* selected) {
   if (sh == nullptr || selected == nullptr) return BIBO_ERR_NULL_POINTER;
   const int rc = check_dims(sh->T, sh->H, sh->E, sh->k, sh->I, sh->dtype, sh->n_pos, sh->n_neg);
   if (rc != BIBO_OK) return rc;
-  return resolve_algo(algo, sh->T, sh->H, sh->E, sh->k, sh->I, sh->dtype, true, selected);
+  return resolve_algo(algo, sh->T, sh->H, sh->E, sh->k, sh->I, sh->dtype, true, true, selected);
 }
 
 int bibo_moe_router_fwd(const void* x, const void* w_router, const float* bias, int T, int H, int E, int k, int dtype,
@@ -259,15 +268,16 @@ int bibo_moe_permute(const int32_t* idx, int T, int E, int k, int32_t* counts, i
 }
 
 int bibo_moe_gateup_fwd(const void* x, const void* w_gate_up, const float* theta, const int32_t* offsets,
-                        const int32_t* perm_token, int T, int H, int E, int k, int I, int dtype, int algo, void* hidden,
-                        void* stream) {
+                        const int32_t* perm_token, int T, int H, int E, int k, int I, int dtype, int algo, int act,
+                        void* hidden, void* stream) {
   int rc = check_dims(T, H, E, k, I, dtype);
   if (rc != BIBO_OK) return rc;
+  if (!act_ok(act)) return BIBO_ERR_UNSUPPORTED;
   int a;
-  if ((rc = resolve_algo(algo, T, H, E, k, I, dtype, false, &a)) != BIBO_OK) return rc;
+  if ((rc = resolve_algo(algo, T, H, E, k, I, dtype, false, false, &a)) != BIBO_OK) return rc;
   if (T == 0) return BIBO_OK;
-  if (!x || !w_gate_up || !theta || !offsets || !perm_token || !hidden) return BIBO_ERR_NULL_POINTER;
-  return gateup_dispatch(x, w_gate_up, theta, offsets, perm_token, T, H, E, k, I, dtype, a, hidden,
+  if (!x || !w_gate_up || (!theta && act != BIBO_ACT_SILU) || !offsets || !perm_token || !hidden) return BIBO_ERR_NULL_POINTER;
+  return gateup_dispatch(x, w_gate_up, theta, offsets, perm_token, T, H, E, k, I, dtype, a, act, hidden,
                          static_cast<hipStream_t>(stream));
 }
 
@@ -277,9 +287,10 @@ int bibo_moe_down_combine_fwd(const void* hidden, const void* w_down, const floa
   int rc = check_dims(T, H, E, k, I, dtype);
   if (rc != BIBO_OK) return rc;
   int a;
-  if ((rc = resolve_algo(algo, T, H, E, k, I, dtype, false, &a)) != BIBO_OK) return rc;
+  if ((rc = resolve_algo(algo, T, H, E, k, I, dtype, false, false, &a)) != BIBO_OK) return rc;
   if (T == 0) return BIBO_OK;
   if (!hidden || !w_down || !w || !offsets || !perm_slot || !out || !workspace) return BIBO_ERR_NULL_POINTER;
+  if (!aligned_ws(workspace)) return BIBO_ERR_MISALIGNED;       // the slot rows live there, 16 bytes at a time
   if (workspace_bytes < (size_t)T * k * H * sizeof(float)) return BIBO_ERR_WORKSPACE_TOO_SMALL;
   return down_dispatch(hidden, w_down, w, offsets, perm_slot, CombineArgs{}, T, H, E, k, I, dtype, a, out,
                        static_cast<float*>(workspace), static_cast<hipStream_t>(stream));
@@ -287,17 +298,17 @@ int bibo_moe_down_combine_fwd(const void* hidden, const void* w_down, const floa
 
 int bibo_moe_gateup_down_fwd(const void* x, const void* w_gate_up, const void* w_down, const float* theta,
                              const float* w, const int32_t* offsets, const int32_t* perm_slot,
-                             const int32_t* perm_token, int T, int H, int E, int k, int I, int dtype, void* yw,
-                             void* stream) {
+                             const int32_t* perm_token, int T, int H, int E, int k, int I, int dtype, int act,
+                             void* yw, void* stream) {
   const int rc = check_dims(T, H, E, k, I, dtype);
   if (rc != BIBO_OK) return rc;
-  if (!fused_supported(H, I, dtype)) return BIBO_ERR_UNSUPPORTED;
+  if (!fused_supported(H, I, dtype) || !act_ok(act)) return BIBO_ERR_UNSUPPORTED;
   if (T == 0) return BIBO_OK;
-  if (!x || !w_gate_up || !w_down || !theta || !w || !offsets || !perm_slot || !perm_token || !yw)
+  if (!x || !w_gate_up || !w_down || (!theta && act != BIBO_ACT_SILU) || !w || !offsets || !perm_slot || !perm_token || !yw)
     return BIBO_ERR_NULL_POINTER;
   if (!aligned16(x) || !aligned16(w_gate_up) || !aligned16(w_down) || !aligned16(yw)) return BIBO_ERR_MISALIGNED;
-  return hip_rc(launch_experts_fused(x, w_gate_up, w_down, theta, w, offsets, perm_slot, perm_token, T, H, E, k, I, yw,
-                                     static_cast<hipStream_t>(stream)));
+  return hip_rc(launch_experts_fused(x, w_gate_up, w_down, theta, w, offsets, perm_slot, perm_token, T, H, E, k, I, act,
+                                     yw, static_cast<hipStream_t>(stream)));
 }
 
 int bibo_moe_combine_fwd(const void* yw, int yw_is_bf16, int T, int H, int k, int dtype, void* out, void* stream) {
@@ -332,10 +343,14 @@ int bibo_moe_experts_fwd(const void* x, const int32_t* idx, const float* w, cons
   int rc = check_dims(T, H, E, k, I, dtype, sh->n_pos, sh->n_neg);
   if (rc != BIBO_OK) return rc;
   const int Eg = E - sh->n_pos - sh->n_neg;
+  if (!act_ok(sh->act)) return BIBO_ERR_UNSUPPORTED;
   int a;
-  if ((rc = resolve_algo(algo, T, H, E, k, I, dtype, true, &a)) != BIBO_OK) return rc;
+  // a caller's indices may repeat an expert inside a token (moe.py:46-71 accepts that)
+  if ((rc = resolve_algo(algo, T, H, E, k, I, dtype, true, false, &a)) != BIBO_OK) return rc;
   if (!workspace) return BIBO_ERR_NULL_POINTER;
-  if (T > 0 && (!x || !idx || !w || !w_gate_up || !w_down || !theta || !out)) return BIBO_ERR_NULL_POINTER;
+  if (!aligned_ws(workspace)) return BIBO_ERR_MISALIGNED;
+  if (T > 0 && (!x || !idx || !w || !w_gate_up || !w_down || !out)) return BIBO_ERR_NULL_POINTER;
+  if (T > 0 && !theta && sh->act != BIBO_ACT_SILU) return BIBO_ERR_NULL_POINTER;
   const Workspace ws = carve(T, H, E, k, I, dtype);
   if (workspace_bytes < ws.total) return BIBO_ERR_WORKSPACE_TOO_SMALL;
   char* base = static_cast<char*>(workspace);
@@ -351,7 +366,7 @@ int bibo_moe_experts_fwd(const void* x, const int32_t* idx, const float* w, cons
     return rc;
   if (T == 0) return BIBO_OK;
   return experts_dispatch(x, w_gate_up, w_down, theta, idx, w, offsets, perm_slot, perm_token, nullptr, false, T, H, Eg,
-                          sh->n_pos, sh->n_neg, k, I, dtype, a, out, base, ws, s);
+                          sh->n_pos, sh->n_neg, k, I, dtype, a, sh->act, 0, out, base, ws, s);
 }
 
 int bibo_moe_forward(const void* x, const void* w_router, const float* bias, const void* w_gate_up, const void* w_down,
@@ -387,6 +402,7 @@ int bibo_moe_ffn_forward(const void* h, const float* norm_weight, float eps, con
   const int rc = check_dims(sh->T, sh->H, sh->E, sh->k, sh->I, sh->dtype, sh->n_pos, sh->n_neg);
   if (rc != BIBO_OK) return rc;
   if (!workspace) return BIBO_ERR_NULL_POINTER;
+  if (!aligned_ws(workspace)) return BIBO_ERR_MISALIGNED;
   if (sh->T > 0 && (!h || !norm_weight || !out)) return BIBO_ERR_NULL_POINTER;
   const size_t inner = carve(sh->T, sh->H, sh->E, sh->k, sh->I, sh->dtype).total;
   const size_t xn_bytes = align_up((size_t)sh->T * sh->H * elt_size(sh->dtype));

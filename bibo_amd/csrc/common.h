@@ -84,6 +84,23 @@ __device__ __forceinline__ float sigmoid32_canonical(float x) {
   return (float)(1.0 / d);
 }
 
+// Exponent p of the radial gain r^p for expert activation `act` (enum bibo_act): sigmoid(theta) as the
+// reference module computes it (src/modeling/ffn/moe.py:89) or tanh(theta) (act code 10 of
+// ablate/common/patches.py:53-61).  Plain SwiGLU has no gain: callers set r = 1 and never read theta.
+__device__ __forceinline__ float radial_exponent(const float* __restrict__ theta, int e, int act) {
+  if (act == BIBO_ACT_SILU) return 0.f;
+  const float t = theta[e];
+  return act == BIBO_ACT_RADIAL_TANH ? tanhf(t) : 1.f / (1.f + expf(-t));
+}
+
+// (1/r, r^p) of a row from its sum of squared gate values: r^2 = sum / I + eps (moe.py:88); plain SwiGLU: (1, 1).
+__device__ __forceinline__ void radial_row_scalars(float sum_sq, int I, float p, int act, float& rinv, float& gain) {
+  if (act == BIBO_ACT_SILU) { rinv = 1.f; gain = 1.f; return; }
+  const float r2 = sum_sq * (1.f / (float)I) + kNormSiluEps;
+  rinv = __builtin_amdgcn_rsqf(r2);
+  gain = __builtin_amdgcn_exp2f(0.5f * p * __builtin_amdgcn_logf(r2));       // r^p = 2^(p/2 * log2 r^2)
+}
+
 // Ballot ranking of 64 consecutive slots.  `peers` = lanes whose slot has my expert, `mine` = lanes whose
 // slot has the expert whose id is my lane id.
 __device__ __forceinline__ void match64(int e, bool valid, int lane, unsigned long long& peers,
@@ -123,8 +140,8 @@ hipError_t launch_permute_from_hist(const int32_t* idx, int T, int E, int k, con
                                     int32_t* counts, int32_t* offsets, int32_t* perm_slot, int32_t* perm_token,
                                     hipStream_t s);
 hipError_t launch_gateup_generic(const void* x, const void* wgu, const float* theta, const int32_t* offsets,
-                                 const int32_t* perm_token, int T, int H, int E, int k, int I, int dtype, void* hidden,
-                                 hipStream_t s);
+                                 const int32_t* perm_token, int T, int H, int E, int k, int I, int dtype, int act,
+                                 void* hidden, hipStream_t s);
 hipError_t launch_down_generic(const void* hidden, const void* wd, const float* w, const int32_t* offsets,
                                const int32_t* perm_slot, int T, int H, int E, int k, int I, int dtype, float* yw,
                                hipStream_t s);
@@ -135,6 +152,7 @@ struct CombineArgs {
   const void* x = nullptr;         // [T,H] in the output dtype; needed for specials
   int E_glu = 0, n_pos = 0, n_neg = 0;
   const void* residual = nullptr;  // [T,H] in the output dtype
+  int round_block = 0;             // round the sum of the slot rows to the output dtype before the residual is added
 };
 hipError_t launch_combine(const void* yw, int yw_is_bf16, const CombineArgs& a, int T, int H, int k, int dtype,
                           void* out, hipStream_t s);
@@ -142,18 +160,19 @@ hipError_t launch_rmsnorm(const void* x, const float* weight, float eps, int T, 
                           hipStream_t s);
 bool mfma_supported(int H, int I, int dtype);
 hipError_t launch_gateup_mfma(const void* x, const void* wgu, const float* theta, const int32_t* offsets,
-                              const int32_t* perm_token, int T, int H, int E, int k, int I, void* hidden, hipStream_t s);
+                              const int32_t* perm_token, int T, int H, int E, int k, int I, int act, void* hidden,
+                              hipStream_t s);
 hipError_t launch_down_mfma(const void* hidden, const void* wd, const float* w, const int32_t* offsets,
                             const int32_t* perm_slot, int T, int H, int E, int k, int I, void* yw, hipStream_t s);
 
 bool fused_supported(int H, int I, int dtype);
 hipError_t launch_experts_fused(const void* x, const void* wgu, const void* wd, const float* theta, const float* w,
                                 const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token, int T,
-                                int H, int E, int k, int I, void* yw, hipStream_t s);
+                                int H, int E, int k, int I, int act, void* yw, hipStream_t s);
 bool stream_supported(int H, int I, int dtype);
 hipError_t launch_gateup_stream(const void* x, const void* wgu, const int32_t* idx, int T, int H, int E, int k, int I,
                                 void* gu, hipStream_t s);
 hipError_t launch_down_stream(const void* gu, const void* wd, const float* theta, const float* w, const int32_t* idx,
-                              int T, int H, int E, int k, int I, void* hidden, float* yw, hipStream_t s);
+                              int T, int H, int E, int k, int I, int act, void* hidden, float* yw, hipStream_t s);
 
 }  // namespace bibo

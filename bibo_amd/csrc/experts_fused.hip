@@ -56,7 +56,7 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
                                                             const int32_t* __restrict__ offsets,
                                                             const int32_t* __restrict__ perm_slot,
                                                             const int32_t* __restrict__ perm_token, int H, int E,
-                                                            bf16_t* __restrict__ yw) {
+                                                            int act, bf16_t* __restrict__ yw) {
   using F = FusedShape<NT, CT>;
   using S1 = typename F::S1;
   constexpr int MT = F::MT, BM = F::BM, I = F::I, NTW = 2 * NT;
@@ -124,11 +124,9 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
   }
   __syncthreads();
   if (tid < BM) {
-    const float p = 1.f / (1.f + __expf(-theta[e]));                                  // moe.py:89
+    const float p = radial_exponent(theta, e, act);                                   // moe.py:89
     const float ms = ((ssq[tid] + ssq[BM + tid]) + ssq[2 * BM + tid]) + ssq[3 * BM + tid];
-    const float r2 = ms * (1.f / (float)I) + kNormSiluEps;                            // r^2, moe.py:88
-    rinv_s[tid] = __builtin_amdgcn_rsqf(r2);
-    gain_s[tid] = __builtin_amdgcn_exp2f(0.5f * p * __builtin_amdgcn_logf(r2));       // r^p
+    radial_row_scalars(ms, I, p, act, rinv_s[tid], gain_s[tid]);                      // 1/r and r^p, moe.py:88-89
     const int slot = perm_slot[row0 + min(tid, rows - 1)];
     slot_s[tid] = slot;
     w_s[tid] = w[slot];
@@ -260,19 +258,19 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
 template <int NT, int CT>
 void launch_fused_t(const bf16_t* x, const bf16_t* wgu, const bf16_t* wd, const float* theta, const float* w,
                     const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token, int S, int H, int E,
-                    bf16_t* yw, hipStream_t s) {
+                    int act, bf16_t* yw, hipStream_t s) {
   const int grid = ((S / 128 + E + 7) & ~7) + 8;
   hipLaunchKernelGGL((experts_fused_kernel<NT, CT>), dim3(grid), dim3(512), 0, s, x, wgu, wd, theta, w, offsets,
-                     perm_slot, perm_token, H, E, yw);
+                     perm_slot, perm_token, H, E, act, yw);
 }
 
 template <int NT>
 void launch_fused_nt(const bf16_t* x, const bf16_t* wgu, const bf16_t* wd, const float* theta, const float* w,
                      const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token, int S, int H, int E,
-                     bf16_t* yw, hipStream_t s) {
-  if (H % 384 == 0) launch_fused_t<NT, 3>(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, S, H, E, yw, s);
-  else if (H % 256 == 0) launch_fused_t<NT, 2>(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, S, H, E, yw, s);
-  else launch_fused_t<NT, 1>(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, S, H, E, yw, s);
+                     int act, bf16_t* yw, hipStream_t s) {
+  if (H % 384 == 0) launch_fused_t<NT, 3>(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, S, H, E, act, yw, s);
+  else if (H % 256 == 0) launch_fused_t<NT, 2>(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, S, H, E, act, yw, s);
+  else launch_fused_t<NT, 1>(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, S, H, E, act, yw, s);
 }
 
 }  // namespace
@@ -284,7 +282,7 @@ bool fused_supported(int H, int I, int dtype) {
 
 hipError_t launch_experts_fused(const void* x, const void* wgu, const void* wd, const float* theta, const float* w,
                                 const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token, int T,
-                                int H, int E, int k, int I, void* yw, hipStream_t s) {
+                                int H, int E, int k, int I, int act, void* yw, hipStream_t s) {
   const int S = T * k;
   if (S == 0) return hipSuccess;
   const bf16_t* xp = static_cast<const bf16_t*>(x);
@@ -292,9 +290,9 @@ hipError_t launch_experts_fused(const void* x, const void* wgu, const void* wd, 
   const bf16_t* dp = static_cast<const bf16_t*>(wd);
   bf16_t* yp = static_cast<bf16_t*>(yw);
   switch (I) {
-    case 128: launch_fused_nt<1>(xp, gp, dp, theta, w, offsets, perm_slot, perm_token, S, H, E, yp, s); break;
-    case 256: launch_fused_nt<2>(xp, gp, dp, theta, w, offsets, perm_slot, perm_token, S, H, E, yp, s); break;
-    case 384: launch_fused_nt<3>(xp, gp, dp, theta, w, offsets, perm_slot, perm_token, S, H, E, yp, s); break;
+    case 128: launch_fused_nt<1>(xp, gp, dp, theta, w, offsets, perm_slot, perm_token, S, H, E, act, yp, s); break;
+    case 256: launch_fused_nt<2>(xp, gp, dp, theta, w, offsets, perm_slot, perm_token, S, H, E, act, yp, s); break;
+    case 384: launch_fused_nt<3>(xp, gp, dp, theta, w, offsets, perm_slot, perm_token, S, H, E, act, yp, s); break;
     default: return hipErrorInvalidValue;
   }
   return hipGetLastError();

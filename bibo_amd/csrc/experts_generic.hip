@@ -21,7 +21,7 @@ __global__ __launch_bounds__(256) void gateup_generic_kernel(const TIn* __restri
                                                              const float* __restrict__ theta,
                                                              const int32_t* __restrict__ offsets,
                                                              const int32_t* __restrict__ perm_token, int H, int E,
-                                                             int I, TIn* __restrict__ hidden) {
+                                                             int I, int act, TIn* __restrict__ hidden) {
   extern __shared__ float smem[];
   float* xs = smem;            // [H]
   float* gu = smem + H;        // [2I]
@@ -49,9 +49,9 @@ __global__ __launch_bounds__(256) void gateup_generic_kernel(const TIn* __restri
   if (lane == 0) red[wave] = ss;
   __syncthreads();
   const float ms = ((red[0] + red[1]) + red[2]) + red[3];
-  const float r = sqrtf(ms / (float)I + kNormSiluEps);                 // moe.py:88
-  const float p = 1.f / (1.f + expf(-theta[e]));                       // moe.py:89
-  const float gain = powf(r, p);
+  const float r = act == BIBO_ACT_SILU ? 1.f : sqrtf(ms / (float)I + kNormSiluEps);   // moe.py:88
+  const float p = radial_exponent(theta, e, act);                      // moe.py:89
+  const float gain = act == BIBO_ACT_SILU ? 1.f : powf(r, p);
   for (int i = tid; i < I; i += 256) {
     const float z = gu[i] / r;
     const float act = z / (1.f + expf(-z)) * gain;                     // SiLU(g/r) * r^p
@@ -119,7 +119,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const TY* __restrict__ yw,
       }
       acc += to_float(yw[(t * k + j) * H + h]);
     }
-    if (residual != nullptr) acc += to_float(residual[i]);
+    if (residual != nullptr) acc = (a.round_block ? to_float(from_float<TOut>(acc)) : acc) + to_float(residual[i]);
     out[i] = from_float<TOut>(acc);
   }
 }
@@ -152,7 +152,7 @@ __global__ __launch_bounds__(256) void combine_bf16x8_kernel(const bf16_t* __res
     if (a.residual != nullptr) {
       const bf16x8 r = reinterpret_cast<const bf16x8*>(a.residual)[i];
 #pragma unroll
-      for (int q = 0; q < 8; ++q) acc[q] += (float)r[q];
+      for (int q = 0; q < 8; ++q) acc[q] = (a.round_block ? (float)(bf16_t)acc[q] : acc[q]) + (float)r[q];
     }
     bf16x8 o;
 #pragma unroll
@@ -164,18 +164,18 @@ __global__ __launch_bounds__(256) void combine_bf16x8_kernel(const bf16_t* __res
 }  // namespace
 
 hipError_t launch_gateup_generic(const void* x, const void* wgu, const float* theta, const int32_t* offsets,
-                                 const int32_t* perm_token, int T, int H, int E, int k, int I, int dtype, void* hidden,
-                                 hipStream_t s) {
+                                 const int32_t* perm_token, int T, int H, int E, int k, int I, int dtype, int act,
+                                 void* hidden, hipStream_t s) {
   const int S = T * k;
   if (S == 0) return hipSuccess;
   const size_t shm = (size_t)(H + 2 * I) * sizeof(float);
   if (dtype == BIBO_DTYPE_BF16)
     hipLaunchKernelGGL(gateup_generic_kernel<bf16_t>, dim3(S), dim3(256), shm, s, static_cast<const bf16_t*>(x),
-                       static_cast<const bf16_t*>(wgu), theta, offsets, perm_token, H, E, I,
+                       static_cast<const bf16_t*>(wgu), theta, offsets, perm_token, H, E, I, act,
                        static_cast<bf16_t*>(hidden));
   else
     hipLaunchKernelGGL(gateup_generic_kernel<float>, dim3(S), dim3(256), shm, s, static_cast<const float*>(x),
-                       static_cast<const float*>(wgu), theta, offsets, perm_token, H, E, I,
+                       static_cast<const float*>(wgu), theta, offsets, perm_token, H, E, I, act,
                        static_cast<float*>(hidden));
   return hipGetLastError();
 }

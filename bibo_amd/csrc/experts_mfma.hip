@@ -26,7 +26,7 @@ __global__ __launch_bounds__(256 * WM) void gateup_dma_kernel(const bf16_t* __re
                                                               const float* __restrict__ theta,
                                                               const int32_t* __restrict__ offsets,
                                                               const int32_t* __restrict__ perm_token, int H, int E,
-                                                              bf16_t* __restrict__ hidden) {
+                                                              int act, bf16_t* __restrict__ hidden) {
   constexpr int NTW = 2 * NT;
   using S = Stripe<MT, NTW, WM>;
   constexpr int BM = S::BM;
@@ -85,11 +85,9 @@ __global__ __launch_bounds__(256 * WM) void gateup_dma_kernel(const bf16_t* __re
   }
   __syncthreads();                       // also: every wave is done reading the stage buffers
   if (tid < BM) {
-    const float p = 1.f / (1.f + __expf(-theta[e]));                                  // moe.py:89
+    const float p = radial_exponent(theta, e, act);                                   // moe.py:89
     const float ms = ((ssq[tid] + ssq[BM + tid]) + ssq[2 * BM + tid]) + ssq[3 * BM + tid];
-    const float r2 = ms * (1.f / (float)I) + kNormSiluEps;                            // r^2, moe.py:88
-    rinv_s[tid] = __builtin_amdgcn_rsqf(r2);
-    gain_s[tid] = __builtin_amdgcn_exp2f(0.5f * p * __builtin_amdgcn_logf(r2));       // r^p = 2^(p/2 * log2 r^2)
+    radial_row_scalars(ms, I, p, act, rinv_s[tid], gain_s[tid]);                      // 1/r and r^p, moe.py:88-89
   }
   __syncthreads();
   constexpr int kOutCols = NT * 32;                 // gate-paired columns owned by this wave
@@ -221,11 +219,11 @@ inline int round_up8(int v) { return (v + 7) & ~7; }
 
 template <int MT, int NT, int WM>
 void launch_gateup_dma_t(const bf16_t* x, const bf16_t* wgu, const float* theta, const int32_t* offsets,
-                         const int32_t* perm_token, int S, int H, int E, bf16_t* hidden, hipStream_t s) {
+                         const int32_t* perm_token, int S, int H, int E, int act, bf16_t* hidden, hipStream_t s) {
   constexpr int BM = 32 * MT * WM;
   const int grid = round_up8(S / BM + E) + 8;
   hipLaunchKernelGGL((gateup_dma_kernel<MT, NT, WM>), dim3(grid), dim3(256 * WM), 0, s, x, wgu, theta, offsets,
-                     perm_token, H, E, hidden);
+                     perm_token, H, E, act, hidden);
 }
 
 template <int MT, int NTW, int WM, typename TY, int BK = kBK>
@@ -257,7 +255,7 @@ bool mfma_supported(int H, int I, int dtype) {
 }
 
 hipError_t launch_gateup_mfma(const void* x, const void* wgu, const float* theta, const int32_t* offsets,
-                              const int32_t* perm_token, int T, int H, int E, int k, int I, void* hidden,
+                              const int32_t* perm_token, int T, int H, int E, int k, int I, int act, void* hidden,
                               hipStream_t s) {
   const int S = T * k;
   if (S == 0) return hipSuccess;
@@ -265,10 +263,10 @@ hipError_t launch_gateup_mfma(const void* x, const void* wgu, const float* theta
   const bf16_t* wp = static_cast<const bf16_t*>(wgu);
   bf16_t* hp = static_cast<bf16_t*>(hidden);
   switch (I) {
-    case 128: launch_gateup_dma_t<2, 1, 2>(xp, wp, theta, offsets, perm_token, S, H, E, hp, s); break;
-    case 256: launch_gateup_dma_t<2, 2, 2>(xp, wp, theta, offsets, perm_token, S, H, E, hp, s); break;
-    case 384: launch_gateup_dma_t<2, 3, 2>(xp, wp, theta, offsets, perm_token, S, H, E, hp, s); break;
-    case 512: launch_gateup_dma_t<1, 4, 2>(xp, wp, theta, offsets, perm_token, S, H, E, hp, s); break;
+    case 128: launch_gateup_dma_t<2, 1, 2>(xp, wp, theta, offsets, perm_token, S, H, E, act, hp, s); break;
+    case 256: launch_gateup_dma_t<2, 2, 2>(xp, wp, theta, offsets, perm_token, S, H, E, act, hp, s); break;
+    case 384: launch_gateup_dma_t<2, 3, 2>(xp, wp, theta, offsets, perm_token, S, H, E, act, hp, s); break;
+    case 512: launch_gateup_dma_t<1, 4, 2>(xp, wp, theta, offsets, perm_token, S, H, E, act, hp, s); break;
     default: return hipErrorInvalidValue;
   }
   return hipGetLastError();

@@ -53,7 +53,9 @@ __device__ __forceinline__ void scan_issue(ScanRegs& r, const int32_t* __restric
 }
 
 // Slots routed to expert e, ascending, into rows_s; returns how many.  All 256 threads call it; ends with a
-// barrier.  Only the ceil(S / 256) index groups that hold slots are looked at.
+// barrier.  Only the ceil(S / 256) index groups that hold slots are looked at.  The host only launches these
+// kernels when no expert can get more than kStreamMaxRows rows; entries past the list's end are dropped rather
+// than written all the same.
 __device__ __forceinline__ int scan_finish(const ScanRegs& r, int S, int e, unsigned short* rows_s, int* cnt_s) {
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const unsigned long long lt = (1ull << lane) - 1ull;
@@ -73,12 +75,13 @@ __device__ __forceinline__ int scan_finish(const ScanRegs& r, int S, int e, unsi
     if (q < nq) {
 #pragma unroll
       for (int ww = 0; ww < 4; ++ww) {
-        if (ww == wave && r.v[q] == e) rows_s[run + rank[q]] = (unsigned short)(q * 256 + tid);
+        if (ww == wave && r.v[q] == e && run + rank[q] < kStreamMaxRows)
+          rows_s[run + rank[q]] = (unsigned short)(q * 256 + tid);
         run += cnt_s[q * 4 + ww];
       }
     }
   __syncthreads();
-  return run;
+  return min(run, kStreamMaxRows);
 }
 
 struct WChunk {
@@ -216,7 +219,7 @@ void gateup_stream_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict
 
 // One workgroup per slot: hidden[slot] = r^p SiLU(g/r) up from the bf16 pre-activations (moe.py:87-92).
 __global__ __launch_bounds__(256) void activate_rows_kernel(const bf16_t* __restrict__ gu, const float* __restrict__ theta,
-                                                            const int32_t* __restrict__ idx, int E, int I,
+                                                            const int32_t* __restrict__ idx, int E, int I, int act,
                                                             bf16_t* __restrict__ hidden) {
   __shared__ float red[4];
   const int slot = blockIdx.x;
@@ -229,9 +232,8 @@ __global__ __launch_bounds__(256) void activate_rows_kernel(const bf16_t* __rest
   ss = wave_sum(ss);
   if (lane == 0) red[wave] = ss;
   __syncthreads();
-  const float r2 = (((red[0] + red[1]) + red[2]) + red[3]) / (float)I + kNormSiluEps;    // moe.py:88
-  const float p = 1.f / (1.f + __expf(-theta[e]));                                        // moe.py:89
-  const float rinv = rsqrtf(r2), gain = __expf(0.5f * p * __logf(r2));                     // 1/r, r^p
+  float rinv, gain;                                                                       // 1/r, r^p (moe.py:88-89)
+  radial_row_scalars(((red[0] + red[1]) + red[2]) + red[3], I, radial_exponent(theta, e, act), act, rinv, gain);
   for (int i = tid; i < I; i += 256) {
     const float z = (float)grow[i] * rinv;
     hidden[(size_t)slot * I + i] = (bf16_t)(z / (1.f + __expf(-z)) * gain * (float)grow[I + i]);
@@ -245,7 +247,7 @@ __global__ __launch_bounds__(256) void activate_rows_kernel(const bf16_t* __rest
 // first round's loads are requested ahead of chunk `b` of the weights, like the rows in stage_rows.
 // I <= kFusedActMaxI.
 template <bool kWhole>
-__device__ __forceinline__ void stage_activated(const bf16_t* __restrict__ gu, float theta_e,
+__device__ __forceinline__ void stage_activated(const bf16_t* __restrict__ gu, float p, int act,
                                                 const unsigned short* rows_s, int r0, int nrow, int I, bf16_t* hs,
                                                 WChunk& b, const bf16_t* __restrict__ wp, int nlines, bool load_b) {
   constexpr int kPer = kFusedActMaxI / 8 / 32;                 // granules per thread and half at 32 threads per row
@@ -253,7 +255,6 @@ __device__ __forceinline__ void stage_activated(const bf16_t* __restrict__ gu, f
   const int tpr = nrow <= 4 ? 64 : 32;
   const int row_in = tid / tpr, part = tid - row_in * tpr;
   const int gran = I / 8;
-  const float p = 1.f / (1.f + __expf(-theta_e));                                          // moe.py:89
   for (int rb = 0; rb < nrow; rb += 256 / tpr) {
     const int row = rb + row_in;
     const bool live = row < nrow;                              // whole groups of tpr lanes are live or not
@@ -276,8 +277,8 @@ __device__ __forceinline__ void stage_activated(const bf16_t* __restrict__ gu, f
         for (int q = 0; q < 8; ++q) ss = fmaf((float)g[j][q], (float)g[j][q], ss);
       }
     for (int o = tpr >> 1; o > 0; o >>= 1) ss += __shfl_xor(ss, o, kWave);   // the row's threads are adjacent lanes
-    const float r2 = ss / (float)I + kNormSiluEps;                                        // moe.py:88
-    const float rinv = rsqrtf(r2), gain = __expf(0.5f * p * __logf(r2));                   // 1/r, r^p
+    float rinv, gain;                                                                     // 1/r, r^p (moe.py:88-89)
+    radial_row_scalars(ss, I, p, act, rinv, gain);
     const float nrl = -1.4426950408889634f * rinv, rg = rinv * gain;
 #pragma unroll
     for (int j = 0; j < kPer; ++j) {
@@ -298,13 +299,13 @@ __device__ __forceinline__ void stage_activated(const bf16_t* __restrict__ gu, f
   }
 }
 
-// grid = (H / 64, E).  yw[slot, c] = w[slot] * (hidden[slot] . w_down[e, c, :]).  kFusedAct: `act` holds the bf16
-// gate/up pre-activations [slot, 2I] and the activation happens here; otherwise it holds hidden [slot, I].
+// grid = (H / 64, E).  yw[slot, c] = w[slot] * (hidden[slot] . w_down[e, c, :]).  kFusedAct: `rows_in` holds the bf16
+// gate/up pre-activations [slot, 2I] and the activation `act` happens here; otherwise it holds hidden [slot, I].
 // kWhole: I is a whole number of chunks.
 template <bool kFusedAct, bool kWhole>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4)))
-void down_stream_kernel(const bf16_t* __restrict__ act, const bf16_t* __restrict__ wd, const float* __restrict__ theta,
-                        const float* __restrict__ w, const int32_t* __restrict__ idx, int S, int H, int I,
+void down_stream_kernel(const bf16_t* __restrict__ rows_in, const bf16_t* __restrict__ wd, const float* __restrict__ theta,
+                        const float* __restrict__ w, const int32_t* __restrict__ idx, int S, int H, int I, int act,
                         float* __restrict__ yw) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   __shared__ unsigned short rows_s[kStreamMaxRows];
@@ -318,7 +319,7 @@ void down_stream_kernel(const bf16_t* __restrict__ act, const bf16_t* __restrict
   const bool resident = nlines <= 2 * kChunk;
   ScanRegs sr;
   scan_issue(sr, idx, S);
-  const float theta_e = kFusedAct ? theta[e] : 0.f;
+  const float p_e = kFusedAct ? radial_exponent(theta, e, act) : 0.f;                       // moe.py:89
   WChunk ca, cb;
   load_chunk<kWhole>(ca, wp, 0, nlines);
   const int n = scan_finish(sr, S, e, rows_s, cnt_s);
@@ -329,8 +330,8 @@ void down_stream_kernel(const bf16_t* __restrict__ act, const bf16_t* __restrict
       __syncthreads();
       if (reload) load_chunk<kWhole>(ca, wp, 0, nlines);
     }
-    if (kFusedAct) stage_activated<kWhole>(act, theta_e, rows_s, r0, nrow, I, hs, cb, wp, nlines, reload);
-    else stage_rows<kWhole>(act, rows_s, r0, nrow, 1, I, hs, cb, wp, nlines, reload);
+    if (kFusedAct) stage_activated<kWhole>(rows_in, p_e, act, rows_s, r0, nrow, I, hs, cb, wp, nlines, reload);
+    else stage_rows<kWhole>(rows_in, rows_s, r0, nrow, 1, I, hs, cb, wp, nlines, reload);
     __syncthreads();
     // the fused activation is only used up to I = kFusedActMaxI = two chunks
     const floatx4 acc = stream_rows<kWhole, kFusedAct>(wp, hs, I, lane, ca, cb);
@@ -368,7 +369,7 @@ hipError_t launch_gateup_stream(const void* x, const void* wgu, const int32_t* i
 }
 
 hipError_t launch_down_stream(const void* gu, const void* wd, const float* theta, const float* w, const int32_t* idx,
-                              int T, int H, int E, int k, int I, void* hidden, float* yw, hipStream_t s) {
+                              int T, int H, int E, int k, int I, int act, void* hidden, float* yw, hipStream_t s) {
   if (T * k == 0) return hipSuccess;
   if (T * k > kStreamMaxSlots || T > kStreamMaxRows) return hipErrorInvalidValue;
   const size_t shm = (size_t)kTok * (I + 8) * sizeof(bf16_t);
@@ -379,13 +380,13 @@ hipError_t launch_down_stream(const void* gu, const void* wd, const float* theta
   // The fused activation is computed by every one of the H/64 workgroups of an expert, once per 16-row pass:
   // cheap next to a launch for one pass, not for several
   if (I <= kFusedActMaxI && T * k <= kTok * E) {
-    if (whole) hipLaunchKernelGGL((down_stream_kernel<true, true>), grid, dim3(256), shm, s, g, wdp, theta, w, idx, T * k, H, I, yw);
-    else hipLaunchKernelGGL((down_stream_kernel<true, false>), grid, dim3(256), shm, s, g, wdp, theta, w, idx, T * k, H, I, yw);
+    if (whole) hipLaunchKernelGGL((down_stream_kernel<true, true>), grid, dim3(256), shm, s, g, wdp, theta, w, idx, T * k, H, I, act, yw);
+    else hipLaunchKernelGGL((down_stream_kernel<true, false>), grid, dim3(256), shm, s, g, wdp, theta, w, idx, T * k, H, I, act, yw);
   } else {
     bf16_t* hp = static_cast<bf16_t*>(hidden);
-    hipLaunchKernelGGL(activate_rows_kernel, dim3(T * k), dim3(256), 0, s, g, theta, idx, E, I, hp);
-    if (whole) hipLaunchKernelGGL((down_stream_kernel<false, true>), grid, dim3(256), shm, s, hp, wdp, theta, w, idx, T * k, H, I, yw);
-    else hipLaunchKernelGGL((down_stream_kernel<false, false>), grid, dim3(256), shm, s, hp, wdp, theta, w, idx, T * k, H, I, yw);
+    hipLaunchKernelGGL(activate_rows_kernel, dim3(T * k), dim3(256), 0, s, g, theta, idx, E, I, act, hp);
+    if (whole) hipLaunchKernelGGL((down_stream_kernel<false, true>), grid, dim3(256), shm, s, hp, wdp, theta, w, idx, T * k, H, I, act, yw);
+    else hipLaunchKernelGGL((down_stream_kernel<false, false>), grid, dim3(256), shm, s, hp, wdp, theta, w, idx, T * k, H, I, act, yw);
   }
   return hipGetLastError();
 }

@@ -28,10 +28,18 @@ def _forward_only_guard(*tensors):
 
 
 class _CastCache:
-    """Device copies of parameters in the dtype the kernels want, refreshed when the parameter changes."""
+    """Device copies of parameters in the dtype the kernels want, refreshed when the parameter changes.
+
+    A change is seen through the parameter's storage address, version counter, device and dtype.  In-place writes
+    through `p.data` (`p.data.copy_(...)`, `p.data.fill_(...)`) bump none of them; after such a write call
+    `invalidate()` (the modules below expose it as `refresh_weights()`), as `load_state_dict` and `Module._apply`
+    (`.to()`, `.cuda()`, `.bfloat16()`) do by themselves here."""
 
     def __init__(self):
         self._store = {}
+
+    def invalidate(self):
+        self._store.clear()
 
     def get(self, name: str, p: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
         if p.dtype == dtype and p.is_contiguous():
@@ -73,6 +81,15 @@ class BiBoMoERouter(nn.Module):
         self.gate_proj = nn.Linear(config.hidden_size, self.num_routed_experts, bias=False)
         nn.init.normal_(self.gate_proj.weight, mean=0.0, std=getattr(config, "initializer_range", 0.02))
         self._cache = _CastCache()
+        self.register_load_state_dict_post_hook(lambda module, incompatible: module._cache.invalidate())
+
+    def refresh_weights(self):
+        """Drop the cached kernel-dtype copies of weight and bias (needed after a write through `.data`)."""
+        self._cache.invalidate()
+
+    def _apply(self, fn, *a, **kw):
+        self._cache.invalidate()
+        return super()._apply(fn, *a, **kw)
 
     def _operands(self, hidden_states):
         cd = _compute_dtype(hidden_states)
@@ -128,7 +145,30 @@ class BiBoFusedExperts(nn.Module):
         nn.init.normal_(self.down_proj, mean=0.0, std=std)
         self.radial_theta = nn.Parameter(torch.zeros(self.num_glu_experts))
         self.algo = "auto"
+        # The reference module hardcodes p = sigmoid(theta) (moe.py:89); its harness switches the external kernel
+        # to p = tanh(theta) or to plain SwiGLU through two globals (RADIAL_P / EXPERT_ACT,
+        # ablate/common/patches.py:53-69).  Here they are attributes of the module.
+        self.radial_p = getattr(config, "radial_p", "sigmoid")
+        self.expert_act = getattr(config, "expert_act", "radial")
         self._cache = _CastCache()
+        self.register_load_state_dict_post_hook(lambda module, incompatible: module._cache.invalidate())
+
+    @property
+    def act(self) -> str:
+        if self.expert_act == "silu":
+            return "silu"
+        if self.expert_act != "radial" or self.radial_p not in ("sigmoid", "tanh"):
+            raise ValueError(f"expert_act={self.expert_act!r} / radial_p={self.radial_p!r}: expected 'radial' or 'silu' "
+                             "and 'sigmoid' or 'tanh'")
+        return "radial_tanh" if self.radial_p == "tanh" else "radial"
+
+    def refresh_weights(self):
+        """Drop the cached kernel-dtype copies of the weights (needed after a write through `.data`)."""
+        self._cache.invalidate()
+
+    def _apply(self, fn, *a, **kw):
+        self._cache.invalidate()
+        return super()._apply(fn, *a, **kw)
 
     def _weights(self, cd):
         return (self._cache.get("gu", self.gate_up_proj, cd), self._cache.get("dn", self.down_proj, cd),
@@ -145,7 +185,7 @@ class BiBoFusedExperts(nn.Module):
         w = top_k_weights.detach().to(torch.float32).contiguous()
         gu, dn, th = self._weights(cd)
         out, counts = ops.experts_fwd(x, idx, w, gu, dn, th, algo=self.algo, want_counts=_want_counts,
-                                      n_pos=self.num_pos, n_neg=self.num_neg)          # specials: moe.py:95-99
+                                      n_pos=self.num_pos, n_neg=self.num_neg, act=self.act)   # specials: moe.py:95-99
         out = out if out.dtype == hidden_states.dtype else out.to(hidden_states.dtype)   # moe.py:101
         return (out, counts) if _want_counts else out
 
@@ -169,6 +209,30 @@ class BiBoSharedMLP(nn.Module):
         return self.down_proj(nn.functional.silu(self.gate_proj(x)) * self.up_proj(x))         # mlp.py:34-35
 
 
+class BiBoCausalConv1D(nn.Module):
+    """The convolutional shared expert (src/modeling/ffn/experts.py:11-34): the gate is a causal Conv1d over the
+    sequence (left padding kernel_size - 1), up and down are linear; same parameter names, so
+    `shared_experts_list.0.*` of a reference checkpoint loads.  Dense over every token: stock operations."""
+
+    def __init__(self, config):
+        super().__init__()
+        act = getattr(config, "hidden_act", "silu")
+        if act != "silu":
+            raise NotImplementedError(f"shared expert with hidden_act={act!r}; only 'silu' is implemented")
+        self.hidden_size = config.hidden_size
+        self.intermediate_size = config.moe_intermediate_size
+        self.kernel_size_gate = int(getattr(config, "kernel_size", 3))
+        self.causal_padding_gate = self.kernel_size_gate - 1
+        self.gate_conv = nn.Conv1d(self.hidden_size, self.intermediate_size, self.kernel_size_gate, padding=0, bias=False)
+        self.up_proj = nn.Linear(self.hidden_size, self.intermediate_size, bias=False)
+        self.down_proj = nn.Linear(self.intermediate_size, self.hidden_size, bias=False)
+
+    def forward(self, x):
+        xp = nn.functional.pad(x.transpose(1, 2), (self.causal_padding_gate, 0))              # experts.py:26-27
+        gate = self.gate_conv(xp).transpose(1, 2)                                              # [B,S,I]
+        return self.down_proj(nn.functional.silu(gate) * self.up_proj(x))                      # experts.py:30
+
+
 class BiBoMoELayer(nn.Module):
     """Router + experts + balancing state (src/modeling/ffn/moe.py:104-183)."""
 
@@ -188,10 +252,11 @@ class BiBoMoELayer(nn.Module):
         if self.use_shared_expert:
             # moe.py:118-127.  The shared expert is a dense SwiGLU over every token: stock GEMMs, not part of the
             # sparse path, so it runs as ordinary tensor operations next to the library call.
-            if getattr(config, "shared_expert_type", "mlp") != "mlp":
-                raise NotImplementedError("shared_expert_type='conv' is not implemented; use 'mlp'")
-            n_sh = int(getattr(config, "num_shared_experts", 1))
-            self.shared_experts_list.append(BiBoSharedMLP(config, config.moe_intermediate_size * n_sh))
+            if getattr(config, "shared_expert_type", "mlp") == "conv":
+                self.shared_experts_list.append(BiBoCausalConv1D(config))
+            else:
+                n_sh = int(getattr(config, "num_shared_experts", 1))
+                self.shared_experts_list.append(BiBoSharedMLP(config, config.moe_intermediate_size * n_sh))
         self.gate = BiBoMoERouter(config)
 
     # ---- balancing (host logic over device tensors, moe.py:131-155) ----
@@ -254,7 +319,7 @@ class BiBoMoELayer(nn.Module):
             out, _, _, counts, _ = ops.moe_forward(x, wr, b, gu, dn, th, self.num_experts_per_tok,
                                                    norm=self.gate.norm_topk_prob, algo=self.experts.algo,
                                                    want_counts=balancing, n_pos=self.experts.num_pos,
-                                                   n_neg=self.experts.num_neg)
+                                                   n_neg=self.experts.num_neg, act=self.experts.act)
             out = out if out.dtype == hidden_states.dtype else out.to(hidden_states.dtype)
             top_idx = None
         out = out.view(bsz, seq, hdim)
@@ -268,20 +333,24 @@ class BiBoMoELayer(nn.Module):
 
     @_no_compile
     def ffn_forward(self, hidden_states: torch.Tensor, norm_weight: torch.Tensor, eps: float,
-                    bf16_stream: bool = False) -> torch.Tensor:
+                    bf16_stream: bool = False, bf16_moe_out: bool = False) -> torch.Tensor:
         """The caller's seam, BiBoDecoderLayer._ffn_forward (src/modeling/layers.py:57-67):
         `hidden_states + self(rmsnorm(hidden_states))` with `norm_weight`/`eps` of post_attention_layernorm
         (src/modeling/norm.py:19-24), as ONE library call: the norm feeds the block from the workspace and the
         residual is added in the combine kernel.  With hooks or a gap probe present, or with an fp32 stream
         under bf16 autocast, the block runs as in forward and norm and residual are ordinary tensor operations
-        around it."""
+        around it.  `bf16_stream` and `bf16_moe_out` are the decoder layer's two switches (layers.py:28,37):
+        the sum is cast to bf16, and the block's output is rounded to bf16 before it enters the sum."""
         bsz, seq, hdim = hidden_states.shape
         num_tokens = bsz * seq
-        if self._hooks_present() or self.use_shared_expert or hidden_states.dtype != _compute_dtype(hidden_states):
+        if (self._hooks_present() or self.use_shared_expert or hidden_states.dtype != _compute_dtype(hidden_states)
+                or (bf16_moe_out and hidden_states.dtype != torch.bfloat16)):
             # (an fp32 residual stream under bf16 autocast keeps its fp32 norm and fp32 residual add)
             xf = hidden_states.float()
             xn = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)).to(hidden_states.dtype)    # norm.py:21-24
-            out = hidden_states + self.forward(norm_weight * xn).to(hidden_states.dtype)               # layers.py:60-64
+            blk = self.forward(norm_weight * xn)                                                       # layers.py:60-61
+            blk = blk.to(torch.bfloat16) if bf16_moe_out else blk                                      # layers.py:62-63
+            out = hidden_states + blk.to(hidden_states.dtype)                                          # layers.py:64
             return out.to(torch.bfloat16) if bf16_stream else out
         balancing = self.training and self.bias_update_factor > 0
         _forward_only_guard(hidden_states, self.gate.gate_proj.weight, self.experts.gate_up_proj)
@@ -294,7 +363,8 @@ class BiBoMoELayer(nn.Module):
         nw = norm_weight.detach().float().contiguous()
         out, _, _, counts = ops.ffn_forward(h, nw, float(eps), wr, b, gu, dn, th, self.num_experts_per_tok,
                                             norm=self.gate.norm_topk_prob, algo=self.experts.algo, want_counts=balancing,
-                                            n_pos=self.experts.num_pos, n_neg=self.experts.num_neg)
+                                            n_pos=self.experts.num_pos, n_neg=self.experts.num_neg, act=self.experts.act,
+                                            round_block_out=bf16_moe_out and cd == torch.bfloat16)
         if balancing:                                          # exactly once per training forward
             tpe = self._balance_step(None, num_tokens, counts=counts)
             if tpe is not None:

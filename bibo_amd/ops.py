@@ -12,6 +12,20 @@ _ALGO = {"auto": L.ALGO_AUTO, "generic": L.ALGO_GENERIC, "mfma": L.ALGO_MFMA, "s
          "fused": L.ALGO_FUSED}
 
 
+_ACT = {"radial": L.ACT_RADIAL_SIGMOID, "radial_sigmoid": L.ACT_RADIAL_SIGMOID, "sigmoid": L.ACT_RADIAL_SIGMOID,
+        "radial_tanh": L.ACT_RADIAL_TANH, "tanh": L.ACT_RADIAL_TANH, "silu": L.ACT_SILU}
+
+
+def act_code(v) -> int:
+    """Expert activation: 'radial' (= 'sigmoid', the reference module, kernel act code 8 of
+    ablate/common/patches.py:53-69), 'tanh' (code 10: p = tanh(theta)) or 'silu' (code 0: plain SwiGLU)."""
+    if isinstance(v, int) and not isinstance(v, bool):
+        return v
+    if v in _ACT:
+        return _ACT[v]
+    raise ValueError(f"act must be one of {sorted(_ACT)}, got {v!r}")
+
+
 def norm_mode(v) -> int:
     if isinstance(v, str) or isinstance(v, bool) or v is None:
         if v in _NORM:
@@ -116,7 +130,7 @@ def permute(idx, E):
     return counts, offsets, perm_slot, perm_token
 
 
-def gateup_fwd(x, w_gate_up, theta, offsets, perm_token, k, algo="auto"):
+def gateup_fwd(x, w_gate_up, theta, offsets, perm_token, k, algo="auto", act="radial"):
     """-> hidden [T*k, I] in x.dtype, rows in permuted order."""
     T, H = x.shape
     E, two_i, _ = w_gate_up.shape
@@ -127,7 +141,8 @@ def gateup_fwd(x, w_gate_up, theta, offsets, perm_token, k, algo="auto"):
     hidden = torch.empty(T * k, I, dtype=x.dtype, device=x.device)
     with torch.cuda.device(x.device):
         L.check(L.lib().bibo_moe_gateup_fwd(_ptr(x), _ptr(w_gate_up), _ptr(theta), _ptr(offsets), _ptr(perm_token),
-                                            T, H, E, k, I, dc, algo_code(algo), _ptr(hidden), _stream(x.device)),
+                                            T, H, E, k, I, dc, algo_code(algo), act_code(act), _ptr(hidden),
+                                            _stream(x.device)),
                 "bibo_moe_gateup_fwd")
     return hidden
 
@@ -149,7 +164,7 @@ def down_combine_fwd(hidden, w_down, w, offsets, perm_slot, T, algo="auto"):
     return out
 
 
-def gateup_down_fwd(x, w_gate_up, w_down, theta, w, offsets, perm_slot, perm_token):
+def gateup_down_fwd(x, w_gate_up, w_down, theta, w, offsets, perm_slot, perm_token, act="radial"):
     """Both projections in one launch -> yw [T*k, H] bf16, routing-weighted rows in slot order."""
     T, H = x.shape
     E, two_i, _ = w_gate_up.shape
@@ -164,7 +179,7 @@ def gateup_down_fwd(x, w_gate_up, w_down, theta, w, offsets, perm_slot, perm_tok
     with torch.cuda.device(x.device):
         L.check(L.lib().bibo_moe_gateup_down_fwd(_ptr(x), _ptr(w_gate_up), _ptr(w_down), _ptr(theta), _ptr(w),
                                                  _ptr(offsets), _ptr(perm_slot), _ptr(perm_token), T, H, E, k, I, dc,
-                                                 _ptr(yw), _stream(x.device)), "bibo_moe_gateup_down_fwd")
+                                                 act_code(act), _ptr(yw), _stream(x.device)), "bibo_moe_gateup_down_fwd")
     return yw
 
 
@@ -194,7 +209,7 @@ def combine_fwd(yw, T, k, dtype=None, idx=None, w=None, x=None, n_glu=0, n_pos=0
     return out
 
 
-def experts_fwd(x, idx, w, w_gate_up, w_down, theta, algo="auto", want_counts=False, n_pos=0, n_neg=0):
+def experts_fwd(x, idx, w, w_gate_up, w_down, theta, algo="auto", want_counts=False, n_pos=0, n_neg=0, act="radial"):
     """Seam 2.  x [T,H]; idx int32 [T,k]; w fp32 [T,k] -> out [T,H] (x.dtype), counts int32 [E]|None.
     The weight tensors hold the GLU experts; expert ids Eg .. Eg+n_pos-1 are +Identity, the next n_neg -Identity
     specials (moe.py:39-44,95-99), and E = Eg + n_pos + n_neg."""
@@ -211,7 +226,7 @@ def experts_fwd(x, idx, w, w_gate_up, w_down, theta, algo="auto", want_counts=Fa
     out = torch.empty(T, H, dtype=x.dtype, device=dev)
     counts = torch.empty(E, dtype=torch.int32, device=dev) if want_counts else None
     ws = workspace(dev, workspace_bytes(T, H, E, k, I, dc))
-    sh = L.Shape(T, H, E, k, I, dc, n_pos, n_neg)
+    sh = L.Shape(T, H, E, k, I, dc, n_pos, n_neg, act_code(act), 0)
     with torch.cuda.device(dev):
         L.check(L.lib().bibo_moe_experts_fwd(_ptr(x), _ptr(idx), _ptr(w), _ptr(w_gate_up), _ptr(w_down), _ptr(theta),
                                              ctypes.byref(sh), algo_code(algo), _ptr(out), _ptr(counts), _ptr(ws),
@@ -220,7 +235,7 @@ def experts_fwd(x, idx, w, w_gate_up, w_down, theta, algo="auto", want_counts=Fa
 
 
 def moe_forward(x, w_router, bias, w_gate_up, w_down, theta, k, norm="sum", algo="auto", want_routing=False,
-                want_counts=False, want_logits=False, n_pos=0, n_neg=0):
+                want_counts=False, want_logits=False, n_pos=0, n_neg=0, act="radial"):
     """Seam 1.  -> out [T,H], idx int32 [T,k]|None, w fp32 [T,k]|None, counts int32 [E]|None, logits fp32 [T,E]|None.
     w_router / bias have E = Eg + n_pos + n_neg rows, the expert weights Eg (see experts_fwd)."""
     T, H = x.shape
@@ -238,7 +253,7 @@ def moe_forward(x, w_router, bias, w_gate_up, w_down, theta, k, norm="sum", algo
     counts = torch.empty(E, dtype=torch.int32, device=dev) if want_counts else None
     logits = torch.empty(T, E, dtype=torch.float32, device=dev) if want_logits else None
     ws = workspace(dev, workspace_bytes(T, H, E, k, I, dc))
-    sh = L.Shape(T, H, E, k, I, dc, n_pos, n_neg)
+    sh = L.Shape(T, H, E, k, I, dc, n_pos, n_neg, act_code(act), 0)
     with torch.cuda.device(dev):
         L.check(L.lib().bibo_moe_forward(_ptr(x), _ptr(w_router), _ptr(bias), _ptr(w_gate_up), _ptr(w_down),
                                          _ptr(theta), ctypes.byref(sh), norm_mode(norm), algo_code(algo), _ptr(out),
@@ -259,8 +274,9 @@ def rmsnorm_fwd(x, norm_weight, eps):
 
 
 def ffn_forward(h, norm_weight, eps, w_router, bias, w_gate_up, w_down, theta, k, norm="sum", algo="auto",
-                want_routing=False, want_counts=False, n_pos=0, n_neg=0):
-    """Seam 3 (the block's caller).  -> out = h + moe(rmsnorm(h)) [T,H], idx|None, w|None, counts|None."""
+                want_routing=False, want_counts=False, n_pos=0, n_neg=0, act="radial", round_block_out=False):
+    """Seam 3 (the block's caller).  -> out = h + moe(rmsnorm(h)) [T,H], idx|None, w|None, counts|None.
+    round_block_out: round the block's output to h.dtype before the residual add (bf16_moe_out, layers.py:62-63)."""
     T, H = h.shape
     Eg, two_i, _ = w_gate_up.shape
     E = Eg + n_pos + n_neg
@@ -274,7 +290,7 @@ def ffn_forward(h, norm_weight, eps, w_router, bias, w_gate_up, w_down, theta, k
     idx = torch.empty(T, k, dtype=torch.int32, device=dev) if want_routing else None
     w = torch.empty(T, k, dtype=torch.float32, device=dev) if want_routing else None
     counts = torch.empty(E, dtype=torch.int32, device=dev) if want_counts else None
-    sh = L.Shape(T, H, E, k, I, dc, n_pos, n_neg)
+    sh = L.Shape(T, H, E, k, I, dc, n_pos, n_neg, act_code(act), L.FLAG_ROUND_BLOCK_OUT if round_block_out else 0)
     nbytes = ctypes.c_size_t(0)
     L.check(L.lib().bibo_moe_ffn_workspace_bytes(ctypes.byref(sh), ctypes.byref(nbytes)), "bibo_moe_ffn_workspace_bytes")
     ws = workspace(dev, nbytes.value)

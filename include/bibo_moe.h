@@ -37,7 +37,7 @@
 extern "C" {
 #endif
 
-#define BIBO_MOE_ABI_VERSION 2
+#define BIBO_MOE_ABI_VERSION 3
 #define BIBO_MOE_MAX_EXPERTS 64
 #define BIBO_MOE_MAX_TOPK 8
 
@@ -46,6 +46,25 @@ enum bibo_dtype { BIBO_DTYPE_BF16 = 0, BIBO_DTYPE_F32 = 1 };
 /* norm_topk_prob of the reference router (src/modeling/ffn/router.py:42-47) */
 enum bibo_norm_mode { BIBO_NORM_NONE = 0, BIBO_NORM_SUM = 1, BIBO_NORM_SOFTMAX = 2 };
 
+/*
+ * Activation of the GLU experts.  The reference module computes RADIAL_SIGMOID (src/modeling/ffn/moe.py:87-90);
+ * its training harness can switch the external kernel to the other two (act codes 8 / 10 / 0 of
+ * ablate/common/patches.py:53-69):
+ *   RADIAL_SIGMOID  r^p * SiLU(g/r) * up,  r = sqrt(mean_I(g^2) + 1e-6),  p = sigmoid(theta[e])     (code 8)
+ *   RADIAL_TANH     the same with p = tanh(theta[e]) in (-1, 1)                                      (code 10)
+ *   SILU            SiLU(g) * up, plain SwiGLU; theta is not read                                    (code 0)
+ * The value 0 is the reference module's behaviour, so a zero-initialised shape means what moe.py computes.
+ */
+enum bibo_act { BIBO_ACT_RADIAL_SIGMOID = 0, BIBO_ACT_RADIAL_TANH = 1, BIBO_ACT_SILU = 2 };
+
+/* bits of bibo_moe_shape.flags */
+enum bibo_flags {
+  /* bibo_moe_ffn_forward only: round the block's output to `dtype` before the residual is added, then round the sum
+     (bf16_moe_out of the reference's decoder layer, src/modeling/layers.py:37,62-63).  Without it the sum is formed
+     in fp32 and rounded once. */
+  BIBO_FLAG_ROUND_BLOCK_OUT = 1
+};
+
 /* kernel family for the expert GEMMs */
 enum bibo_algo {
   BIBO_ALGO_AUTO = 0,    /* pick by shape */
@@ -53,7 +72,10 @@ enum bibo_algo {
   BIBO_ALGO_MFMA = 2,    /* grouped bf16 MFMA tiles, one kernel per GEMM; needs bf16, H % 128 == 0 and
                             I in {128,256,384,512} */
   BIBO_ALGO_STREAM = 3,  /* weight-streaming kernels for few rows per expert (decode); bf16, H and I
-                            multiples of 64; only bibo_moe_experts_fwd / bibo_moe_forward, T*k <= 32*E */
+                            multiples of 64 up to 1728; only the composite entry points; T*k <= 40*E when
+                            H, I <= 512, 32*E up to H = 768, 24*E above, and at most 4096 slots and 2048 rows per
+                            expert: T <= 2048 for bibo_moe_forward / bibo_moe_ffn_forward (a token's experts are
+                            distinct), T*k <= 2048 for bibo_moe_experts_fwd (a caller's indices may repeat) */
   BIBO_ALGO_FUSED = 4    /* both GEMMs of a 128-row tile in one kernel, activations stay in LDS; bf16,
                             H % 128 == 0, I in {128,256,384}; only bibo_moe_experts_fwd / bibo_moe_forward */
 };
@@ -77,14 +99,18 @@ typedef struct bibo_moe_shape {
   int32_t dtype;
   int32_t n_pos; /* +Identity specials (moe.py:39-44,95-96): out += w * x; usually 0 */
   int32_t n_neg; /* -Identity specials (moe.py:97-99): out -= w * x; usually 0 */
-} bibo_moe_shape; /* w_gate_up, w_down and theta hold E - n_pos - n_neg (GLU) experts */
+  int32_t act;   /* enum bibo_act; 0 = the reference module's Radial NormSiLU */
+  int32_t flags; /* enum bibo_flags bits; 0 = none */
+} bibo_moe_shape; /* ten int32; w_gate_up, w_down and theta hold E - n_pos - n_neg (GLU) experts */
 
 int bibo_moe_abi_version(void);
 
 /* Static, NUL-terminated description of a negative code; for positive codes the HIP error string. */
 const char* bibo_moe_strerror(int code);
 
-/* Bytes of workspace that any entry point below needs for this shape (256-byte aligned base). */
+/* Bytes of workspace that any entry point below needs for this shape.  The base must be 256-byte aligned
+ * (segments are carved at multiples of 256 bytes and accessed 16 bytes at a time); every entry point that takes
+ * a workspace returns BIBO_ERR_MISALIGNED otherwise. */
 int bibo_moe_workspace_bytes(const bibo_moe_shape* shape, size_t* bytes);
 
 /*
@@ -124,12 +150,12 @@ int bibo_moe_permute(const int32_t* idx, int T, int E, int k, int32_t* counts, i
 
 /*
  * Grouped gate/up projection with the Radial NormSiLU epilogue r^p * SiLU(g/r) * up,
- * r = sqrt(mean_I(g^2) + 1e-6), p = sigmoid(theta[e]).  Replaces moe.py:81-90 and the
- * `activated * up` of moe.py:92.
+ * r = sqrt(mean_I(g^2) + 1e-6), p = sigmoid(theta[e]) (or the activation `act` names, enum bibo_act).
+ * Replaces moe.py:81-90 and the `activated * up` of moe.py:92.
  *   hidden  [T*k, I] in `dtype`, rows in permuted (sorted-by-expert) order
  */
 int bibo_moe_gateup_fwd(const void* x, const void* w_gate_up, const float* theta, const int32_t* offsets,
-                        const int32_t* perm_token, int T, int H, int E, int k, int I, int dtype, int algo,
+                        const int32_t* perm_token, int T, int H, int E, int k, int I, int dtype, int algo, int act,
                         void* hidden, void* stream);
 
 /*
@@ -150,8 +176,8 @@ int bibo_moe_down_combine_fwd(const void* hidden, const void* w_down, const floa
  */
 int bibo_moe_gateup_down_fwd(const void* x, const void* w_gate_up, const void* w_down, const float* theta,
                              const float* w, const int32_t* offsets, const int32_t* perm_slot,
-                             const int32_t* perm_token, int T, int H, int E, int k, int I, int dtype, void* yw,
-                             void* stream);
+                             const int32_t* perm_token, int T, int H, int E, int k, int I, int dtype, int act,
+                             void* yw, void* stream);
 
 /*
  * out[t, :] = sum_j yw[t*k + j, :], summed in fp32 in ascending j and rounded once to `dtype`

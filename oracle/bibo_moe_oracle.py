@@ -140,22 +140,30 @@ def permute(idx: np.ndarray, E: int):
 # --------------------------------------------------------------------------------------
 # experts (moe.py:73-101)
 # --------------------------------------------------------------------------------------
-def radial_normsilu(gate: torch.Tensor, theta_e: torch.Tensor) -> torch.Tensor:
+def radial_normsilu(gate: torch.Tensor, theta_e: torch.Tensor, act: str = "radial") -> torch.Tensor:
     """r^p * SiLU(g/r), r = sqrt(mean(g^2) + 1e-6) over the last dim, p = sigmoid(theta_e) (moe.py:87-89).
-    Computed in gate's dtype (pass fp32 or fp64)."""
+    Computed in gate's dtype (pass fp32 or fp64).
+
+    `act` selects what the reference's training harness can switch its external kernel to
+    (ablate/common/patches.py:53-69): "radial" = the module's own p = sigmoid(theta) (kernel act code 8),
+    "tanh" = p = tanh(theta) in (-1,1) (code 10), "silu" = plain SiLU(g), no norm and no gain (code 0)."""
+    if act == "silu":
+        return F.silu(gate)
     r = torch.sqrt(gate.square().mean(-1, keepdim=True) + NORMSILU_EPS)
-    p = torch.sigmoid(theta_e.to(gate.dtype))
+    t = theta_e.to(gate.dtype)
+    p = torch.tanh(t) if act == "tanh" else torch.sigmoid(t)
     return F.silu(gate / r) * r.pow(p)
 
 
-def expert_hidden(x_rows: torch.Tensor, w_gate_up_e: torch.Tensor, theta_e: torch.Tensor) -> torch.Tensor:
+def expert_hidden(x_rows: torch.Tensor, w_gate_up_e: torch.Tensor, theta_e: torch.Tensor, act: str = "radial") -> torch.Tensor:
     """act(gate) * up for one expert (moe.py:84-92).  w_gate_up_e [2I,H]: rows 0..I-1 gate, I..2I-1 up."""
     gu = x_rows @ w_gate_up_e.t()
     gate, up = gu.chunk(2, dim=-1)                                            # moe.py:85
-    return radial_normsilu(gate, theta_e) * up
+    return radial_normsilu(gate, theta_e, act) * up
 
 
-def experts_forward(x, idx, w, w_gate_up, w_down, theta, dtype=torch.float32, return_hidden=False, n_pos=0, n_neg=0):
+def experts_forward(x, idx, w, w_gate_up, w_down, theta, dtype=torch.float32, return_hidden=False, n_pos=0, n_neg=0,
+                    act="radial"):
     """Weighted sum over each token's experts, evaluated in `dtype` (moe.py:46-101).
 
     x [T,H]; idx [T,k] integer; w [T,k]; w_gate_up [Eg,2I,H]; w_down [Eg,H,I]; theta [Eg] hold the GLU experts;
@@ -184,7 +192,7 @@ def experts_forward(x, idx, w, w_gate_up, w_down, theta, dtype=torch.float32, re
             sign = 1.0 if e < Eg + n_pos else -1.0
             out.index_add_(0, tok, x[tok] * (sign * w_flat[slot]).unsqueeze(-1))
             continue
-        h = expert_hidden(x[tok], w_gate_up[e].to(dtype), theta[e])
+        h = expert_hidden(x[tok], w_gate_up[e].to(dtype), theta[e], act)
         if return_hidden:
             hidden[lo:hi] = h
         y = h @ w_down[e].to(dtype).t()                                       # moe.py:92

@@ -56,6 +56,19 @@ def test_misaligned_operands_are_reported_not_launched():
     assert forward(x_off, L.ALGO_FUSED) == -5 and forward(x_off, L.ALGO_MFMA) == -5
     assert b"align" in lib.bibo_moe_strerror(-5)
     assert forward(x_off, L.ALGO_GENERIC) == 0
+    # the workspace is carved at multiples of 256 bytes and accessed 16 bytes at a time: its base must be aligned
+    big = torch.empty(ws.numel() + 256, dtype=torch.uint8, device=DEV)
+    for off in (2, 16, 128):
+        rc = lib.bibo_moe_forward(P(x), P(wr), P(b), P(gu), P(dn), P(th), ctypes.byref(sh), L.NORM_SUM, L.ALGO_AUTO, P(out),
+                                  None, None, None, None, ctypes.c_void_p(big.data_ptr() + off), ws.numel(), stream)
+        assert rc == -5
+    idx = torch.zeros(T, k, dtype=torch.int32, device=DEV)
+    w = torch.ones(T, k, dtype=torch.float32, device=DEV)
+    assert lib.bibo_moe_experts_fwd(P(x), P(idx), P(w), P(gu), P(dn), P(th), ctypes.byref(sh), L.ALGO_AUTO, P(out), None,
+                                    ctypes.c_void_p(big.data_ptr() + 16), ws.numel(), stream) == -5
+    assert lib.bibo_moe_ffn_forward(P(x), P(th.new_ones(H)), ctypes.c_float(1e-6), P(wr), P(b), P(gu), P(dn), P(th),
+                                    ctypes.byref(sh), L.NORM_SUM, L.ALGO_AUTO, P(out), None, None, None,
+                                    ctypes.c_void_p(big.data_ptr() + 16), big.numel() - 16, stream) == -5
     gen = out.clone()
     assert forward(x, L.ALGO_FUSED) == 0
     torch.cuda.synchronize()

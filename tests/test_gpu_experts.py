@@ -122,7 +122,7 @@ def test_bf16_experts_reduced_prefill_and_ragged_shapes(T, H, I, bias, theta, al
 
 @pytest.mark.parametrize("T,H,I,k,theta", [(64, 1024, 512, 6, "zero"), (7, 1024, 512, 6, "normal"), (1, 768, 384, 6, "normal"),
                                            (200, 256, 128, 6, "normal"), (130, 128, 256, 2, "normal"),
-                                           (40, 64, 64, 1, "normal"), (400, 512, 256, 6, "normal")])
+                                           (40, 64, 64, 1, "normal"), (341, 512, 256, 6, "normal")])
 def test_streaming_kernels_match_oracle(T, H, I, k, theta):
     """Weight-streaming (decode) kernels: few rows per expert, several 16-row passes, idle experts."""
     p = O.make_inputs(T=T, H=H, E=64, k=k, I=I, bias="uniform", theta=theta, seed=T + I)
@@ -284,3 +284,60 @@ def test_full_size_prefill_properties(name, algo):
     pp = dict(p, x=p["x"][perm].contiguous())
     outp, _ = _gpu_experts(pp, idx[perm.numpy()], w[perm.numpy()], algo)
     assert torch.equal(outp, out[perm])
+
+
+# ------------------------------------------------------------------ activation variants (act codes 10 and 0)
+@pytest.mark.parametrize("act", ["tanh", "silu"])
+@pytest.mark.parametrize("algo,T,H,I", [("generic", 60, 96, 40), ("mfma", 400, 256, 128), ("fused", 400, 256, 128),
+                                        ("stream", 40, 256, 128), ("stream", 30, 256, 576), ("mfma", 300, 256, 512)])
+def test_activation_variants_match_oracle(algo, T, H, I, act):
+    """p = tanh(theta) (negative exponents shrink high-rms rows) and plain SwiGLU, the two activations the
+    reference's harness can switch its external kernel to (ablate/common/patches.py:53-69), in every family."""
+    E = 8 if algo == "generic" else 64
+    p = O.make_inputs(T=T, H=H, E=E, k=2 if E == 8 else 6, I=I, bias="uniform", theta="normal", seed=T + I)
+    p["theta"] = p["theta"] * 3 - 0.5                       # tanh(theta) spread over (-1, 1), mostly away from 0
+    idx, w = _route(p)
+    ref = O.experts_forward(p["x"], idx, w, p["w_gate_up"], p["w_down"], p["theta"], act=act)
+    other = O.experts_forward(p["x"], idx, w, p["w_gate_up"], p["w_down"], p["theta"])
+    assert rel_err(other, ref) > 0.05                        # the variants really differ from the default activation
+    out, _ = ops.experts_fwd(p["x"].to(DEV), torch.from_numpy(idx).to(DEV), torch.from_numpy(w).to(DEV),
+                             p["w_gate_up"].to(DEV), p["w_down"].to(DEV), p["theta"].to(DEV), algo=algo, act=act)
+    torch.cuda.synchronize()
+    assert rel_err(out.cpu(), ref) <= BF16_TOL
+
+
+def test_activation_variants_through_the_stage_entry_points():
+    p = O.make_inputs(T=300, H=256, E=64, k=6, I=128, bias="uniform", theta="normal", seed=12)
+    p["theta"] = p["theta"] * 3 - 0.5
+    idx, w = _route(p)
+    idx_d, w_d = torch.from_numpy(idx).to(DEV), torch.from_numpy(w).to(DEV)
+    counts, offsets, perm_slot, perm_token = ops.permute(idx_d, 64)
+    for act in ("tanh", "silu"):
+        ref, ref_hidden = O.experts_forward(p["x"], idx, w, p["w_gate_up"], p["w_down"], p["theta"], return_hidden=True,
+                                            act=act)
+        for algo in ("generic", "mfma"):
+            hidden = ops.gateup_fwd(p["x"].to(DEV), p["w_gate_up"].to(DEV), p["theta"].to(DEV), offsets, perm_token, 6,
+                                    algo=algo, act=act)
+            torch.cuda.synchronize()
+            assert rel_err(hidden.cpu(), ref_hidden) <= BF16_TOL
+        yw = ops.gateup_down_fwd(p["x"].to(DEV), p["w_gate_up"].to(DEV), p["w_down"].to(DEV), p["theta"].to(DEV), w_d,
+                                 offsets, perm_slot, perm_token, act=act)
+        out = ops.combine_fwd(yw, 300, 6)
+        torch.cuda.synchronize()
+        assert rel_err(out.cpu(), ref) <= BF16_TOL
+
+
+def test_fp32_tanh_exponent_matches_the_fp64_closed_form():
+    g = torch.Generator().manual_seed(3)
+    E, H, I, N = 4, 64, 96, 40
+    p = dict(x=torch.randn(N, H, generator=g), w_gate_up=torch.randn(E, 2 * I, H, generator=g) * 0.1,
+             w_down=torch.randn(E, H, I, generator=g) * 0.1, theta=torch.tensor([-2.0, -0.4, 0.0, 1.5]))
+    for e in range(E):
+        idx = np.full((N, 1), e, dtype=np.int32)
+        w = np.ones((N, 1), dtype=np.float32)
+        out, _ = ops.experts_fwd(p["x"].to(DEV), torch.from_numpy(idx).to(DEV), torch.from_numpy(w).to(DEV),
+                                 p["w_gate_up"].to(DEV), p["w_down"].to(DEV), p["theta"].to(DEV), algo="generic", act="tanh")
+        gate, up = (p["x"].double() @ p["w_gate_up"][e].double().t()).chunk(2, -1)
+        r = (gate.square().mean(-1, keepdim=True) + 1e-6).sqrt()
+        ref = (torch.nn.functional.silu(gate / r) * r.pow(np.tanh(float(p["theta"][e]))) * up) @ p["w_down"][e].double().t()
+        assert rel_err(out.cpu(), ref) < 1e-5

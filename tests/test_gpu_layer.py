@@ -246,3 +246,66 @@ def test_layer_ffn_forward_equals_norm_block_residual_composition():
         o32 = layer32.ffn_forward(h32, torch.ones(256, device="cuda:0"), 1e-6)
     assert o32.dtype == torch.float32
     assert (o32 - h32).abs().max() < 1.0 and torch.isfinite(o32).all()
+
+
+def test_ffn_forward_bf16_moe_out_rounds_the_block_before_the_sum():
+    """bf16_moe_out (src/modeling/layers.py:37,62-63): the block's output is rounded to bf16 before it enters the
+    residual sum.  With a residual of zero the two roundings collapse, so out == round(block); with a real residual
+    the result equals bf16(residual + bf16(block)) exactly, which the fp32-sum path does not."""
+    torch.manual_seed(5)
+    cfg = make_config(hidden_size=256, moe_intermediate_size=128, num_routed_experts=64, num_experts_per_tok=6)
+    layer = bibo_amd.BiBoMoELayer(cfg).to("cuda:0").bfloat16().eval()
+    h = (torch.randn(2, 150, 256, device="cuda:0") * 2).bfloat16()
+    nw = (torch.rand(256, device="cuda:0") + 0.5).bfloat16()
+    with torch.no_grad():
+        hf = h.float()
+        xn = (hf * torch.rsqrt(hf.pow(2).mean(-1, keepdim=True) + 1e-6)).bfloat16()
+        blk = layer(nw * xn)                                   # bf16 block output, rounded once
+        rounded = layer.ffn_forward(h, nw, 1e-6, bf16_moe_out=True)
+        plain = layer.ffn_forward(h, nw, 1e-6)
+    assert torch.equal(rounded, h + blk)                        # bf16 + bf16: one more rounding of the sum
+    assert not torch.equal(plain, rounded)                      # the fp32 sum keeps bits the rounded block lost
+    assert rel_err(plain.cpu(), rounded.cpu().float()) <= 1e-2
+    # an fp32 stream: stock tensor operations around the block, same contract
+    layer32 = bibo_amd.BiBoMoELayer(cfg).to("cuda:0").eval()
+    h32 = torch.randn(2, 50, 256, device="cuda:0")
+    with torch.no_grad():
+        a = layer32.ffn_forward(h32, nw.float(), 1e-6, bf16_moe_out=True)
+        hf = h32
+        xn = hf * torch.rsqrt(hf.pow(2).mean(-1, keepdim=True) + 1e-6)
+        b = h32 + layer32(nw.float() * xn).bfloat16().float()
+    assert a.dtype == torch.float32 and torch.equal(a, b)
+
+
+def test_layer_with_tanh_exponent_and_conv_shared_expert():
+    """Module-level switches: radial_p='tanh' reaches the kernels; the conv shared expert is added to the routed
+    output (moe.py:174-176 with experts.py:11-34)."""
+    p = O.make_inputs(T=96, H=256, E=64, k=6, I=128, bias="uniform", theta="normal", seed=31)
+    p["theta"] = p["theta"] * 3 - 0.5
+    c = bibo_amd.BiBoMoEConfig(hidden_size=256, moe_intermediate_size=128, num_routed_experts=64, special_expert_pairs=0,
+                               num_experts_per_tok=6, use_shared_expert=True, shared_expert_type="conv", kernel_size=3)
+    layer = bibo_amd.BiBoMoELayer(c)
+    missing = layer.load_state_dict({"gate.gate_proj.weight": p["w_router"].float(), "gate.bias": p["bias"],
+                                     "experts.gate_up_proj": p["w_gate_up"].float(),
+                                     "experts.down_proj": p["w_down"].float(), "experts.radial_theta": p["theta"],
+                                     "accumulated_tpe": torch.zeros(64)}, strict=False)
+    assert sorted(missing.missing_keys) == ["shared_experts_list.0.down_proj.weight",
+                                            "shared_experts_list.0.gate_conv.weight", "shared_experts_list.0.up_proj.weight"]
+    with torch.no_grad():
+        for q in layer.shared_experts_list.parameters():       # keep the shared term at the routed term's magnitude
+            q.mul_(0.7)
+    layer = layer.to(DEV).bfloat16().eval()
+    layer.experts.radial_p = "tanh"
+    x3 = p["x"].view(2, 48, 256).to(DEV)
+    with torch.no_grad():
+        out = layer(x3)
+        logits = layer.gate.router_logits(x3)
+        shared = layer.shared_experts_list[0](x3)
+    # .bfloat16() rounded the selection bias and theta too (a quirk the reference shares, tests/test_moe.py:252-259):
+    # the oracle gets the module's values
+    idx, w, _ = O.route_from_logits(logits.cpu().numpy(), layer.gate.bias.float().cpu().numpy(), 6)
+    ref = O.experts_forward(p["x"], idx, w, p["w_gate_up"], p["w_down"], layer.experts.radial_theta.float().cpu(), act="tanh")
+    sh = shared.float().view(-1, 256).cpu()
+    assert 0.2 < sh.abs().max() / ref.abs().max() < 5                                    # neither term hides the other
+    assert rel_err(out.view(-1, 256).cpu(), ref + sh) <= 2e-2
+    assert rel_err(out.view(-1, 256).cpu(), sh) > 0.1 and rel_err(out.view(-1, 256).cpu(), ref) > 0.1

@@ -30,7 +30,23 @@ def test_library_exports_every_declared_symbol():
     lib = L.lib()
     for name in declared:
         assert hasattr(lib, name)
-    assert lib.bibo_moe_abi_version() == L.ABI_VERSION == 2
+    assert lib.bibo_moe_abi_version() == L.ABI_VERSION == 3
+    m = re.search(r"#define BIBO_MOE_ABI_VERSION (\d+)", header)
+    assert m and int(m.group(1)) == L.ABI_VERSION
+
+
+def test_shape_struct_matches_the_header_and_the_documented_binding():
+    """bibo_moe_shape is read by pointer: a binding with fewer fields makes the library read past the caller's
+    struct.  The ctypes structure, the header and the example in INTEGRATION.md must agree field for field."""
+    header = (ROOT / "include" / "bibo_moe.h").read_text()
+    body = re.search(r"typedef struct bibo_moe_shape \{(.*?)\} bibo_moe_shape;", header, re.S).group(1)
+    fields = re.findall(r"int32_t\s+(\w+);", body)
+    assert fields == [n for n, _ in L.Shape._fields_]
+    assert ctypes.sizeof(L.Shape) == 4 * len(fields) == 40
+    doc = (ROOT / "INTEGRATION.md").read_text()
+    names = re.search(r"for n in \(([^)]*)\)\]", doc).group(1)
+    assert [n.strip().strip('"') for n in names.split(",")] == fields
+    assert "strerror.restype = ctypes.c_char_p" in doc
 
 
 def test_argument_errors_are_reported_without_a_gpu():
@@ -46,13 +62,14 @@ def test_argument_errors_are_reported_without_a_gpu():
     # stage entry points validate before launching
     assert lib.bibo_moe_router_fwd(None, None, None, 4, 64, 8, 2, 0, 1, None, None, None, None, None) == -1
     assert lib.bibo_moe_router_fwd(None, None, None, 4, 64, 8, 9, 0, 1, None, None, None, None, None) == -2
-    assert lib.bibo_moe_gateup_fwd(None, None, None, None, None, 4, 64, 8, 2, 96, 0, L.ALGO_MFMA, None, None) == -6
+    assert lib.bibo_moe_gateup_fwd(None, None, None, None, None, 4, 64, 8, 2, 96, 0, L.ALGO_MFMA, 0, None, None) == -6
     # the streaming kernels exist only behind the composite entry points
-    assert lib.bibo_moe_gateup_fwd(None, None, None, None, None, 4, 1024, 64, 6, 512, 0, L.ALGO_STREAM, None, None) == -6
+    assert lib.bibo_moe_gateup_fwd(None, None, None, None, None, 4, 1024, 64, 6, 512, 0, L.ALGO_STREAM, 0, None, None) == -6
+    assert lib.bibo_moe_gateup_fwd(None, None, None, None, None, 4, 64, 8, 2, 96, 0, L.ALGO_GENERIC, 3, None, None) == -6   # no such activation
     assert lib.bibo_moe_permute(None, 4, 8, 2, None, None, None, None, None, 0, None) == -1
     # fused-kernel and caller-seam entry points
-    assert lib.bibo_moe_gateup_down_fwd(None, None, None, None, None, None, None, None, 4, 768, 64, 6, 512, 0, None, None) == -6
-    assert lib.bibo_moe_gateup_down_fwd(None, None, None, None, None, None, None, None, 4, 768, 64, 6, 384, 0, None, None) == -1
+    assert lib.bibo_moe_gateup_down_fwd(None, None, None, None, None, None, None, None, 4, 768, 64, 6, 512, 0, 0, None, None) == -6
+    assert lib.bibo_moe_gateup_down_fwd(None, None, None, None, None, None, None, None, 4, 768, 64, 6, 384, 0, 0, None, None) == -1
     assert lib.bibo_moe_combine_fwd(None, 1, 4, 64, 2, L.DTYPE_F32, None, None) == -3      # bf16 slot rows need a bf16 output
     assert lib.bibo_moe_rmsnorm_fwd(None, None, ctypes.c_float(1e-6), 4, 64, 0, None, None) == -1
     ffn = ctypes.c_size_t(0)
@@ -131,12 +148,77 @@ def test_state_dict_layout_matches_the_reference_layer():
 
 
 def test_unsupported_configurations_raise():
-    with pytest.raises(NotImplementedError, match="conv"):
-        bibo_amd.BiBoMoELayer(make_config(use_shared_expert=True, shared_expert_type="conv"))
+    with pytest.raises(NotImplementedError, match="hidden_act"):
+        bibo_amd.BiBoMoELayer(make_config(use_shared_expert=True, shared_expert_type="conv", hidden_act="gelu"))
     with pytest.raises(NotImplementedError, match="hidden_act"):
         bibo_amd.BiBoMoELayer(make_config(use_shared_expert=True, hidden_act="gelu"))
     with pytest.raises(ValueError, match="GLU"):
         make_config(num_routed_experts=4, num_pos_identity_experts=2, num_neg_identity_experts=2)
+
+
+def test_conv_shared_expert_layout_and_causality():
+    """src/modeling/ffn/experts.py:11-34: parameter names and shapes of the reference's conv expert; the gate is a
+    causal convolution (output at position s sees inputs s-2..s only) and equals an explicit sum of shifted GEMMs."""
+    layer = bibo_amd.BiBoMoELayer(make_config(use_shared_expert=True, shared_expert_type="conv", kernel_size=3))
+    sd = layer.state_dict()
+    assert sd["shared_experts_list.0.gate_conv.weight"].shape == (96, 64, 3)
+    assert sd["shared_experts_list.0.up_proj.weight"].shape == (96, 64)
+    assert sd["shared_experts_list.0.down_proj.weight"].shape == (64, 96)
+    conv = layer.shared_experts_list[0].double()
+    x = torch.randn(2, 7, 64, dtype=torch.float64, generator=torch.Generator().manual_seed(0))
+    y = conv(x)
+    w = conv.gate_conv.weight                                                    # [I, H, 3]; tap j looks back 2 - j
+    xp = torch.nn.functional.pad(x, (0, 0, 2, 0))
+    gate = sum(xp[:, j:j + 7] @ w[:, :, j].t() for j in range(3))
+    ref = (torch.nn.functional.silu(gate) * (x @ conv.up_proj.weight.t())) @ conv.down_proj.weight.t()
+    assert torch.allclose(y, ref, atol=1e-12)
+    x2 = x.clone(); x2[:, 4:] += 1.0                                            # the future must not leak backwards
+    assert torch.equal(conv(x2)[:, :4], y[:, :4]) and not torch.allclose(conv(x2)[:, 4:], y[:, 4:])
+
+
+def test_expert_activation_switches():
+    """The harness's RADIAL_P / EXPERT_ACT globals (ablate/common/patches.py:53-69) as module attributes."""
+    e = bibo_amd.BiBoFusedExperts(make_config())
+    assert e.act == "radial" and ops.act_code(e.act) == L.ACT_RADIAL_SIGMOID
+    e.radial_p = "tanh"
+    assert ops.act_code(e.act) == L.ACT_RADIAL_TANH
+    e.expert_act = "silu"
+    assert ops.act_code(e.act) == L.ACT_SILU
+    e.expert_act = "gelu"
+    with pytest.raises(ValueError, match="expert_act"):
+        e.act
+    with pytest.raises(ValueError, match="act must be"):
+        ops.act_code("relu")
+    assert ops.act_code(bibo_amd.BiBoFusedExperts(make_config(radial_p="tanh")).act) == L.ACT_RADIAL_TANH
+
+
+def test_cast_cache_refreshes_on_load_and_on_request():
+    """Kernel-dtype copies of the parameters follow load_state_dict, .to() and refresh_weights(); a write through
+    `.data` alone is not seen (documented on _CastCache)."""
+    from bibo_amd.moe import _CastCache
+    c = _CastCache()
+    p = torch.nn.Parameter(torch.ones(4))
+    a = c.get("w", p, torch.bfloat16)
+    assert a.dtype == torch.bfloat16 and c.get("w", p, torch.bfloat16) is a           # cached
+    with torch.no_grad():
+        p.mul_(2)                                                                      # in-place op: version bump
+    assert float(c.get("w", p, torch.bfloat16)[0]) == 2.0
+    p.data.fill_(5.0)                                                                  # invisible to the cache ...
+    assert float(c.get("w", p, torch.bfloat16)[0]) == 2.0
+    c.invalidate()                                                                     # ... until asked
+    assert float(c.get("w", p, torch.bfloat16)[0]) == 5.0
+    layer = bibo_amd.BiBoMoELayer(make_config())
+    layer.experts._cache.get("gu", layer.experts.gate_up_proj, torch.bfloat16)
+    layer.gate._cache.get("w", layer.gate.gate_proj.weight, torch.bfloat16)
+    assert layer.experts._cache._store and layer.gate._cache._store
+    layer.load_state_dict(layer.state_dict())
+    assert not layer.experts._cache._store and not layer.gate._cache._store
+    layer.experts._cache.get("gu", layer.experts.gate_up_proj, torch.bfloat16)
+    layer.double()
+    assert not layer.experts._cache._store
+    layer.experts._cache.get("gu", layer.experts.gate_up_proj, torch.bfloat16)
+    layer.experts.refresh_weights()
+    assert not layer.experts._cache._store
 
 
 def test_specials_and_shared_expert_follow_the_reference_layout():

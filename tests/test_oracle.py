@@ -195,6 +195,34 @@ def test_radial_special_cases():
     assert torch.allclose(O.radial_normsilu(g[:2], torch.tensor(0.3)), O.radial_normsilu(g, torch.tensor(0.3))[:2])
 
 
+def test_activation_variants_of_the_training_harness():
+    """The two activations the reference's harness can switch its external kernel to
+    (ablate/common/patches.py:53-69): p = tanh(theta) and plain SiLU."""
+    x, wgu, wd = _tiny(seed=2)
+    g = (x @ wgu[0].t())[:, :8]
+    # tanh exponent: degree-p homogeneity with p = tanh(theta), which a NEGATIVE theta makes negative
+    # (a sigmoid exponent, or a dropped sign, fails: 3^p would exceed 1)
+    for theta in (-1.5, -0.3, 0.0, 0.9):
+        pexp = math.tanh(theta)
+        lhs = O.radial_normsilu(3.0 * g, torch.tensor(theta), "tanh")
+        assert torch.allclose(lhs, (3.0 ** pexp) * O.radial_normsilu(g, torch.tensor(theta), "tanh"), rtol=1e-5)
+    assert (O.radial_normsilu(3.0 * g, torch.tensor(-1.5), "tanh").abs().max()
+            < O.radial_normsilu(g, torch.tensor(-1.5), "tanh").abs().max())         # gain r^p shrinks with r for p < 0
+    # theta = 0 gives p = 0 under tanh (NormSiLU) but p = 1/2 under sigmoid
+    r = (g.square().mean(-1, keepdim=True) + 1e-6).sqrt()
+    assert torch.allclose(O.radial_normsilu(g, torch.tensor(0.0), "tanh"), F.silu(g / r), rtol=1e-9)
+    assert torch.allclose(O.radial_normsilu(g, torch.tensor(0.0)), F.silu(g / r) * r.sqrt(), rtol=1e-9)
+    # large |theta|: tanh -> +/-1
+    assert torch.allclose(O.radial_normsilu(g, torch.tensor(20.0), "tanh"), g * torch.sigmoid(g / r), rtol=1e-9)
+    assert torch.allclose(O.radial_normsilu(g, torch.tensor(-20.0), "tanh"), F.silu(g / r) / r, rtol=1e-9)
+    # plain SwiGLU: the library routine, rows independent of theta and of the other columns
+    assert torch.equal(O.radial_normsilu(g, torch.tensor(0.7), "silu"), F.silu(g))
+    idx = np.zeros((x.shape[0], 1), np.int64); w = np.ones((x.shape[0], 1), np.float32)
+    out = O.experts_forward(x, idx, w, wgu, wd, torch.full((wgu.shape[0],), 0.7), dtype=torch.float64, act="silu")
+    gate, up = (x @ wgu[0].t()).chunk(2, -1)
+    assert torch.allclose(out, (F.silu(gate) * up) @ wd[0].t(), rtol=1e-9)
+
+
 def test_gate_is_the_first_half_of_gate_up_rows():
     """moe.py:85 chunk(2): rows 0..I-1 gate, I..2I-1 up.  Zeroing the up half must zero the output;
     zeroing the gate half must too (SiLU(0) = 0)."""
