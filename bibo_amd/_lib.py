@@ -22,8 +22,9 @@ SYMBOLS = (
     "bibo_moe_abi_version", "bibo_moe_strerror", "bibo_moe_workspace_bytes", "bibo_moe_select_algo", "bibo_moe_router_fwd",
     "bibo_moe_permute", "bibo_moe_gateup_fwd", "bibo_moe_down_combine_fwd", "bibo_moe_gateup_down_fwd",
     "bibo_moe_combine_fwd", "bibo_moe_combine_ex_fwd", "bibo_moe_experts_fwd", "bibo_moe_forward", "bibo_moe_rmsnorm_fwd",
-    "bibo_moe_ffn_workspace_bytes", "bibo_moe_ffn_forward",
+    "bibo_moe_ffn_workspace_bytes", "bibo_moe_ffn_forward", "bibo_moe_forward_static",
 )
+STATIC_SCRATCH_BYTES = 16 << 20
 
 
 class Shape(ctypes.Structure):
@@ -69,6 +70,8 @@ def _declare(l):
     l.bibo_moe_ffn_forward.restype = ci
     l.bibo_moe_ffn_forward.argtypes = [vp, vp, ctypes.c_float, vp, vp, vp, vp, vp, ctypes.POINTER(Shape), ci, ci, vp, vp, vp,
                                        vp, vp, sz, vp]
+    l.bibo_moe_forward_static.restype = ci
+    l.bibo_moe_forward_static.argtypes = [vp, vp, vp, vp, vp, vp, ctypes.POINTER(Shape), ci, ci, vp, vp, vp, vp, vp, vp]
     l.bibo_moe_forward.restype = ci
     l.bibo_moe_forward.argtypes = [vp, vp, vp, vp, vp, vp, ctypes.POINTER(Shape), ci, ci, vp, vp, vp, vp, vp, vp, sz, vp]
 

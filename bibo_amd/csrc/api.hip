@@ -1,10 +1,38 @@
 // extern "C" entry points: host-side argument checks, workspace carving and kernel dispatch.
 // Nothing here allocates or synchronises; see include/bibo_moe.h for the contract.
+#include <mutex>
+
 #include "common.h"
+
+// Workspace of bibo_moe_forward_static: one copy per GPU, alive until the process ends.  In host code the
+// name is only a handle for hipGetSymbolAddress; kernels get the per-device address looked up below.
+static __device__ __align__(256) unsigned char scratch[BIBO_MOE_STATIC_SCRATCH_BYTES];
 
 namespace {
 
 using namespace bibo;
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// Address of `scratch` on the current device, looked up once per device.
+int static_scratch(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= kMaxDevices) return BIBO_ERR_UNSUPPORTED;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (p == nullptr) return (int)hipErrorInvalidSymbol;
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return BIBO_OK;
+}
 
 constexpr size_t kAlign = 256;
 inline size_t align_up(size_t v) { return (v + kAlign - 1) & ~(kAlign - 1); }
@@ -224,6 +252,9 @@ const char* bibo_moe_strerror(int code) {
     case BIBO_ERR_WORKSPACE_TOO_SMALL: return "workspace smaller than bibo_moe_workspace_bytes() for this shape";
     case BIBO_ERR_MISALIGNED: return "tensor base pointers must be 16-byte aligned and the workspace 256-byte aligned";
     case BIBO_ERR_UNSUPPORTED: return "requested kernel family does not support this shape or dtype";
+    case BIBO_ERR_STATIC_SCRATCH:
+      return "shape needs more workspace than the static scratch array holds (BIBO_MOE_STATIC_SCRATCH_BYTES = 16 MiB); "
+             "use bibo_moe_forward with a caller-owned workspace";
     default: break;
   }
   if (code > 0) return hipGetErrorString((hipError_t)code);
@@ -375,6 +406,21 @@ int bibo_moe_forward(const void* x, const void* w_router, const float* bias, con
                      void* stream) {
   return forward_impl(x, w_router, bias, w_gate_up, w_down, theta, sh, norm_mode, algo, nullptr, out, idx_out, w_out,
                       counts_out, logits_out, workspace, workspace_bytes, stream);
+}
+
+int bibo_moe_forward_static(const void* x, const void* w_router, const float* bias, const void* w_gate_up,
+                            const void* w_down, const float* theta, const bibo_moe_shape* sh, int norm_mode, int algo,
+                            void* out, int32_t* idx_out, float* w_out, int32_t* counts_out, float* logits_out,
+                            void* stream) {
+  if (sh == nullptr) return BIBO_ERR_NULL_POINTER;
+  int rc = check_dims(sh->T, sh->H, sh->E, sh->k, sh->I, sh->dtype, sh->n_pos, sh->n_neg);
+  if (rc != BIBO_OK) return rc;
+  if (carve(sh->T, sh->H, sh->E, sh->k, sh->I, sh->dtype).total > (size_t)BIBO_MOE_STATIC_SCRATCH_BYTES)
+    return BIBO_ERR_STATIC_SCRATCH;
+  void* ws = nullptr;
+  if ((rc = static_scratch(&ws)) != BIBO_OK) return rc;
+  return forward_impl(x, w_router, bias, w_gate_up, w_down, theta, sh, norm_mode, algo, nullptr, out, idx_out, w_out,
+                      counts_out, logits_out, ws, (size_t)BIBO_MOE_STATIC_SCRATCH_BYTES, stream);
 }
 
 int bibo_moe_rmsnorm_fwd(const void* x, const float* norm_weight, float eps, int T, int H, int dtype, void* out,

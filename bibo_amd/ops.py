@@ -262,6 +262,32 @@ def moe_forward(x, w_router, bias, w_gate_up, w_down, theta, k, norm="sum", algo
     return out, idx, w, counts, logits
 
 
+def moe_forward_static(x, w_router, bias, w_gate_up, w_down, theta, k, out, norm="sum", algo="auto", idx=None, w=None,
+                       counts=None, logits=None, n_pos=0, n_neg=0, act="radial"):
+    """bibo_moe_forward_static: the whole layer with the library's static per-GPU scratch array as workspace.  Nothing
+    is allocated here either: `out` [T,H] and the optional `idx`, `w`, `counts`, `logits` are the caller's tensors."""
+    T, H = x.shape
+    Eg, two_i, _ = w_gate_up.shape
+    E = Eg + n_pos + n_neg
+    I = two_i // 2
+    dc = _dtype_code(x)
+    _chk(x, "x"); _chk(w_router, "w_router", x.dtype, (E, H)); _chk(bias, "bias", torch.float32, (E,))
+    _chk(w_gate_up, "w_gate_up", x.dtype, (Eg, 2 * I, H)); _chk(w_down, "w_down", x.dtype, (Eg, H, I))
+    _chk(theta, "theta", torch.float32, (Eg,)); _chk(out, "out", x.dtype, (T, H))
+    for t_, n_, d_, sh_ in ((idx, "idx", torch.int32, (T, k)), (w, "w", torch.float32, (T, k)),
+                            (counts, "counts", torch.int32, (E,)), (logits, "logits", torch.float32, (T, E))):
+        if t_ is not None:
+            _chk(t_, n_, d_, sh_)
+    sh = L.Shape(T, H, E, k, I, dc, n_pos, n_neg, act_code(act), 0)
+    dev = x.device
+    with torch.cuda.device(dev):
+        L.check(L.lib().bibo_moe_forward_static(_ptr(x), _ptr(w_router), _ptr(bias), _ptr(w_gate_up), _ptr(w_down),
+                                                _ptr(theta), ctypes.byref(sh), norm_mode(norm), algo_code(algo), _ptr(out),
+                                                _ptr(idx), _ptr(w), _ptr(counts), _ptr(logits), _stream(dev)),
+                "bibo_moe_forward_static")
+    return out
+
+
 def rmsnorm_fwd(x, norm_weight, eps):
     """out = norm_weight * round(x * rsqrt(mean(x^2) + eps)) in x.dtype (the block's input norm, norm.py:19-24)."""
     T, H = x.shape

@@ -87,7 +87,8 @@ enum bibo_error {
   BIBO_ERR_BAD_DTYPE = -3,
   BIBO_ERR_WORKSPACE_TOO_SMALL = -4,
   BIBO_ERR_MISALIGNED = -5,
-  BIBO_ERR_UNSUPPORTED = -6
+  BIBO_ERR_UNSUPPORTED = -6,
+  BIBO_ERR_STATIC_SCRATCH = -7 /* bibo_moe_forward_static: the shape needs more than BIBO_MOE_STATIC_SCRATCH_BYTES */
 };
 
 typedef struct bibo_moe_shape {
@@ -215,6 +216,25 @@ int bibo_moe_forward(const void* x, const void* w_router, const float* bias, con
                      const void* w_down, const float* theta, const bibo_moe_shape* shape, int norm_mode, int algo,
                      void* out, int32_t* idx_out, float* w_out, int32_t* counts_out, float* logits_out,
                      void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * bibo_moe_forward for callers that cannot allocate device memory or pass a workspace: code running under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.
+ * Same arguments and results as bibo_moe_forward, without `workspace`: the intermediates (routing, permutation,
+ * pre-activations, slot rows) live in a static device array of BIBO_MOE_STATIC_SCRATCH_BYTES that every GPU the
+ * library runs on holds until the process ends.  The call allocates and frees nothing.  A shape whose
+ * bibo_moe_workspace_bytes() exceeds the array is refused with BIBO_ERR_STATIC_SCRATCH before anything is
+ * launched (decode-size shapes fit: T=64, H=1024, I=512 needs 2.8 MB).  All calls on one GPU share that GPU's
+ * array, on whatever stream: calls that may overlap on one GPU race and must be ordered by the caller.  Nothing
+ * in the array has to start at zero (every segment is written before it is read within a call), so it is
+ * never cleared.  The first call on a device looks the array's address up (no stream work); make that call
+ * before capturing a graph.
+ */
+#define BIBO_MOE_STATIC_SCRATCH_BYTES (16u << 20)
+int bibo_moe_forward_static(const void* x, const void* w_router, const float* bias, const void* w_gate_up,
+                            const void* w_down, const float* theta, const bibo_moe_shape* shape, int norm_mode,
+                            int algo, void* out, int32_t* idx_out, float* w_out, int32_t* counts_out,
+                            float* logits_out, void* stream);
 
 /*
  * Seam 3: the caller of the block, BiBoDecoderLayer._ffn_forward (src/modeling/layers.py:57-67):
