@@ -62,6 +62,9 @@ inline long long stream_rows_per_expert(int H, int I) {
 // `distinct`: the k experts of a token are known to differ (indices that come straight from the router kernel), so
 // one expert gets at most T rows.  A caller's indices may name an expert several times per token, up to all T*k
 // slots on one expert, and the row list of a streaming workgroup holds kStreamMaxRows entries.
+// the fused kernel addresses hidden-state rows with 32-bit byte offsets
+inline bool fused_fits(int T, int H) { return (long long)T * H < (1LL << 31); }
+
 inline bool stream_eligible(int T, int H, int E, int k, int I, int dtype, bool distinct) {
   return stream_supported(H, I, dtype) && (long long)T * k <= stream_rows_per_expert(H, I) * E &&
          (long long)T * k <= kStreamMaxSlots && (distinct ? T : (long long)T * k) <= kStreamMaxRows;
@@ -74,7 +77,7 @@ int resolve_algo(int algo, int T, int H, int E, int k, int I, int dtype, bool co
   switch (algo) {
     case BIBO_ALGO_AUTO:
       if (composite && stream_eligible(T, H, E, k, I, dtype, distinct)) *out = BIBO_ALGO_STREAM;
-      else if (composite && fused_supported(H, I, dtype)) *out = BIBO_ALGO_FUSED;
+      else if (composite && fused_supported(H, I, dtype) && fused_fits(T, H)) *out = BIBO_ALGO_FUSED;
       else *out = mfma_supported(H, I, dtype) ? BIBO_ALGO_MFMA : BIBO_ALGO_GENERIC;
       break;
     case BIBO_ALGO_GENERIC: *out = BIBO_ALGO_GENERIC; break;
@@ -88,7 +91,7 @@ int resolve_algo(int algo, int T, int H, int E, int k, int I, int dtype, bool co
       *out = BIBO_ALGO_STREAM;
       break;
     case BIBO_ALGO_FUSED:
-      if (!composite || !fused_supported(H, I, dtype)) return BIBO_ERR_UNSUPPORTED;
+      if (!composite || !fused_supported(H, I, dtype) || !fused_fits(T, H)) return BIBO_ERR_UNSUPPORTED;
       *out = BIBO_ALGO_FUSED;
       break;
     default: return BIBO_ERR_UNSUPPORTED;
@@ -333,7 +336,7 @@ int bibo_moe_gateup_down_fwd(const void* x, const void* w_gate_up, const void* w
                              void* yw, void* stream) {
   const int rc = check_dims(T, H, E, k, I, dtype);
   if (rc != BIBO_OK) return rc;
-  if (!fused_supported(H, I, dtype) || !act_ok(act)) return BIBO_ERR_UNSUPPORTED;
+  if (!fused_supported(H, I, dtype) || !fused_fits(T, H) || !act_ok(act)) return BIBO_ERR_UNSUPPORTED;
   if (T == 0) return BIBO_OK;
   if (!x || !w_gate_up || !w_down || (!theta && act != BIBO_ACT_SILU) || !w || !offsets || !perm_slot || !perm_token || !yw)
     return BIBO_ERR_NULL_POINTER;

@@ -1,18 +1,24 @@
 // Kernels 3 and 4 in one launch: a workgroup takes 128 permuted rows of one expert through the gate/up
 // projection, Radial NormSiLU and the down projection without the activations leaving the CU.
 //
-// Phase 1 is the gate/up main loop of gateup_dma_kernel (x rows and w_gate_up rows by LDS-DMA, two
-// stages `P` and `Q`) with the MFMA operands swapped, so a lane ends up with one ROW's values.  Phase 2 turns the accumulators into bf16 activations and parks them in LDS as an
-// operand of the second GEMM: rows 0..63 live in P, rows 64..127 in Q, whose stage contents are dead by
-// then; row r keeps 16-byte granule c at position c ^ (r & 15), which spreads the 16 lanes of a fragment
-// read over all banks although the row stride is a multiple of 256 bytes.
+// Phase 1 (gate/up GEMM, 2 x 4 waves, v_mfma_f32_32x32x16_bf16, operands swapped so that a lane ends up with
+// one ROW's values) walks K in steps of 64 elements, so every row an LDS-DMA instruction fetches is a whole
+// 128-byte line: the L2 -> LDS path moves almost twice the bytes per second for whole lines than for the
+// half lines of a 32-element step.  A step of all 2I weight rows would not fit LDS twice, so a step is cut
+// into a gate half and an up half: while the MFMAs multiply the I gate rows of step s from one buffer, the up
+// rows of step s arrive in the other, then the gate rows of step s+1 in the first, and so on; the x rows of
+// step s+1 arrive in two halves over the two sub-steps of step s.
+// Phase 2 turns the accumulators into bf16 activations and parks them in LDS as an operand of the second
+// GEMM: rows 0..63 live in B0, rows 64..127 in B1, whose contents are dead by then; row r keeps 16-byte
+// granule c at position c ^ (r & 15), which spreads the 16 lanes of a fragment read over all banks although
+// the row stride is a multiple of 256 bytes.
 // Phase 3 has no barriers and no LDS traffic for the weights: the eight waves split a block of 128*CT
 // output columns (16*CT each), every wave multiplies ALL 128 resident rows with v_mfma_f32_16x16x32_bf16
 // and pulls its own w_down rows straight from global memory into registers, up to three 128-byte K
 // blocks ahead (lane (r, g) takes bytes [32g, 32g+32) of each line of weight row r; the activation fragments
 // are read with the same K permutation).  Keeping the in-flight bytes in registers instead of LDS is
 // what lets a CU cover the memory latency here: the activations already fill most of the LDS.
-// Each block of columns is scaled by the routing weight, staged through LDS 64 rows at a time and
+// Each block of columns is scaled by the routing weight, staged through LDS 32 rows at a time and
 // scattered to slot order as whole 16-byte row segments.
 // Reference: BiBoFusedExperts.forward, src/modeling/ffn/moe.py:81-93.
 #include "stripe.h"
@@ -22,17 +28,54 @@ namespace {
 
 template <int NT, int CT>
 struct FusedShape {
-  static constexpr int MT = 2, WM = 2, BM = 128;
+  static constexpr int MT = 2, WM = 2, BM = 128, BK = 64;
   static constexpr int I = 128 * NT;
   static constexpr int BN2 = 128 * CT;                             // output columns per block: 8 waves x CT x 16
-  using S1 = Stripe<MT, 2 * NT, WM>;
-  static constexpr int kHalfElems = 64 * I;                        // activations of one M half
-  static constexpr int kTailElems = S1::kStageElems - kHalfElems;  // = 4096: free behind the activations
-  static constexpr int kOutElems = 64 * BN2;                       // output staging: 64 rows of a column block
-  static_assert(kTailElems * 2 >= 4 * BM * 4 + 4 * BM * 4, "row scalars do not fit behind the activations");
+  static constexpr int kHalfElems = 64 * I;                        // one weight half-stage = activations of one M half
+  static constexpr int kAElems = BM * BK;                          // x rows of one K step
+  static constexpr int kOutRows = 32;                              // rows of a column block staged at a time
+  static constexpr int kOutElems = kOutRows * BN2;
+  static constexpr int kBInstr = I * (BK / 8) / 512;               // load instructions per thread and weight half-stage
+  static_assert(I * (BK / 8) % 512 == 0 && BM * (BK / 8) == 2 * 512, "stage does not divide over the threads");
+};
+
+// LDS-DMA through a buffer descriptor: the address is descriptor base + 32-bit per-thread byte offset (one
+// vector register) + a wave-uniform byte offset (scalar), so the loop keeps no 64-bit per-thread addresses.
+__device__ __forceinline__ void dma16_buf(__amdgpu_buffer_rsrc_t rsrc, unsigned voff, unsigned soff, bf16_t* l) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void*)l, 16, voff, soff, 0, 0);
+}
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, unsigned bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);   // raw buffer, 32-bit data format
+}
+
+// The load instructions one thread issues during one sub-step: the next weight half-stage and half of the
+// next step's x rows.  Shaped like StripeLoader so that stripe_step can spread them between its MFMAs.
+template <typename F>
+struct SubLoader {
+  __amdgpu_buffer_rsrc_t w_rsrc, x_rsrc;   // this expert's w_gate_up block; the hidden states
+  unsigned b_voff;         // byte offset of this thread's row and granule inside the first instruction's 64 rows
+  unsigned b_soff;         // byte offset of the half-stage to fetch, K offset included (uniform)
+  unsigned bstep;          // bytes between the rows of consecutive instructions (uniform)
+  bf16_t* b_dst;           // LDS half-stage
+  unsigned a_voff;         // byte offset of this thread's token row and granule
+  unsigned a_soff;         // K offset in bytes (uniform)
+  bf16_t* a_dst;           // LDS position of that instruction's granules
+  static constexpr int kInstr = F::kBInstr + 1;
+  template <int Q>
+  __device__ __forceinline__ void issue(int, bf16_t*) const {
+    const int wave = threadIdx.x >> 6;
+    if constexpr (Q < F::kBInstr) dma16_buf(w_rsrc, b_voff, b_soff + Q * bstep, b_dst + (Q * 512 + wave * 64) * 8);
+    else if constexpr (Q == F::kBInstr) dma16_buf(x_rsrc, a_voff, a_soff, a_dst + wave * 64 * 8);
+  }
 };
 
 // this lane's 32 bytes of one 128-byte K block for each of its CT weight tiles
+#ifdef BIBO_P3_OLD
+constexpr int W3_SECOND = 8, W3_LANE = 16;
+#else
+constexpr int W3_SECOND = 32, W3_LANE = 8;     // the four lanes of a row fetch 64 contiguous bytes per instruction
+#endif
 template <int CT>
 struct WBlock {
   bf16x8 w[CT][2];
@@ -44,7 +87,7 @@ __device__ __forceinline__ void load_wblock(WBlock<CT>& b, const bf16_t* __restr
   for (int ct = 0; ct < CT; ++ct) {
     const bf16_t* p = wp + ct * tile_stride + kb * 64;
     b.w[ct][0] = *reinterpret_cast<const bf16x8*>(p);
-    b.w[ct][1] = *reinterpret_cast<const bf16x8*>(p + 8);
+    b.w[ct][1] = *reinterpret_cast<const bf16x8*>(p + W3_SECOND);
   }
 }
 
@@ -56,53 +99,87 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
                                                             const int32_t* __restrict__ offsets,
                                                             const int32_t* __restrict__ perm_slot,
                                                             const int32_t* __restrict__ perm_token, int H, int E,
-                                                            int act, bf16_t* __restrict__ yw) {
+                                                            int act, unsigned x_bytes, bf16_t* __restrict__ yw) {
   using F = FusedShape<NT, CT>;
-  using S1 = typename F::S1;
-  constexpr int MT = F::MT, BM = F::BM, I = F::I, NTW = 2 * NT;
-  __shared__ __attribute__((aligned(16))) bf16_t P[S1::kStageElems];
-  __shared__ __attribute__((aligned(16))) bf16_t Q[S1::kStageElems];
-  __shared__ __attribute__((aligned(16))) bf16_t O[F::kOutElems];
-  // row scalars, behind the activations of M half 0 (valid from phase 2 on)
-  float* ssq = reinterpret_cast<float*>(P + F::kHalfElems);        // [4][BM]
-  float* rinv_s = ssq + 4 * BM;                                    // [BM]
-  float* gain_s = rinv_s + BM;                                     // [BM]
-  float* w_s = gain_s + BM;                                        // [BM]
-  int* slot_s = reinterpret_cast<int*>(w_s + BM);                  // [BM]
+  constexpr int MT = F::MT, BM = F::BM, I = F::I, BK = F::BK;
+  __shared__ __attribute__((aligned(16))) bf16_t P[F::kHalfElems];    // weight half-stage 0, then activations of rows 0..63
+  __shared__ __attribute__((aligned(16))) bf16_t Q[F::kHalfElems];    // weight half-stage 1, then activations of rows 64..127
+  // Every buffer that is read while LDS-DMA fills another is a variable of its own: the compiler orders a DMA
+  // transfer against later LDS reads of the same variable with a full wait for the transfer.
+  __shared__ __attribute__((aligned(16))) bf16_t A0[F::kAElems];      // x rows of even K steps
+  __shared__ __attribute__((aligned(16))) bf16_t A1[F::kAElems];      // x rows of odd K steps
+  __shared__ __attribute__((aligned(16))) bf16_t O[F::kOutElems];     // output staging
+  __shared__ float ssq[4 * BM];
+  __shared__ float rinv_s[BM], gain_s[BM], w_s[BM];
+  __shared__ int slot_s[BM];
 
   const TileMap tm = make_tile_map(offsets, E, BM);
   const int tile = xcd_tile(blockIdx.x, tm.total);
   if (tile >= tm.total) return;
   int e, row0, rows;
   find_tile(tm, offsets, BM, tile, e, row0, rows);
+  e = __builtin_amdgcn_readfirstlane(e);                // the same for every lane: keep them in scalar registers
+  row0 = __builtin_amdgcn_readfirstlane(row0);
+  rows = __builtin_amdgcn_readfirstlane(rows);
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int wn = wave & 3, wm = wave >> 2;
   const int n = lane & 31;
-  const int chunk = S1::dma_chunk(tid);
   const int mbase = wm * MT * 32;
 
   // ---- phase 1: gate/up projection (moe.py:81-86) ----
-  floatx16 acc[MT][NTW];
+  floatx16 acc[MT][2 * NT];               // [..][0..NT) gate tiles, [..][NT..2NT) the up tiles of the same columns
   {
-    StripeLoader<S1> ld;
-    ld.b_src = wgu + ((size_t)e * 2 * I + S1::dma_row(tid)) * H + chunk * 8;
-    ld.bstep = (size_t)S1::kRowsPerInstr * H;
-    ld.issue_b(0, P);                        // weight rows first: they do not wait for the row indices
+    // DMA side: thread t of an instruction fills granule t (row t/8, position t%8) of its 64 rows and fetches
+    // logical granule (t%8) ^ ((row >> 1) & 7) of that row: granule c of a stage row sits at c ^ ((row >> 1) & 7)
+    const int chunk = (tid & 7) ^ ((tid >> 4) & 7);
+    const int drow = tid >> 3;
+    SubLoader<F> ld;
+    ld.w_rsrc = make_rsrc(wgu + (size_t)e * 2 * I * H, 2u * I * H * sizeof(bf16_t));   // gate rows; the up rows are I further
+    ld.x_rsrc = make_rsrc(x, x_bytes);
+    const unsigned up_off = (unsigned)I * H * sizeof(bf16_t);
+    ld.b_voff = ((unsigned)drow * H + chunk * 8) * sizeof(bf16_t);
+    ld.bstep = 64u * H * sizeof(bf16_t);
+    unsigned a_voff[2];
 #pragma unroll
-    for (int i = 0; i < S1::A_PER; ++i) {
-      const int m = min(S1::dma_row(tid) + i * S1::kRowsPerInstr, rows - 1);   // rows past the end re-read the last valid row
-      ld.a_src[i] = x + (size_t)perm_token[row0 + m] * H + chunk * 8;
+    for (int a = 0; a < 2; ++a) {
+      const int m = min(a * 64 + drow, rows - 1);                                // rows past the end re-read the last valid row
+      a_voff[a] = ((unsigned)perm_token[row0 + m] * H + chunk * 8) * sizeof(bf16_t);   // gather, moe.py:81
     }
-    ld.issue_a(0, P);
+    // prologue: gate half-stage and x rows of step 0 (weight rows first: they do not wait for the row indices)
+#pragma unroll
+    for (int q = 0; q < F::kBInstr; ++q) dma16_buf(ld.w_rsrc, ld.b_voff, q * ld.bstep, P + (q * 512 + wave * 64) * 8);
+    dma16_buf(ld.x_rsrc, a_voff[0], 0, A0 + (wave * 64) * 8);
+    dma16_buf(ld.x_rsrc, a_voff[1], 0, A0 + (512 + wave * 64) * 8);
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-      for (int j = 0; j < NTW; ++j)
+      for (int j = 0; j < 2 * NT; ++j)
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[mt][j][i] = 0.f;
-    auto frag_row = [&](int j) { return (j < NT ? 0 : I) + (wn * NT + (j < NT ? j : j - NT)) * 32; };
-    stripe_mainloop_dma<MT, NTW, F::WM, S1::BK, true>(acc, ld, H, P, Q, wm, frag_row);
+    // fragment side: lane (n, h) reads logical granule 2*ss + h of rows congruent to n mod 32
+    const int pos0 = ((lane >> 5) ^ ((n >> 1) & 7)) * 8;
+    auto frag_row = [&](int j) { return (wn * NT + j) * 32; };
+    // one K step: x rows in `Acur`, the next step's go to `Anext`
+    auto step = [&](const bf16_t* Acur, bf16_t* Anext, int k0, bool last) {
+      const unsigned kb = (unsigned)k0 * sizeof(bf16_t);
+      const unsigned kn = last ? kb : kb + BK * sizeof(bf16_t);                  // (the last step fetches its own x rows again: unused)
+      const bf16_t* a0 = Acur + (mbase + n) * BK + pos0;
+      // gate sub-step: multiplies P; the up rows of this step arrive in Q, rows 0..63 of the next x stage in Anext
+      wait_loads_and_sync();
+      ld.b_soff = up_off + kb; ld.b_dst = Q;
+      ld.a_soff = kn; ld.a_voff = a_voff[0]; ld.a_dst = Anext;
+      stripe_step<MT, NT, BK, true, 2 * NT, 0>(acc, a0, 32 * BK, P + n * BK, pos0, frag_row, ld, true, 0, nullptr);
+      // up sub-step: multiplies Q; the gate rows of the next step arrive in P, rows 64..127 of the next x stage
+      wait_loads_and_sync();
+      ld.b_soff = kn; ld.b_dst = P;
+      ld.a_voff = a_voff[1]; ld.a_dst = Anext + 512 * 8;
+      stripe_step<MT, NT, BK, true, 2 * NT, NT>(acc, a0, 32 * BK, Q + n * BK, pos0, frag_row, ld, !last, 0, nullptr);
+    };
+    for (int k0 = 0; k0 < H; k0 += 2 * BK) {                                     // H / BK is even
+      step(A0, A1, k0, false);
+      step(A1, A0, k0 + BK, k0 + 2 * BK >= H);
+    }
   }
   __syncthreads();                         // every wave is done with the gate/up stages
 
@@ -165,7 +242,7 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
   const size_t tile_stride = (size_t)16 * I;
   // activation fragment of row tile rt, K block kb, half s: granule (8*kb + 2*g4 + s) ^ r16 of row 16*rt + r16
   const int nblk = H / F::BN2;
-  const bf16_t* wp = wd + ((size_t)e * H + wave * (16 * CT) + r16) * I + g4 * 16;
+  const bf16_t* wp = wd + ((size_t)e * H + wave * (16 * CT) + r16) * I + g4 * W3_LANE;
   constexpr int D = KB > 3 ? 3 : KB - 1;      // K blocks requested ahead of the one being multiplied
   constexpr int NB = D + 1;
   WBlock<CT> wb[NB];
@@ -181,7 +258,11 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
     // Activation fragments are read a row tile ahead of the MFMAs that consume them (across K block
     // boundaries too).
     auto frag = [&](int kb, int rt, int s) {
+#ifdef BIBO_P3_OLD
       const int gq = (((kb * 8 + 2 * g4) ^ r16) * 8) ^ (s * 8);
+#else
+      const int gq = (((kb * 8 + g4) ^ r16) * 8) ^ (s * 32);      // K elements 64 kb + 32 s + 8 g4 .. + 8 of the row
+#endif
       return *reinterpret_cast<const bf16x8*>((rt < 4 ? P : Q) + ((rt & 3) * 16 + r16) * I + gq);
     };
     constexpr int AD = 1;                    // row tiles whose fragments are requested ahead (2 and 3 measured the same)
@@ -225,11 +306,11 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
     asm volatile("" : "+v"(tid_o));
     const int r16o = tid_o & 15, g4o = (tid_o >> 4) & 3;
 #pragma unroll
-    for (int hf = 0; hf < 2; ++hf) {
+    for (int hf = 0; hf < BM / F::kOutRows; ++hf) {
       __syncthreads();                       // the previous copy-out is done with O
 #pragma unroll
-      for (int rq = 0; rq < 4; ++rq) {
-        const int rt = hf * 4 + rq;
+      for (int rq = 0; rq < F::kOutRows / 16; ++rq) {
+        const int rt = hf * (F::kOutRows / 16) + rq;
         const float ws = w_s[rt * 16 + r16o];                                            // moe.py:93
         bf16_t* orow = O + (rq * 16 + r16o) * F::BN2 + (g4o & 1) * 4;
 #pragma unroll
@@ -243,10 +324,10 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
       }
       __syncthreads();
 #pragma unroll
-      for (int q = 0; q < 64 * G / 512; ++q) {
+      for (int q = 0; q < F::kOutRows * G / 512; ++q) {
         const int idx = q * 512 + tid_o;
         const int r = idx / G, pc = idx - r * G;
-        const int m = hf * 64 + r;
+        const int m = hf * F::kOutRows + r;
         if (m < rows)
           *reinterpret_cast<u32x4*>(yw + (size_t)slot_s[m] * H + n0 + (pc ^ (r & 15)) * 8) =
               *reinterpret_cast<const u32x4*>(O + r * F::BN2 + pc * 8);
@@ -258,19 +339,19 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
 template <int NT, int CT>
 void launch_fused_t(const bf16_t* x, const bf16_t* wgu, const bf16_t* wd, const float* theta, const float* w,
                     const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token, int S, int H, int E,
-                    int act, bf16_t* yw, hipStream_t s) {
+                    int act, unsigned x_bytes, bf16_t* yw, hipStream_t s) {
   const int grid = ((S / 128 + E + 7) & ~7) + 8;
   hipLaunchKernelGGL((experts_fused_kernel<NT, CT>), dim3(grid), dim3(512), 0, s, x, wgu, wd, theta, w, offsets,
-                     perm_slot, perm_token, H, E, act, yw);
+                     perm_slot, perm_token, H, E, act, x_bytes, yw);
 }
 
 template <int NT>
 void launch_fused_nt(const bf16_t* x, const bf16_t* wgu, const bf16_t* wd, const float* theta, const float* w,
                      const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token, int S, int H, int E,
-                     int act, bf16_t* yw, hipStream_t s) {
-  if (H % 384 == 0) launch_fused_t<NT, 3>(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, S, H, E, act, yw, s);
-  else if (H % 256 == 0) launch_fused_t<NT, 2>(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, S, H, E, act, yw, s);
-  else launch_fused_t<NT, 1>(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, S, H, E, act, yw, s);
+                     int act, unsigned x_bytes, bf16_t* yw, hipStream_t s) {
+  if (H % 384 == 0) launch_fused_t<NT, 3>(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, S, H, E, act, x_bytes, yw, s);
+  else if (H % 256 == 0) launch_fused_t<NT, 2>(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, S, H, E, act, x_bytes, yw, s);
+  else launch_fused_t<NT, 1>(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, S, H, E, act, x_bytes, yw, s);
 }
 
 }  // namespace
@@ -285,14 +366,16 @@ hipError_t launch_experts_fused(const void* x, const void* wgu, const void* wd, 
                                 int H, int E, int k, int I, int act, void* yw, hipStream_t s) {
   const int S = T * k;
   if (S == 0) return hipSuccess;
+  if ((unsigned long long)T * H * sizeof(bf16_t) >= (1ull << 32)) return hipErrorInvalidValue;   // 32-bit byte offsets into x
+  const unsigned xb = (unsigned)((size_t)T * H * sizeof(bf16_t));
   const bf16_t* xp = static_cast<const bf16_t*>(x);
   const bf16_t* gp = static_cast<const bf16_t*>(wgu);
   const bf16_t* dp = static_cast<const bf16_t*>(wd);
   bf16_t* yp = static_cast<bf16_t*>(yw);
   switch (I) {
-    case 128: launch_fused_nt<1>(xp, gp, dp, theta, w, offsets, perm_slot, perm_token, S, H, E, act, yp, s); break;
-    case 256: launch_fused_nt<2>(xp, gp, dp, theta, w, offsets, perm_slot, perm_token, S, H, E, act, yp, s); break;
-    case 384: launch_fused_nt<3>(xp, gp, dp, theta, w, offsets, perm_slot, perm_token, S, H, E, act, yp, s); break;
+    case 128: launch_fused_nt<1>(xp, gp, dp, theta, w, offsets, perm_slot, perm_token, S, H, E, act, xb, yp, s); break;
+    case 256: launch_fused_nt<2>(xp, gp, dp, theta, w, offsets, perm_slot, perm_token, S, H, E, act, xb, yp, s); break;
+    case 384: launch_fused_nt<3>(xp, gp, dp, theta, w, offsets, perm_slot, perm_token, S, H, E, act, xb, yp, s); break;
     default: return hipErrorInvalidValue;
   }
   return hipGetLastError();

@@ -9,7 +9,10 @@
 namespace bibo {
 namespace {
 
-constexpr int kLoadsPerPair = 1;
+#ifndef BIBO_LOADS_PER_PAIR
+#define BIBO_LOADS_PER_PAIR 1
+#endif
+constexpr int kLoadsPerPair = BIBO_LOADS_PER_PAIR;
 constexpr int kBK = 32;        // default K elements per LDS stage
 
 struct TileMap {
@@ -122,13 +125,22 @@ struct StripeLoader {
   }
 };
 
+// load instructions FIRST .. FIRST+COUNT-1 of a stage (those that exist)
+template <int FIRST, int COUNT, typename Loader>
+__device__ __forceinline__ void issue_some(const Loader& ld, int k_next, bf16_t* next_stage) {
+  if constexpr (COUNT > 0 && FIRST < Loader::kInstr) {
+    ld.template issue<FIRST>(k_next, next_stage);
+    issue_some<FIRST + 1, COUNT - 1>(ld, k_next, next_stage);
+  }
+}
+
 // One (k16 sub-step, N tile) pair of the software pipeline below; Q is a compile-time index so the
 // scheduling hints get constant arguments.  Pair Q also issues load instruction Q of the NEXT stage
 // (if there is one): spreading the loads through the MFMAs keeps the waves from queueing up at the
 // texture-address unit before they start multiplying.  `a1` points at this lane's A fragment of the
 // second sub-step for M tile 0; tile mt is `astride` elements further.
-template <int Q, int MT, int NTW, int BK, bool TR, typename Loader, typename FragRow>
-__device__ __forceinline__ void stripe_pair(floatx16 (&acc)[MT][NTW], bf16x8 (&a)[2][MT], bf16x8 (&b)[3],
+template <int Q, int MT, int NTW, int BK, bool TR, int NACC, int J0, typename Loader, typename FragRow>
+__device__ __forceinline__ void stripe_pair(floatx16 (&acc)[MT][NACC], bf16x8 (&a)[2][MT], bf16x8 (&b)[3],
                                             const bf16_t* a0, int astride, const bf16_t* bstage, int pos0,
                                             FragRow frag_row, const Loader& ld, bool prefetch, int k_next,
                                             bf16_t* next_stage) {
@@ -138,10 +150,7 @@ __device__ __forceinline__ void stripe_pair(floatx16 (&acc)[MT][NTW], bf16x8 (&a
   // kLoadsPerPair load instructions of the next stage per pair, starting with pair 0
   constexpr int kPer = (Loader::kInstr + kPairs - 1) / kPairs > kLoadsPerPair ? (Loader::kInstr + kPairs - 1) / kPairs
                                                                               : kLoadsPerPair;
-  if (prefetch) {
-    if constexpr (Q * kPer < Loader::kInstr) ld.template issue<Q * kPer>(k_next, next_stage);
-    if constexpr (kPer > 1 && Q * kPer + 1 < Loader::kInstr) ld.template issue<Q * kPer + 1>(k_next, next_stage);
-  }
+  if (prefetch) issue_some<Q * kPer, kPer>(ld, k_next, next_stage);
   if constexpr (Q + 2 < kPairs) {
     constexpr int s2 = (Q + 2) / NTW, j2 = (Q + 2) % NTW;
     b[(Q + 2) % 3] = *reinterpret_cast<const bf16x8*>(bstage + frag_row(j2) * BK + (pos0 ^ (s2 * 16)));
@@ -154,19 +163,19 @@ __device__ __forceinline__ void stripe_pair(floatx16 (&acc)[MT][NTW], bf16x8 (&a
     a[(s + 1) & 1][mt] = *reinterpret_cast<const bf16x8*>(a0 + mt * astride + ((pos0 ^ ((s + 1) * 16)) - pos0));
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
-    acc[mt][j] = TR ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[Q % 3], a[s & 1][mt], acc[mt][j], 0, 0, 0)
-                    : __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[s & 1][mt], b[Q % 3], acc[mt][j], 0, 0, 0);
+    acc[mt][J0 + j] = TR ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[Q % 3], a[s & 1][mt], acc[mt][J0 + j], 0, 0, 0)
+                         : __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[s & 1][mt], b[Q % 3], acc[mt][J0 + j], 0, 0, 0);
   constexpr int kReads = (Q + 2 < kPairs ? 1 : 0) + (kALast >= kAFirst ? kALast - kAFirst + 1 : 0);
   if constexpr (kReads > 0) __builtin_amdgcn_sched_group_barrier(0x100, kReads, 0);
   __builtin_amdgcn_sched_group_barrier(0x008, MT, 0);
 }
 
-template <int MT, int NTW, int BK, bool TR, typename Loader, typename FragRow, int... Qs>
-__device__ __forceinline__ void stripe_pairs(floatx16 (&acc)[MT][NTW], bf16x8 (&a)[2][MT], bf16x8 (&b)[3],
+template <int MT, int NTW, int BK, bool TR, int NACC, int J0, typename Loader, typename FragRow, int... Qs>
+__device__ __forceinline__ void stripe_pairs(floatx16 (&acc)[MT][NACC], bf16x8 (&a)[2][MT], bf16x8 (&b)[3],
                                              const bf16_t* a0, int astride, const bf16_t* bstage, int pos0,
                                              FragRow frag_row, const Loader& ld, bool prefetch, int k_next,
                                              bf16_t* next_stage, std::integer_sequence<int, Qs...>) {
-  (stripe_pair<Qs, MT, NTW, BK, TR>(acc, a, b, a0, astride, bstage, pos0, frag_row, ld, prefetch, k_next, next_stage), ...);
+  (stripe_pair<Qs, MT, NTW, BK, TR, NACC, J0>(acc, a, b, a0, astride, bstage, pos0, frag_row, ld, prefetch, k_next, next_stage), ...);
 }
 
 // Multiply one K step of BK into the accumulators while the load instructions of the next stage are
@@ -174,21 +183,21 @@ __device__ __forceinline__ void stripe_pairs(floatx16 (&acc)[MT][NTW], bf16x8 (&
 // through three buffers and are read two pairs ahead of the MFMAs that consume them; the A fragments
 // of the next sub-step are read while the current one is still multiplying.  a0: this lane's A
 // fragment of sub-step 0 for M tile 0 (position pos0 of its row; sub-step s sits at pos0 ^ 16s, M tile
-// mt `astride` elements further); bstage: this lane's row of the B stage (N tile 0).
-template <int MT, int NTW, int BK, bool TR, typename Loader, typename FragRow>
-__device__ __forceinline__ void stripe_step(floatx16 (&acc)[MT][NTW], const bf16_t* a0, int astride, const bf16_t* bstage,
+// mt `astride` elements further); bstage: this lane's row of the B stage (N tile 0).  The NTW tiles multiplied
+// here are columns J0 .. J0+NTW-1 of an accumulator array NACC tiles wide.
+template <int MT, int NTW, int BK, bool TR, int NACC = NTW, int J0 = 0, typename Loader, typename FragRow>
+__device__ __forceinline__ void stripe_step(floatx16 (&acc)[MT][NACC], const bf16_t* a0, int astride, const bf16_t* bstage,
                                             int pos0, FragRow frag_row, const Loader& ld, bool prefetch, int k_next,
                                             bf16_t* next_stage) {
   constexpr int SS = BK / 16;
-  static_assert(Loader::kInstr <= 2 * (SS * NTW), "at most two load instructions per pair");
   bf16x8 a[2][MT], b[3];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) a[0][mt] = *reinterpret_cast<const bf16x8*>(a0 + mt * astride);
   b[0] = *reinterpret_cast<const bf16x8*>(bstage + frag_row(0) * BK + pos0);
   b[1] = *reinterpret_cast<const bf16x8*>(bstage + frag_row(NTW > 1 ? 1 : 0) * BK + (NTW > 1 ? pos0 : (pos0 ^ 16)));
   __builtin_amdgcn_sched_group_barrier(0x100, MT + 2, 0);
-  stripe_pairs<MT, NTW, BK, TR>(acc, a, b, a0, astride, bstage, pos0, frag_row, ld, prefetch, k_next, next_stage,
-                            std::make_integer_sequence<int, SS * NTW>{});
+  stripe_pairs<MT, NTW, BK, TR, NACC, J0>(acc, a, b, a0, astride, bstage, pos0, frag_row, ld, prefetch, k_next, next_stage,
+                                          std::make_integer_sequence<int, SS * NTW>{});
 }
 
 // A and B both come from `stage` (A rows first).
