@@ -20,12 +20,18 @@ if str(ROOT) not in sys.path:
 PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
 
-# HBM-side bytes per launch of the dominant expert kernel on workload c2, from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE (KiB per dispatch), scaled by what the same counters read for a 256 MiB device copy
-# (FETCH_SIZE x2.0, WRITE_SIZE x1.0).  Fused kernel: 208.0 MB fetched + 76.4 MB written; gate/up kernel of the
-# two-kernel family: 158.4 MB + 37.7 MB.
-MEASURED_TRAFFIC_BYTES = {("c2", "gateup_down"): 284.4e6, ("c2", "gateup"): 196.1e6,
-                          ("c3", "stream"): 137.0e6 + 0.8e6 + 73.7e6 + 1.6e6}   # both streaming kernels, fetch + write
+REPEATS = 5                   # timed repeats of --steps forwards; the median is reported
+
+
+def measured_traffic(workload, kernel):
+    """HBM-side bytes per launch of a kernel, as the rocprofv3 --pmc summaries under profiles/ record them
+    (lines `traffic_bytes_per_launch <workload> <kernel> = <bytes>`); None when no profile covers it."""
+    import re
+    for f in sorted((ROOT / "profiles").glob("*.md")):
+        m = re.search(rf"^traffic_bytes_per_launch {workload} {kernel} = (\d+)", f.read_text(), re.M)
+        if m:
+            return int(m.group(1))
+    return None
 
 
 def flops_layer(T, H, E, k, I):
@@ -139,19 +145,37 @@ class Layer:
         if rc != 0:
             self.L.check(rc, name)
 
-    def time_forward(self, steps, warmup):
+    def time_forward(self, steps, warmup, repeats=REPEATS, weight_sets=1):
+        """Seconds per step: `repeats` timed runs of `steps` forwards each (after `warmup` untimed ones), every run
+        bracketed by a device synchronisation; returns (median, all runs).  weight_sets > 1 rotates the expert
+        weights over that many separately allocated copies, so that no step finds its weights in the 256 MB
+        Infinity Cache the step before left behind."""
         torch = self.torch
-        for _ in range(warmup):
-            self.forward()
-        torch.cuda.synchronize(self.dev)
-        t0 = time.perf_counter()
-        for _ in range(steps):
-            self.forward()
-        torch.cuda.synchronize(self.dev)
-        return (time.perf_counter() - t0) / steps
+        calls = [self._fwd_args]
+        if weight_sets > 1:
+            P = lambda t: ctypes.c_void_p(t.data_ptr())
+            self._rot = [(self.wgu.clone(), self.wd.clone()) for _ in range(weight_sets - 1)]
+            for gu, dn in self._rot:
+                a = list(self._fwd_args)
+                a[3], a[4] = P(gu), P(dn)
+                calls.append(tuple(a))
+        fn = self.lib.bibo_moe_forward
+        for i in range(warmup):
+            self.L.check(fn(*calls[i % len(calls)]), "bibo_moe_forward")
+        runs = []
+        for _ in range(repeats):
+            torch.cuda.synchronize(self.dev)
+            t0 = time.perf_counter()
+            for i in range(steps):
+                fn(*calls[i % len(calls)])
+            torch.cuda.synchronize(self.dev)
+            runs.append((time.perf_counter() - t0) / steps)
+        self._rot = None
+        return sorted(runs)[len(runs) // 2], runs
 
     def time_stages(self, steps):
-        """Average duration of each stage, HIP events on the launch stream around every call."""
+        """Average duration of each stage, HIP events on the launch stream around every call (an event pair also
+        spans the gap to the next launch, so a stage reads 1-2 us longer than its kernel alone)."""
         torch = self.torch
         names = list(self._stages)
         for n in names:
@@ -188,29 +212,55 @@ class Layer:
 
 
 def cpu_baseline(name, budget_s=20.0, sample_tokens=8192):
-    """The reference's eager CPU path (oracle restatement) timed on this box's host cores."""
+    """The reference's eager CPU path (oracle restatement) timed on this box's host cores: bf16 weights and
+    activations as the workload names them, and fp32 as a second line (CPU bf16 GEMMs are slow without a matrix
+    unit); 3 warm-up forwards, then at least 5 timed ones within the time budget, median."""
+    import statistics
     import torch
     from oracle import bibo_moe_oracle as O
     cfg = dict(O.CONFIGS[name])
     T = min(cfg["T"], sample_tokens)
     p = O.make_inputs(**{**cfg, "T": T})
     cores = torch.get_num_threads()
-    best = None
+    lines = {}
     for label, cast in (("bf16", lambda t: t), ("fp32", lambda t: t.float())):
         q = {k_: (cast(v) if isinstance(v, torch.Tensor) and v.dtype == torch.bfloat16 else v) for k_, v in p.items()}
-        O.eager_loop_forward(**q)                       # warm-up
-        t0 = time.perf_counter()
-        reps = 0
-        while reps < 3 or (time.perf_counter() - t0) < budget_s / 2:
+        for _ in range(3):
             O.eager_loop_forward(**q)
-            reps += 1
-        dt = (time.perf_counter() - t0) / max(reps, 1)
-        tps = T / dt
-        if best is None or tps > best[0]:
-            best = (tps, label, reps, dt)
-    return {"value": best[0], "unit": "tokens/s", "cores": cores, "kind": "port",
-            "sample": f"first {T} tokens of the {name} workload (same weights), eager per-expert loop in {best[1]}, "
-                      f"{best[2]} timed forwards of {best[3]:.2f} s after one warm-up"}
+        times = []
+        t_start = time.perf_counter()
+        while len(times) < 5 or (time.perf_counter() - t_start) < budget_s / 2:
+            t0 = time.perf_counter()
+            O.eager_loop_forward(**q)
+            times.append(time.perf_counter() - t0)
+            if len(times) >= 400:
+                break
+        med = statistics.median(times)
+        lines[label] = {"tokens_per_s": T / med, "median_s": med, "timed_forwards": len(times)}
+    best = max(lines, key=lambda l: lines[l]["tokens_per_s"])
+    return {"value": lines[best]["tokens_per_s"], "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": f"first {T} tokens of the {name} workload (same weights), eager per-expert loop; value = the faster "
+                      f"dtype ({best}); 3 warm-up forwards, median of the timed ones",
+            "bf16": lines["bf16"], "fp32": lines["fp32"]}
+
+
+def side_workload(name, dev, algo, steps, warmup):
+    """A parity-test workload timed next to the headline one: us/step, TFLOP/s, % of peak, load shape."""
+    import numpy as np
+    lay = Layer(name, dev, algo)
+    rel, active = lay.check()
+    sec, _ = lay.time_forward(steps, warmup)
+    cnt = np.bincount(lay.idx.cpu().numpy().reshape(-1), minlength=lay.E)
+    fl = flops_layer(lay.T, lay.H, lay.E, lay.k, lay.I)
+    nbytes = bytes_layer(lay.T, lay.H, lay.E, lay.k, lay.I, active)
+    hot = np.sort(cnt)[::-1]
+    return {"workload": f"{name}: T={lay.T} H={lay.H} E={lay.E} k={lay.k} I={lay.I} bf16", "kernel_family": lay.family,
+            "us_per_step": sec * 1e6, "tokens_per_s": lay.T / sec, "tflops": fl / sec / 1e12,
+            "pct_bf16_mfma_peak": 100.0 * fl / sec / 1e12 / PEAK_BF16_TFLOPS,
+            "algorithmic_gbs": nbytes / sec / 1e9, "pct_hbm_peak": 100.0 * nbytes / sec / 1e9 / PEAK_HBM_GBS,
+            "experts_active": active, "rows_per_expert_max": int(hot[0]), "rows_per_expert_min": int(hot[-1]),
+            "share_of_slots_on_4_busiest_experts": float(hot[:4].sum() / max(1, cnt.sum())),
+            "parity_rel_err_sample": rel}
 
 
 def main():
@@ -236,7 +286,7 @@ def main():
 
     layer = Layer(args.workload, dev, args.algo)
     rel, e_active = layer.check()
-    sec = layer.time_forward(args.steps, args.warmup)
+    sec, runs = layer.time_forward(args.steps, args.warmup)
     stages = layer.time_stages(max(10, min(args.steps, 100)))
     T, H, E, k, I, S = layer.T, layer.H, layer.E, layer.k, layer.I, layer.S
     fl = flops_layer(T, H, E, k, I)
@@ -250,22 +300,25 @@ def main():
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"{args.workload}: MoE layer forward T={T} H={H} E={E} k={k} I={I} bf16, seeded synthetic",
                    "algo": args.algo},
+        "timing": f"median of {REPEATS} timed runs of {args.steps} steps each", "ms_per_step_runs": [r * 1e3 for r in runs],
         "tflops": fl / sec / 1e12, "pct_bf16_mfma_peak": 100.0 * fl / sec / 1e12 / PEAK_BF16_TFLOPS,
         "parity_rel_err_sample": rel, "experts_active": e_active,
         "stage_us": {n: v * 1e6 for n, v in stages.items()},
+        "stage_us_note": "HIP events around each stage entry point; includes the gap to the next launch",
         "roofline": {"kernel": dom_name, "bound": "mfma",
                      "achieved": dom_flops / stages[dom] / 1e12, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": dom_flops / stages[dom] / 1e12 / PEAK_BF16_TFLOPS,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, dom))},
+                     "traffic": measured_traffic(args.workload, dom)},
     }
     if layer.family == "stream":
         # The streaming kernels only exist behind the composite call (the stage entry points time the tile kernels):
-        # the roofline of this workload is the HBM one, algorithmic bytes of the layer over the whole step.
+        # the roofline of this workload is the HBM one, algorithmic bytes of the layer over the whole step, with the
+        # expert weights rotated over four copies so that every step streams them from HBM.
         nbytes = bytes_layer(T, H, E, k, I, e_active)
-        out["roofline"] = {"kernel": "gateup_stream_kernel + down_stream_kernel (whole bibo_moe_forward step)", "bound": "hbm",
-                           "achieved": nbytes / sec / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                           "frac": nbytes / sec / 1e9 / PEAK_HBM_GBS,
-                           "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, "stream"))}
+        rsec, _ = layer.time_forward(args.steps, args.warmup, weight_sets=4)
+        out["roofline"] = {"kernel": "gateup_stream_kernel + down_stream_kernel (whole bibo_moe_forward step, 4 weight sets)",
+                           "bound": "hbm", "achieved": nbytes / rsec / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                           "frac": nbytes / rsec / 1e9 / PEAK_HBM_GBS, "traffic": measured_traffic(args.workload, "stream")}
         out["stage_us"] = {n: v for n, v in out["stage_us"].items() if n in ("router", "permute")}
     ffn_sec = layer.time_ffn_seam(args.steps, args.warmup)
     out["ffn_seam"] = {"entry": "bibo_moe_ffn_forward: out = h + moe(rmsnorm(h))", "us_per_step": ffn_sec * 1e6,
@@ -273,14 +326,22 @@ def main():
     if not args.no_decode and args.workload == "c2":
         d = Layer("c3", dev, args.algo)
         drel, dact = d.check()
-        dsec = d.time_forward(args.steps, args.warmup)
+        warm, _ = d.time_forward(args.steps, args.warmup)
+        sets = 4
+        rot, rot_runs = d.time_forward(args.steps, args.warmup, weight_sets=sets)
         db = bytes_layer(d.T, d.H, d.E, d.k, d.I, dact)
-        out["decode"] = {"workload": f"c3: T={d.T} H={d.H} E={d.E} k={d.k} I={d.I} bf16", "tokens_per_s": d.T / dsec,
-                         "us_per_step": dsec * 1e6, "algorithmic_bytes": db, "hbm_gbs": db / dsec / 1e9,
-                         "pct_hbm_peak": 100.0 * db / dsec / 1e9 / PEAK_HBM_GBS, "experts_active": dact,
-                         "parity_rel_err_sample": drel,
-                         "note": "whole layer through bibo_moe_forward (weight-streaming kernels); one weight set, "
-                                 "measured HBM and Infinity-Cache read rates on this part are equal (about 6 TB/s)"}
+        out["decode"] = {"workload": f"c3: T={d.T} H={d.H} E={d.E} k={d.k} I={d.I} bf16", "tokens_per_s": d.T / rot,
+                         "us_per_step": rot * 1e6, "algorithmic_bytes": db, "hbm_gbs": db / rot / 1e9,
+                         "pct_hbm_peak": 100.0 * db / rot / 1e9 / PEAK_HBM_GBS,
+                         "weight_sets": sets, "weight_bytes_rotated": sets * 2 * 3 * d.H * d.I * d.E,
+                         "cache_warm_us_per_step": warm * 1e6, "cache_warm_gbs": db / warm / 1e9,
+                         "cache_warm_pct_hbm_peak": 100.0 * db / warm / 1e9 / PEAK_HBM_GBS,
+                         "experts_active": dact, "parity_rel_err_sample": drel,
+                         "note": "whole layer through bibo_moe_forward (weight-streaming kernels); hbm_gbs rotates the "
+                                 "expert weights over 4 separately allocated sets (805 MB, more than the 256 MB Infinity "
+                                 "Cache) so every step streams them from HBM; cache_warm re-reads one 201 MB set"}
+        out["c1"] = side_workload("c1", dev, args.algo, args.steps, args.warmup)
+        out["c4"] = side_workload("c4", dev, args.algo, max(10, args.steps // 2), args.warmup)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args.workload)
     print(json.dumps(out))
