@@ -14,7 +14,7 @@ NORM_NONE, NORM_SUM, NORM_SOFTMAX = 0, 1, 2
 ALGO_AUTO, ALGO_GENERIC, ALGO_MFMA, ALGO_STREAM, ALGO_FUSED = 0, 1, 2, 3, 4
 MAX_EXPERTS, MAX_TOPK = 64, 8
 ACT_RADIAL_SIGMOID, ACT_RADIAL_TANH, ACT_SILU = 0, 1, 2
-FLAG_ROUND_BLOCK_OUT = 1
+FLAG_ROUND_BLOCK_OUT, FLAG_NO_RESIDUAL = 1, 2
 ABI_VERSION = 3
 
 # every symbol include/bibo_moe.h declares
@@ -68,8 +68,8 @@ def _declare(l):
     l.bibo_moe_ffn_workspace_bytes.restype = ci
     l.bibo_moe_ffn_workspace_bytes.argtypes = [ctypes.POINTER(Shape), ctypes.POINTER(sz)]
     l.bibo_moe_ffn_forward.restype = ci
-    l.bibo_moe_ffn_forward.argtypes = [vp, vp, ctypes.c_float, vp, vp, vp, vp, vp, ctypes.POINTER(Shape), ci, ci, vp, vp, vp,
-                                       vp, vp, sz, vp]
+    l.bibo_moe_ffn_forward.argtypes = [vp, vp, ctypes.c_float, vp, vp, vp, vp, vp, vp, ctypes.POINTER(Shape), ci, ci, vp, vp,
+                                       vp, vp, vp, sz, vp]
     l.bibo_moe_forward_static.restype = ci
     l.bibo_moe_forward_static.argtypes = [vp, vp, vp, vp, vp, vp, ctypes.POINTER(Shape), ci, ci, vp, vp, vp, vp, vp, vp]
     l.bibo_moe_forward.restype = ci

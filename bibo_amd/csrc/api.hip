@@ -443,8 +443,8 @@ int bibo_moe_ffn_workspace_bytes(const bibo_moe_shape* sh, size_t* out) {
   return BIBO_OK;
 }
 
-int bibo_moe_ffn_forward(const void* h, const float* norm_weight, float eps, const void* w_router, const float* bias,
-                         const void* w_gate_up, const void* w_down, const float* theta, const bibo_moe_shape* sh,
+int bibo_moe_ffn_forward(const void* h, const float* norm_weight, float eps, const void* residual, const void* w_router,
+                         const float* bias, const void* w_gate_up, const void* w_down, const float* theta, const bibo_moe_shape* sh,
                          int norm_mode, int algo, void* out, int32_t* idx_out, float* w_out, int32_t* counts_out,
                          void* workspace, size_t workspace_bytes, void* stream) {
   if (sh == nullptr) return BIBO_ERR_NULL_POINTER;
@@ -459,7 +459,9 @@ int bibo_moe_ffn_forward(const void* h, const float* norm_weight, float eps, con
   void* xn = static_cast<char*>(workspace) + inner;              // post_attention_layernorm(h), layers.py:60
   const hipError_t e = launch_rmsnorm(h, norm_weight, eps, sh->T, sh->H, sh->dtype, xn, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return (int)e;
-  return forward_impl(xn, w_router, bias, w_gate_up, w_down, theta, sh, norm_mode, algo, h, out, idx_out, w_out,
+  // what the block's output is added to: h itself (layers.py:62-64), another tensor, or nothing
+  const void* res = (sh->flags & BIBO_FLAG_NO_RESIDUAL) ? nullptr : (residual != nullptr ? residual : h);
+  return forward_impl(xn, w_router, bias, w_gate_up, w_down, theta, sh, norm_mode, algo, res, out, idx_out, w_out,
                       counts_out, nullptr, workspace, inner, stream);
 }
 

@@ -333,14 +333,16 @@ class BiBoMoELayer(nn.Module):
 
     @_no_compile
     def ffn_forward(self, hidden_states: torch.Tensor, norm_weight: torch.Tensor, eps: float,
-                    bf16_stream: bool = False, bf16_moe_out: bool = False) -> torch.Tensor:
+                    bf16_stream: bool = False, bf16_moe_out: bool = False, residual=None) -> torch.Tensor:
         """The caller's seam, BiBoDecoderLayer._ffn_forward (src/modeling/layers.py:57-67):
         `hidden_states + self(rmsnorm(hidden_states))` with `norm_weight`/`eps` of post_attention_layernorm
         (src/modeling/norm.py:19-24), as ONE library call: the norm feeds the block from the workspace and the
         residual is added in the combine kernel.  With hooks or a gap probe present, or with an fp32 stream
         under bf16 autocast, the block runs as in forward and norm and residual are ordinary tensor operations
         around it.  `bf16_stream` and `bf16_moe_out` are the decoder layer's two switches (layers.py:28,37):
-        the sum is cast to bf16, and the block's output is rounded to bf16 before it enters the sum."""
+        the sum is cast to bf16, and the block's output is rounded to bf16 before it enters the sum.
+        `residual`: None adds `hidden_states` itself; a tensor of the same shape is added instead; False adds
+        nothing (norm + block only: `_attn_res_mlp_forward` of the experimental layer, exp/modeling_bibo.py:429-431)."""
         bsz, seq, hdim = hidden_states.shape
         num_tokens = bsz * seq
         if (self._hooks_present() or self.use_shared_expert or hidden_states.dtype != _compute_dtype(hidden_states)
@@ -350,7 +352,8 @@ class BiBoMoELayer(nn.Module):
             xn = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)).to(hidden_states.dtype)    # norm.py:21-24
             blk = self.forward(norm_weight * xn)                                                       # layers.py:60-61
             blk = blk.to(torch.bfloat16) if bf16_moe_out else blk                                      # layers.py:62-63
-            out = hidden_states + blk.to(hidden_states.dtype)                                          # layers.py:64
+            base = hidden_states if residual is None else residual
+            out = blk.to(hidden_states.dtype) if residual is False else base + blk.to(hidden_states.dtype)   # layers.py:64
             return out.to(torch.bfloat16) if bf16_stream else out
         balancing = self.training and self.bias_update_factor > 0
         _forward_only_guard(hidden_states, self.gate.gate_proj.weight, self.experts.gate_up_proj)
@@ -364,7 +367,9 @@ class BiBoMoELayer(nn.Module):
         out, _, _, counts = ops.ffn_forward(h, nw, float(eps), wr, b, gu, dn, th, self.num_experts_per_tok,
                                             norm=self.gate.norm_topk_prob, algo=self.experts.algo, want_counts=balancing,
                                             n_pos=self.experts.num_pos, n_neg=self.experts.num_neg, act=self.experts.act,
-                                            round_block_out=bf16_moe_out and cd == torch.bfloat16)
+                                            round_block_out=bf16_moe_out and cd == torch.bfloat16,
+                                            residual=(residual if residual is None or residual is False
+                                                      else residual.detach().reshape(num_tokens, hdim).to(cd).contiguous()))
         if balancing:                                          # exactly once per training forward
             tpe = self._balance_step(None, num_tokens, counts=counts)
             if tpe is not None:

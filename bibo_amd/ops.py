@@ -300,9 +300,13 @@ def rmsnorm_fwd(x, norm_weight, eps):
 
 
 def ffn_forward(h, norm_weight, eps, w_router, bias, w_gate_up, w_down, theta, k, norm="sum", algo="auto",
-                want_routing=False, want_counts=False, n_pos=0, n_neg=0, act="radial", round_block_out=False):
+                want_routing=False, want_counts=False, n_pos=0, n_neg=0, act="radial", round_block_out=False,
+                residual=None, out=None):
     """Seam 3 (the block's caller).  -> out = h + moe(rmsnorm(h)) [T,H], idx|None, w|None, counts|None.
-    round_block_out: round the block's output to h.dtype before the residual add (bf16_moe_out, layers.py:62-63)."""
+    round_block_out: round the block's output to h.dtype before the residual add (bf16_moe_out, layers.py:62-63).
+    residual: None adds h itself (layers.py:57-64); a [T,H] tensor is added instead of h; False adds nothing,
+    out = moe(rmsnorm(h)) (the experimental layer's _attn_res_mlp_forward, exp/modeling_bibo.py:429-431).
+    out: optional preallocated result (may be the residual tensor)."""
     T, H = h.shape
     Eg, two_i, _ = w_gate_up.shape
     E = Eg + n_pos + n_neg
@@ -312,16 +316,25 @@ def ffn_forward(h, norm_weight, eps, w_router, bias, w_gate_up, w_down, theta, k
     _chk(bias, "bias", torch.float32, (E,)); _chk(w_gate_up, "w_gate_up", h.dtype, (Eg, 2 * I, H))
     _chk(w_down, "w_down", h.dtype, (Eg, H, I)); _chk(theta, "theta", torch.float32, (Eg,))
     dev = h.device
-    out = torch.empty(T, H, dtype=h.dtype, device=dev)
+    if out is None:
+        out = torch.empty(T, H, dtype=h.dtype, device=dev)
+    else:
+        _chk(out, "out", h.dtype, (T, H))
+    flags = L.FLAG_ROUND_BLOCK_OUT if round_block_out else 0
+    if residual is False:
+        flags |= L.FLAG_NO_RESIDUAL
+        residual = None
+    elif residual is not None:
+        _chk(residual, "residual", h.dtype, (T, H))
     idx = torch.empty(T, k, dtype=torch.int32, device=dev) if want_routing else None
     w = torch.empty(T, k, dtype=torch.float32, device=dev) if want_routing else None
     counts = torch.empty(E, dtype=torch.int32, device=dev) if want_counts else None
-    sh = L.Shape(T, H, E, k, I, dc, n_pos, n_neg, act_code(act), L.FLAG_ROUND_BLOCK_OUT if round_block_out else 0)
+    sh = L.Shape(T, H, E, k, I, dc, n_pos, n_neg, act_code(act), flags)
     nbytes = ctypes.c_size_t(0)
     L.check(L.lib().bibo_moe_ffn_workspace_bytes(ctypes.byref(sh), ctypes.byref(nbytes)), "bibo_moe_ffn_workspace_bytes")
     ws = workspace(dev, nbytes.value)
     with torch.cuda.device(dev):
-        L.check(L.lib().bibo_moe_ffn_forward(_ptr(h), _ptr(norm_weight), ctypes.c_float(eps), _ptr(w_router), _ptr(bias),
+        L.check(L.lib().bibo_moe_ffn_forward(_ptr(h), _ptr(norm_weight), ctypes.c_float(eps), _ptr(residual), _ptr(w_router), _ptr(bias),
                                              _ptr(w_gate_up), _ptr(w_down), _ptr(theta), ctypes.byref(sh),
                                              norm_mode(norm), algo_code(algo), _ptr(out), _ptr(idx), _ptr(w),
                                              _ptr(counts), _ptr(ws), ws.numel(), _stream(dev)), "bibo_moe_ffn_forward")

@@ -62,7 +62,11 @@ enum bibo_flags {
   /* bibo_moe_ffn_forward only: round the block's output to `dtype` before the residual is added, then round the sum
      (bf16_moe_out of the reference's decoder layer, src/modeling/layers.py:37,62-63).  Without it the sum is formed
      in fp32 and rounded once. */
-  BIBO_FLAG_ROUND_BLOCK_OUT = 1
+  BIBO_FLAG_ROUND_BLOCK_OUT = 1,
+  /* bibo_moe_ffn_forward only: no residual at all, out = moe(rmsnorm(h)): the block as the reference's experimental
+     decoder layer calls it under Block Attention Residuals (exp/modeling_bibo.py:429-431), where the caller owns
+     the sum. */
+  BIBO_FLAG_NO_RESIDUAL = 2
 };
 
 /* kernel family for the expert GEMMs */
@@ -242,11 +246,16 @@ int bibo_moe_forward_static(const void* x, const void* w_router, const float* bi
  * with norm_weight fp32 [H].  The normalised activations live in the workspace; the residual add happens in
  * the combine, in fp32, before the single rounding to `dtype` (the reference rounds the block output first).
  * h, out [T,H] in `dtype` (out may not alias h).  Workspace size: bibo_moe_ffn_workspace_bytes.
+ * `residual` [T,H] in `dtype` or NULL: what the block's output is added to.  NULL means h itself (layers.py:57-64).
+ * Another tensor gives out = residual + moe(rmsnorm(h)): the experimental layer's
+ * `prefix_sum = prefix_sum + mlp(post_attention_layernorm(h))` (exp/modeling_bibo.py:429-431,666) in one call;
+ * out may alias residual.  With BIBO_FLAG_NO_RESIDUAL in shape->flags nothing is added and `residual` is ignored.
  */
 int bibo_moe_rmsnorm_fwd(const void* x, const float* norm_weight, float eps, int T, int H, int dtype, void* out,
                          void* stream);                 /* the norm alone: out = weight * round(x * rsqrt(mean x^2 + eps)) */
 int bibo_moe_ffn_workspace_bytes(const bibo_moe_shape* shape, size_t* out_bytes);
-int bibo_moe_ffn_forward(const void* h, const float* norm_weight, float eps, const void* w_router, const float* bias,
+int bibo_moe_ffn_forward(const void* h, const float* norm_weight, float eps, const void* residual, const void* w_router,
+                         const float* bias,
                          const void* w_gate_up, const void* w_down, const float* theta, const bibo_moe_shape* shape,
                          int norm_mode, int algo, void* out, int32_t* idx_out, float* w_out, int32_t* counts_out,
                          void* workspace, size_t workspace_bytes, void* stream);

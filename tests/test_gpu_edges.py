@@ -66,7 +66,7 @@ def test_misaligned_operands_are_reported_not_launched():
     w = torch.ones(T, k, dtype=torch.float32, device=DEV)
     assert lib.bibo_moe_experts_fwd(P(x), P(idx), P(w), P(gu), P(dn), P(th), ctypes.byref(sh), L.ALGO_AUTO, P(out), None,
                                     ctypes.c_void_p(big.data_ptr() + 16), ws.numel(), stream) == -5
-    assert lib.bibo_moe_ffn_forward(P(x), P(th.new_ones(H)), ctypes.c_float(1e-6), P(wr), P(b), P(gu), P(dn), P(th),
+    assert lib.bibo_moe_ffn_forward(P(x), P(th.new_ones(H)), ctypes.c_float(1e-6), None, P(wr), P(b), P(gu), P(dn), P(th),
                                     ctypes.byref(sh), L.NORM_SUM, L.ALGO_AUTO, P(out), None, None, None,
                                     ctypes.c_void_p(big.data_ptr() + 16), big.numel() - 16, stream) == -5
     gen = out.clone()
@@ -101,6 +101,6 @@ def test_workspace_too_small_is_an_error():
     rc = lib.bibo_moe_forward(P(x), P(wr), P(b), P(gu), P(dn), P(th), ctypes.byref(sh), L.NORM_SUM, L.ALGO_AUTO, P(out),
                               None, None, None, None, P(ws), need - 1, None)
     assert rc == -4
-    rc = lib.bibo_moe_ffn_forward(P(x), P(th.new_ones(H)), ctypes.c_float(1e-6), P(wr), P(b), P(gu), P(dn), P(th),
+    rc = lib.bibo_moe_ffn_forward(P(x), P(th.new_ones(H)), ctypes.c_float(1e-6), None, P(wr), P(b), P(gu), P(dn), P(th),
                                   ctypes.byref(sh), L.NORM_SUM, L.ALGO_AUTO, P(out), None, None, None, P(ws), need, None)
     assert rc == -4                                                # the seam needs room for the normalised rows too

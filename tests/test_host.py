@@ -75,7 +75,7 @@ def test_argument_errors_are_reported_without_a_gpu():
     ffn = ctypes.c_size_t(0)
     assert lib.bibo_moe_ffn_workspace_bytes(ctypes.byref(ok), ctypes.byref(ffn)) == 0
     assert ffn.value >= out.value + 8192 * 768 * 2                 # the block's workspace plus the normalised activations
-    assert lib.bibo_moe_ffn_forward(None, None, ctypes.c_float(1e-6), None, None, None, None, None, ctypes.byref(ok), 1, 0,
+    assert lib.bibo_moe_ffn_forward(None, None, ctypes.c_float(1e-6), None, None, None, None, None, None, ctypes.byref(ok), 1, 0,
                                     None, None, None, None, None, 0, None) == -1
     assert b"workspace" in lib.bibo_moe_strerror(-4)
     with pytest.raises(RuntimeError, match="workspace"):
