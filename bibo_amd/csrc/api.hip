@@ -189,11 +189,14 @@ int experts_dispatch(const void* x, const void* wgu, const void* wd, const float
   return down_dispatch(base + ws.hidden, wd, w, offsets, perm_slot, ca, T, H, Eg, k, I, dtype, algo, out, yw, s);
 }
 
-// The whole layer on `x`; `residual` (or NULL) is added in the combine.
+// The whole layer on `x`; `residual` (or NULL) is added in the combine.  With `norm_src` given, `x` is a buffer the
+// router kernel first fills with RMSNorm(norm_src) (weight `norm_weight`, `eps`): the caller's seam in one read of
+// the raw rows.
 int forward_impl(const void* x, const void* w_router, const float* bias, const void* w_gate_up, const void* w_down,
                  const float* theta, const bibo_moe_shape* sh, int norm_mode, int algo, const void* residual, void* out,
                  int32_t* idx_out, float* w_out, int32_t* counts_out, float* logits_out, void* workspace,
-                 size_t workspace_bytes, void* stream) {
+                 size_t workspace_bytes, void* stream, const void* norm_src = nullptr, const float* norm_weight = nullptr,
+                 float eps = 0.f) {
   if (sh == nullptr) return BIBO_ERR_NULL_POINTER;
   const int T = sh->T, H = sh->H, E = sh->E, k = sh->k, I = sh->I, dtype = sh->dtype;
   int rc = check_dims(T, H, E, k, I, dtype, sh->n_pos, sh->n_neg);
@@ -223,8 +226,12 @@ int forward_impl(const void* x, const void* w_router, const float* bias, const v
   int32_t* hist = reinterpret_cast<int32_t*>(base + ws.hist);
   int hist_tokens = 0;
   const bool want_hist = need_permute && T > 0 && permute_takes_router_hist(T, k);
-  if (T > 0 && (rc = hip_rc(launch_router(x, w_router, bias, T, H, E, k, dtype, norm_mode, logits_out, idx, w, nullptr,
-                                          want_hist ? hist : nullptr, &hist_tokens, s))) != BIBO_OK)
+  if (T > 0 && norm_src != nullptr) {
+    rc = hip_rc(launch_router_norm(norm_src, norm_weight, eps, w_router, bias, T, H, E, k, norm_mode, const_cast<void*>(x),
+                                   logits_out, idx, w, want_hist ? hist : nullptr, &hist_tokens, s));
+    if (rc != BIBO_OK) return rc;
+  } else if (T > 0 && (rc = hip_rc(launch_router(x, w_router, bias, T, H, E, k, dtype, norm_mode, logits_out, idx, w, nullptr,
+                                                 want_hist ? hist : nullptr, &hist_tokens, s))) != BIBO_OK)
     return rc;
   if (need_permute) {
     const hipError_t e = (want_hist && hist_tokens > 0)
@@ -457,10 +464,14 @@ int bibo_moe_ffn_forward(const void* h, const float* norm_weight, float eps, con
   const size_t xn_bytes = align_up((size_t)sh->T * sh->H * elt_size(sh->dtype));
   if (workspace_bytes < inner + xn_bytes) return BIBO_ERR_WORKSPACE_TOO_SMALL;
   void* xn = static_cast<char*>(workspace) + inner;              // post_attention_layernorm(h), layers.py:60
-  const hipError_t e = launch_rmsnorm(h, norm_weight, eps, sh->T, sh->H, sh->dtype, xn, static_cast<hipStream_t>(stream));
-  if (e != hipSuccess) return (int)e;
   // what the block's output is added to: h itself (layers.py:62-64), another tensor, or nothing
   const void* res = (sh->flags & BIBO_FLAG_NO_RESIDUAL) ? nullptr : (residual != nullptr ? residual : h);
+  if (sh->T > 0 && w_router != nullptr && router_norm_supported(sh->H, sh->dtype, h, w_router, xn))
+    // the router kernel normalises the rows it reads and leaves them in xn: no norm launch, one read of h
+    return forward_impl(xn, w_router, bias, w_gate_up, w_down, theta, sh, norm_mode, algo, res, out, idx_out, w_out,
+                        counts_out, nullptr, workspace, inner, stream, h, norm_weight, eps);
+  const hipError_t e = launch_rmsnorm(h, norm_weight, eps, sh->T, sh->H, sh->dtype, xn, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return (int)e;
   return forward_impl(xn, w_router, bias, w_gate_up, w_down, theta, sh, norm_mode, algo, res, out, idx_out, w_out,
                       counts_out, nullptr, workspace, inner, stream);
 }

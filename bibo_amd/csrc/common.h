@@ -131,6 +131,10 @@ __device__ __forceinline__ int xcd_tile(int bid, int total) {
 hipError_t launch_router(const void* x, const void* w_router, const float* bias, int T, int H, int E, int k, int dtype,
                          int norm_mode, float* logits, int32_t* idx, float* w, float* gap, int32_t* chunk_hist,
                          int* hist_tokens, hipStream_t s);
+bool router_norm_supported(int H, int dtype, const void* h, const void* w_router, const void* xn);
+hipError_t launch_router_norm(const void* h, const float* norm_weight, float eps, const void* w_router, const float* bias,
+                              int T, int H, int E, int k, int norm_mode, void* xn, float* logits, int32_t* idx, float* w,
+                              int32_t* chunk_hist, int* hist_tokens, hipStream_t s);
 size_t permute_workspace_bytes(int T);
 hipError_t launch_permute(const int32_t* idx, int T, int E, int k, int32_t* counts, int32_t* offsets,
                           int32_t* perm_slot, int32_t* perm_token, void* ws, hipStream_t s);

@@ -247,6 +247,43 @@ constexpr int kRouterGran = kRouterKC / 8;           // 16-byte granules per chu
 typedef __attribute__((address_space(3))) void router_lds_void;
 typedef const __attribute__((address_space(1))) void router_gbl_void;
 
+// Everything after the logits of a TOK-token workgroup: canonical sigmoid on the accumulator registers, selection,
+// weights, and the workgroup's histogram of selected experts.  Wave (tm, en) holds the 16x16 logits tile of token
+// tile tm and expert tile en: lane = column (expert) lane%16, rows (tokens) 4*(lane/16)+i.
+template <int TOK>
+__device__ __forceinline__ void router_finish(const floatx4& acc, float* sc, const float* bias_s, int T, int E, int k,
+                                              int norm_mode, int t0, float* __restrict__ logits, int32_t* __restrict__ idx,
+                                              float* __restrict__ w, float* __restrict__ gap,
+                                              int32_t* __restrict__ chunk_hist) {
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63;
+  const int tm = wave >> 2, en = wave & 3;
+  const int r16 = lane & 15, kc = lane >> 4;
+  const int ntok = min(TOK, T - t0);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int tl = tm * 16 + kc * 4 + i, e = en * 16 + r16;
+    if (tl < ntok && e < E) {
+      const float lg = acc[i];
+      if (logits != nullptr) logits[(size_t)(t0 + tl) * E + e] = lg;
+      sc[tl * kRowPad + e] = sigmoid32_canonical(lg);          // router.py:31
+    }
+  }
+  __syncthreads();
+  const unsigned long long mask = select_tokens16(sc, bias_s, E, k, norm_mode, t0, ntok, idx, w, gap);
+  if (chunk_hist != nullptr) {           // histogram of this workgroup's selections, for the permutation kernel
+    __shared__ unsigned long long mask_s[TOK];
+    if ((tid & 15) == 0) mask_s[tid >> 4] = mask;
+    __syncthreads();
+    if (tid < kMaxE) {
+      int c = 0;
+#pragma unroll
+      for (int t = 0; t < TOK; ++t) c += (int)((mask_s[t] >> tid) & 1ull);
+      chunk_hist[blockIdx.x * kMaxE + tid] = c;
+    }
+  }
+}
+
 template <int TOK>
 __global__ __launch_bounds__(TOK * 16) void router_mfma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wr,
                                                                const float* __restrict__ bias, int T, int H, int E,
@@ -309,30 +346,124 @@ __global__ __launch_bounds__(TOK * 16) void router_mfma_kernel(const bf16_t* __r
       multiply(st1);
     }
   }
-  // D layout of the 16x16 tile: lane holds column (expert) lane%16, rows (tokens) 4*(lane/16)+i
-  const int ntok = min(TOK, T - t0);
+  router_finish<TOK>(acc, sc, bias_s, T, E, k, norm_mode, t0, logits, idx, w, gap, chunk_hist);
+}
+
+// ---- MFMA router with the block's input RMSNorm in front (the caller's seam) ----------------------
+// out = h + moe(post_attention_layernorm(h)) (src/modeling/layers.py:57-64) needs the normalised rows twice: as the
+// router's operand and as the rows the expert kernels gather.  This kernel reads the raw rows once: all H elements of
+// its TOK rows arrive in LDS by LDS-DMA, one wave per row computes BiBoRMSNorm (src/modeling/norm.py:19-24) with the
+// arithmetic and the summation order of rmsnorm_bf16x8_kernel (so both produce the same bits), writes the normalised
+// row back to LDS in place and to `xn` in memory, and the logits are then multiplied from the resident rows while
+// w_router streams through two LDS stages as in router_mfma_kernel.  x rows are stored as H/128 chunks of
+// [TOK][128], granule c of a chunk row r at position c ^ (r & 15).
+template <int TOK>
+__global__ __launch_bounds__(TOK * 16) void router_norm_mfma_kernel(const bf16_t* __restrict__ h, const float* __restrict__ nw,
+                                                                    float eps, const bf16_t* __restrict__ wr,
+                                                                    const float* __restrict__ bias, int T, int H, int E,
+                                                                    int k, int norm_mode, bf16_t* __restrict__ xn,
+                                                                    float* __restrict__ logits, int32_t* __restrict__ idx,
+                                                                    float* __restrict__ w, float* __restrict__ gap,
+                                                                    int32_t* __restrict__ chunk_hist) {
+  constexpr int kThreads = TOK * 16;
+  constexpr int kWPer = kMaxE * kRouterGran / kThreads;      // w_router load instructions per thread and chunk
+  extern __shared__ __attribute__((aligned(16))) bf16_t xs[];                 // [H/128][TOK][128]
+  __shared__ __attribute__((aligned(16))) bf16_t wst0[kMaxE * kRouterKC];
+  __shared__ __attribute__((aligned(16))) bf16_t wst1[kMaxE * kRouterKC];
+  __shared__ float sc[TOK * kRowPad];
+  __shared__ float bias_s[kMaxE];
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63;
+  const int t0 = blockIdx.x * TOK;
+  const int nchunks = H / kRouterKC;
+  if (tid < kMaxE) bias_s[tid] = (tid < E) ? bias[tid] : 0.f;
+
+  // w_router chunk loads: thread t of instruction i fills granule i*kThreads + t = (row, position t % 16)
+  const bf16_t* wsrc[kWPer];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int tl = tm * 16 + kc * 4 + i, e = en * 16 + r16;
-    if (tl < ntok && e < E) {
-      const float lg = acc[i];
-      if (logits != nullptr) logits[(size_t)(t0 + tl) * E + e] = lg;
-      sc[tl * kRowPad + e] = sigmoid32_canonical(lg);          // router.py:31
-    }
+  for (int i = 0; i < kWPer; ++i) {
+    const int row = (i * kThreads + tid) / kRouterGran;
+    wsrc[i] = wr + (size_t)min(row, E - 1) * H + ((tid & (kRouterGran - 1)) ^ (row & 15)) * 8;
   }
+  auto issue_w = [&](int k0, bf16_t* st) {
+#pragma unroll
+    for (int i = 0; i < kWPer; ++i)
+      __builtin_amdgcn_global_load_lds((router_gbl_void*)(wsrc[i] + k0), (router_lds_void*)(st + (i * kThreads + wave * 64) * 8),
+                                       16, 0, 0);
+  };
+  issue_w(0, wst0);
+  // the raw rows: instruction i is chunk i of every row (TOK * 16 granules = one per thread)
+  {
+    const int row = tid >> 4;
+    const bf16_t* src = h + (size_t)min(t0 + row, T - 1) * H + ((tid & 15) ^ (row & 15)) * 8;
+    for (int i = 0; i < nchunks; ++i)
+      __builtin_amdgcn_global_load_lds((router_gbl_void*)(src + i * kRouterKC),
+                                       (router_lds_void*)(xs + (i * kThreads + wave * 64) * 8), 16, 0, 0);
+  }
+  __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
-  const unsigned long long mask = select_tokens16(sc, bias_s, E, k, norm_mode, t0, ntok, idx, w, gap);
-  if (chunk_hist != nullptr) {           // histogram of this workgroup's selections, for the permutation kernel
-    __shared__ unsigned long long mask_s[TOK];
-    if ((tid & 15) == 0) mask_s[tid >> 4] = mask;
-    __syncthreads();
-    if (tid < kMaxE) {
-      int c = 0;
+  // RMSNorm, one wave per row, four rows per wave; lane takes logical granules u*64 + lane of the row
+  {
+    const int ngran = H / 8;
 #pragma unroll
-      for (int t = 0; t < TOK; ++t) c += (int)((mask_s[t] >> tid) & 1ull);
-      chunk_hist[blockIdx.x * kMaxE + tid] = c;
+    for (int j = 0; j < 4; ++j) {
+      const int r = wave * 4 + j;
+      bf16x8 v[4];
+      bf16_t* loc[4];
+      float ss = 0.f;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int c = u * kWave + lane;
+        if (c < ngran) {
+          loc[u] = xs + (((c >> 4) * TOK + r) * kRouterGran + ((c & 15) ^ (r & 15))) * 8;
+          v[u] = *reinterpret_cast<const bf16x8*>(loc[u]);
+#pragma unroll
+          for (int q = 0; q < 8; ++q) ss = fmaf((float)v[u][q], (float)v[u][q], ss);
+        }
+      }
+      ss = wave_sum(ss);
+      const float rinv = rsqrtf(ss / (float)H + eps);                                   // norm.py:22-23
+      const bool live = t0 + r < T;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int c = u * kWave + lane;
+        if (c < ngran) {
+          bf16x8 o;
+#pragma unroll
+          for (int q = 0; q < 8; ++q) o[q] = (bf16_t)(nw[c * 8 + q] * (float)(bf16_t)((float)v[u][q] * rinv));   // norm.py:24
+          *reinterpret_cast<bf16x8*>(loc[u]) = o;
+          if (live) *reinterpret_cast<bf16x8*>(xn + (size_t)(t0 + r) * H + c * 8) = o;
+        }
+      }
     }
   }
+  const int tm = wave >> 2, en = wave & 3;
+  const int r16 = lane & 15, kc = lane >> 4;
+  floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+  auto multiply = [&](const bf16_t* xa, const bf16_t* st) {
+    const bf16_t* arow = xa + (tm * 16 + r16) * kRouterKC;
+    const bf16_t* brow = st + (en * 16 + r16) * kRouterKC;
+#pragma unroll
+    for (int s = 0; s < kRouterKC / 32; ++s) {
+      const int pos = ((s * 4 + kc) ^ r16) * 8;
+      const bf16x8 a = *reinterpret_cast<const bf16x8*>(arow + pos);
+      const bf16x8 b = *reinterpret_cast<const bf16x8*>(brow + pos);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+    }
+  };
+  for (int c0 = 0; c0 < nchunks; c0 += 2) {
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();                                   // first pass: also the normalised rows of the other waves
+    if (c0 + 1 < nchunks) issue_w((c0 + 1) * kRouterKC, wst1);
+    multiply(xs + (size_t)c0 * TOK * kRouterKC, wst0);
+    if (c0 + 1 < nchunks) {
+      __builtin_amdgcn_s_waitcnt(0);
+      __syncthreads();
+      if (c0 + 2 < nchunks) issue_w((c0 + 2) * kRouterKC, wst0);
+      multiply(xs + (size_t)(c0 + 1) * TOK * kRouterKC, wst1);
+    }
+  }
+  router_finish<TOK>(acc, sc, bias_s, T, E, k, norm_mode, t0, logits, idx, w, gap, chunk_hist);
 }
 
 // ---- MFMA router for H % 32 == 0 but not % 128: operands straight to registers, K split over 4 waves ----
@@ -402,6 +533,42 @@ __global__ __launch_bounds__(256) void router_mfma_split_kernel(const bf16_t* __
 }
 
 }  // namespace
+
+// The widest hidden size whose TOK raw rows fit LDS next to the w_router stages (TOK = 32: 64 KB of rows).
+bool router_norm_supported(int H, int dtype, const void* h, const void* w_router, const void* xn) {
+  const bool aligned = ((reinterpret_cast<uintptr_t>(h) | reinterpret_cast<uintptr_t>(w_router) |
+                         reinterpret_cast<uintptr_t>(xn)) & 15) == 0;
+  return dtype == BIBO_DTYPE_BF16 && (H % kRouterKC) == 0 && H <= 1024 && aligned;
+}
+
+// RMSNorm + router in one launch (see router_norm_mfma_kernel); `xn` receives the normalised rows.
+hipError_t launch_router_norm(const void* h, const float* norm_weight, float eps, const void* w_router, const float* bias,
+                              int T, int H, int E, int k, int norm_mode, void* xn, float* logits, int32_t* idx, float* w,
+                              int32_t* chunk_hist, int* hist_tokens, hipStream_t s) {
+  if (hist_tokens != nullptr) *hist_tokens = 0;
+  if (T == 0) return hipSuccess;
+  const bf16_t* hp = static_cast<const bf16_t*>(h);
+  const bf16_t* wp = static_cast<const bf16_t*>(w_router);
+  bf16_t* xp = static_cast<bf16_t*>(xn);
+  if (T >= 32 * 256) {
+    const size_t shm = (size_t)32 * H * sizeof(bf16_t);
+    // (dynamic LDS has to be allowed per kernel and device; a host-side call without a launch)
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&router_norm_mfma_kernel<32>),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(router_norm_mfma_kernel<32>, dim3((T + 31) / 32), dim3(512), shm, s, hp, norm_weight, eps, wp, bias, T,
+                       H, E, k, norm_mode, xp, logits, idx, w, nullptr, chunk_hist);
+  } else {
+    const size_t shm = (size_t)16 * H * sizeof(bf16_t);
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&router_norm_mfma_kernel<16>),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(router_norm_mfma_kernel<16>, dim3((T + 15) / 16), dim3(256), shm, s, hp, norm_weight, eps, wp, bias, T,
+                       H, E, k, norm_mode, xp, logits, idx, w, nullptr, chunk_hist);
+  }
+  if (hist_tokens != nullptr && chunk_hist != nullptr) *hist_tokens = T >= 32 * 256 ? 32 : 16;
+  return hipGetLastError();
+}
 
 hipError_t launch_router(const void* x, const void* w_router, const float* bias, int T, int H, int E, int k, int dtype,
                          int norm_mode, float* logits, int32_t* idx, float* w, float* gap, int32_t* chunk_hist,
