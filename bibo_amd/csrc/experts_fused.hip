@@ -4,23 +4,28 @@
 // Phase 1 (gate/up GEMM, 2 x 4 waves, v_mfma_f32_32x32x16_bf16, operands swapped so that a lane ends up with
 // one ROW's values) walks K in steps of 64 elements, so every row an LDS-DMA instruction fetches is a whole
 // 128-byte line: the L2 -> LDS path moves almost twice the bytes per second for whole lines than for the
-// half lines of a 32-element step.  A step of all 2I weight rows would not fit LDS twice, so a step is cut
-// into a gate half and an up half: while the MFMAs multiply the I gate rows of step s from one buffer, the up
-// rows of step s arrive in the other, then the gate rows of step s+1 in the first, and so on; the x rows of
-// step s+1 arrive in two halves over the two sub-steps of step s.
-// Phase 2 turns the accumulators into bf16 activations and parks them in LDS as an operand of the second
-// GEMM: rows 0..63 live in B0, rows 64..127 in B1, whose contents are dead by then; row r keeps 16-byte
-// granule c at position c ^ (r & 15), which spreads the 16 lanes of a fragment read over all banks although
-// the row stride is a multiple of 256 bytes.
+// half lines of a 32-element step.  All 2I weight rows of a step would not fit LDS more than once, so a step
+// is cut into I/128 sub-steps of 256 rows: sub-step t holds, for each of the four N waves, its t-th 32-column
+// gate tile and the up tile of the same columns (16 MFMAs per wave).  The 32 KB stages form a ring (three
+// for I = 384, two otherwise): the rows of sub-step n + ring - 1 are requested while sub-step n is multiplied,
+// and a wave waits only until the loads older than the latest sub-step's have landed (loads complete in order),
+// so the L2 -> LDS path always has a stage or two in flight instead of draining at every barrier.  The x rows of
+// step s+1 arrive during step s in a double buffer of their own.
+// Phase 2 turns the accumulators into bf16 activations and parks them in the stages, whose contents are dead by
+// then, as an operand of the second GEMM: stage t holds columns [128t, 128t+128) of all 128 rows; row r keeps
+// 16-byte granule c at position c ^ (r & 15), which spreads the 16 lanes of a fragment read over all banks
+// although the row stride is 256 bytes.
 // Phase 3 has no barriers and no LDS traffic for the weights: the eight waves split a block of 128*CT
 // output columns (16*CT each), every wave multiplies ALL 128 resident rows with v_mfma_f32_16x16x32_bf16
 // and pulls its own w_down rows straight from global memory into registers, up to three 128-byte K
-// blocks ahead (lane (r, g) takes bytes [32g, 32g+32) of each line of weight row r; the activation fragments
-// are read with the same K permutation).  Keeping the in-flight bytes in registers instead of LDS is
-// what lets a CU cover the memory latency here: the activations already fill most of the LDS.
+// blocks ahead (the four lanes of a weight row fetch 64 contiguous bytes per instruction).  Keeping the
+// in-flight bytes in registers instead of LDS is what lets a CU cover the memory latency here: the
+// activations already fill most of the LDS.
 // Each block of columns is scaled by the routing weight, staged through LDS 32 rows at a time and
 // scattered to slot order as whole 16-byte row segments.
 // Reference: BiBoFusedExperts.forward, src/modeling/ffn/moe.py:81-93.
+#include <type_traits>
+
 #include "stripe.h"
 
 namespace bibo {
@@ -28,15 +33,18 @@ namespace {
 
 template <int NT, int CT>
 struct FusedShape {
-  static constexpr int MT = 2, WM = 2, BM = 128, BK = 64;
+  static constexpr int MT = 2, BM = 128, BK = 64;
   static constexpr int I = 128 * NT;
   static constexpr int BN2 = 128 * CT;                             // output columns per block: 8 waves x CT x 16
-  static constexpr int kHalfElems = 64 * I;                        // one weight half-stage = activations of one M half
+  static constexpr int kRing = NT == 3 ? 3 : 2;                    // weight stages in LDS
+  static constexpr int kDist = kRing - 1;                          // sub-steps between a stage's request and its use
+  static constexpr int kStageRows = 256;                           // 4 N waves x (gate tile + up tile) x 32 rows
+  static constexpr int kStageElems = kStageRows * BK;              // 32 KB = one [128][128] slice of the activations
   static constexpr int kAElems = BM * BK;                          // x rows of one K step
   static constexpr int kOutRows = 32;                              // rows of a column block staged at a time
   static constexpr int kOutElems = kOutRows * BN2;
-  static constexpr int kBInstr = I * (BK / 8) / 512;               // load instructions per thread and weight half-stage
-  static_assert(I * (BK / 8) % 512 == 0 && BM * (BK / 8) == 2 * 512, "stage does not divide over the threads");
+  static constexpr int kBInstr = kStageRows * (BK / 8) / 512;      // load instructions per thread and weight stage
+  static_assert(kBInstr == 4 && BM * (BK / 8) == 2 * 512, "stage does not divide over the threads");
 };
 
 // LDS-DMA through a buffer descriptor: the address is descriptor base + 32-bit per-thread byte offset (one
@@ -49,33 +57,47 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, un
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);   // raw buffer, 32-bit data format
 }
 
-// The load instructions one thread issues during one sub-step: the next weight half-stage and half of the
-// next step's x rows.  Shaped like StripeLoader so that stripe_step can spread them between its MFMAs.
+// Workgroup barrier that lets the N most recent LDS-DMA loads of every thread stay in flight: s_waitcnt vmcnt(N)
+// lgkmcnt(0) (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4 left at "no wait", lgkmcnt 11:8), then s_barrier.
+// __syncthreads() cannot be used for this: its release fence waits for every outstanding LDS-DMA transfer.  The
+// older loads have landed in every wave once all waves have passed, and every wave's LDS reads of the stage that is
+// refilled next have returned.
+template <int N>
+__device__ __forceinline__ void sync_keep_loads() {
+  __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | (0x7 << 4));
+  __builtin_amdgcn_s_barrier();
+}
+
+// What one thread needs to request a weight stage and the x rows of a K step.
 template <typename F>
 struct SubLoader {
   __amdgpu_buffer_rsrc_t w_rsrc, x_rsrc;   // this expert's w_gate_up block; the hidden states
-  unsigned b_voff;         // byte offset of this thread's row and granule inside the first instruction's 64 rows
-  unsigned b_soff;         // byte offset of the half-stage to fetch, K offset included (uniform)
+  unsigned b_voff;         // byte offset of this thread's row and granule inside an instruction's 64 rows
+  unsigned b_soff;         // byte offset of the stage's first tile row, K offset included (uniform)
   unsigned bstep;          // bytes between the rows of consecutive instructions (uniform)
-  bf16_t* b_dst;           // LDS half-stage
-  unsigned a_voff;         // byte offset of this thread's token row and granule
+  bf16_t* b_dst;           // LDS stage
+  unsigned a_voff[2];      // byte offsets of this thread's two token rows and granule
   unsigned a_soff;         // K offset in bytes (uniform)
-  bf16_t* a_dst;           // LDS position of that instruction's granules
-  static constexpr int kInstr = F::kBInstr + 1;
+  bf16_t* a_dst;           // LDS x stage
+};
+
+// The load instructions of one sub-step: the weight stage kDist sub-steps ahead and, in the first sub-step of a K
+// step (WITH_A), the next step's x rows.  Shaped like StripeLoader so that stripe_step can spread them between its
+// MFMAs.
+template <typename F, bool WITH_A>
+struct SubIssuer {
+  const SubLoader<F>& d;
+  static constexpr int kInstr = F::kBInstr + (WITH_A ? 2 : 0);
   template <int Q>
   __device__ __forceinline__ void issue(int, bf16_t*) const {
     const int wave = threadIdx.x >> 6;
-    if constexpr (Q < F::kBInstr) dma16_buf(w_rsrc, b_voff, b_soff + Q * bstep, b_dst + (Q * 512 + wave * 64) * 8);
-    else if constexpr (Q == F::kBInstr) dma16_buf(x_rsrc, a_voff, a_soff, a_dst + wave * 64 * 8);
+    if constexpr (Q < F::kBInstr) dma16_buf(d.w_rsrc, d.b_voff, d.b_soff + Q * d.bstep, d.b_dst + (Q * 512 + wave * 64) * 8);
+    else if constexpr (WITH_A && Q < F::kBInstr + 2)
+      dma16_buf(d.x_rsrc, d.a_voff[Q - F::kBInstr], d.a_soff, d.a_dst + ((Q - F::kBInstr) * 512 + wave * 64) * 8);
   }
 };
 
-// this lane's 32 bytes of one 128-byte K block for each of its CT weight tiles
-#ifdef BIBO_P3_OLD
-constexpr int W3_SECOND = 8, W3_LANE = 16;
-#else
 constexpr int W3_SECOND = 32, W3_LANE = 8;     // the four lanes of a row fetch 64 contiguous bytes per instruction
-#endif
 template <int CT>
 struct WBlock {
   bf16x8 w[CT][2];
@@ -102,10 +124,11 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
                                                             int act, unsigned x_bytes, bf16_t* __restrict__ yw) {
   using F = FusedShape<NT, CT>;
   constexpr int MT = F::MT, BM = F::BM, I = F::I, BK = F::BK;
-  __shared__ __attribute__((aligned(16))) bf16_t P[F::kHalfElems];    // weight half-stage 0, then activations of rows 0..63
-  __shared__ __attribute__((aligned(16))) bf16_t Q[F::kHalfElems];    // weight half-stage 1, then activations of rows 64..127
   // Every buffer that is read while LDS-DMA fills another is a variable of its own: the compiler orders a DMA
   // transfer against later LDS reads of the same variable with a full wait for the transfer.
+  __shared__ __attribute__((aligned(16))) bf16_t S0[F::kStageElems];  // weight stages, then the activations
+  __shared__ __attribute__((aligned(16))) bf16_t S1[F::kStageElems];
+  __shared__ __attribute__((aligned(16))) bf16_t S2[F::kRing == 3 ? F::kStageElems : 8];
   __shared__ __attribute__((aligned(16))) bf16_t A0[F::kAElems];      // x rows of even K steps
   __shared__ __attribute__((aligned(16))) bf16_t A1[F::kAElems];      // x rows of odd K steps
   __shared__ __attribute__((aligned(16))) bf16_t O[F::kOutElems];     // output staging
@@ -126,31 +149,54 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
   const int wn = wave & 3, wm = wave >> 2;
   const int n = lane & 31;
   const int mbase = wm * MT * 32;
+  auto stage = [&](auto ic) -> bf16_t* {
+    constexpr int i = decltype(ic)::value;
+    if constexpr (i == 0) return S0; else if constexpr (i == 1) return S1; else return S2;
+  };
 
   // ---- phase 1: gate/up projection (moe.py:81-86) ----
   floatx16 acc[MT][2 * NT];               // [..][0..NT) gate tiles, [..][NT..2NT) the up tiles of the same columns
   {
     // DMA side: thread t of an instruction fills granule t (row t/8, position t%8) of its 64 rows and fetches
-    // logical granule (t%8) ^ ((row >> 1) & 7) of that row: granule c of a stage row sits at c ^ ((row >> 1) & 7)
+    // logical granule (t%8) ^ ((row >> 1) & 7) of that row: granule c of a stage row sits at c ^ ((row >> 1) & 7).
+    // Stage row (wn*2 + gu)*32 + r of sub-step t is weight row gu*I + (wn*NT + t)*32 + r: instruction q = wn.
     const int chunk = (tid & 7) ^ ((tid >> 4) & 7);
     const int drow = tid >> 3;
+    const unsigned hb = (unsigned)H * sizeof(bf16_t);                            // bytes per weight / hidden-state row
+    const int nsteps = H / BK;
     SubLoader<F> ld;
-    ld.w_rsrc = make_rsrc(wgu + (size_t)e * 2 * I * H, 2u * I * H * sizeof(bf16_t));   // gate rows; the up rows are I further
+    ld.w_rsrc = make_rsrc(wgu + (size_t)e * 2 * I * H, 2u * I * hb);
     ld.x_rsrc = make_rsrc(x, x_bytes);
-    const unsigned up_off = (unsigned)I * H * sizeof(bf16_t);
-    ld.b_voff = ((unsigned)drow * H + chunk * 8) * sizeof(bf16_t);
-    ld.bstep = 64u * H * sizeof(bf16_t);
-    unsigned a_voff[2];
+    ld.b_voff = ((unsigned)((drow >> 5) * I + (drow & 31))) * hb + chunk * 16;
+    ld.bstep = (unsigned)NT * 32 * hb;
 #pragma unroll
     for (int a = 0; a < 2; ++a) {
       const int m = min(a * 64 + drow, rows - 1);                                // rows past the end re-read the last valid row
-      a_voff[a] = ((unsigned)perm_token[row0 + m] * H + chunk * 8) * sizeof(bf16_t);   // gather, moe.py:81
+      ld.a_voff[a] = (unsigned)perm_token[row0 + m] * hb + chunk * 16;          // gather, moe.py:81
     }
-    // prologue: gate half-stage and x rows of step 0 (weight rows first: they do not wait for the row indices)
+    // what sub-step (s, t) requests: the weight rows of sub-step (s, t) + kDist (its K step clamped to the last
+    // one: requests past the end fetch valid rows into a stage nobody reads again), and at t = 0 the x rows of
+    // step s + 1.  Every sub-step issues the same number of loads, so the wait counts below are constants.
+    auto request = [&](auto tc, auto pc, int s) {
+      constexpr int t = decltype(tc)::value, par = decltype(pc)::value;
+      constexpr int tn = (t + F::kDist) % NT, ds = (t + F::kDist) / NT;
+      constexpr int target = NT == 1 ? (par + ds) % 2 : tn;
+      ld.b_soff = (unsigned)tn * 32 * hb + (unsigned)min(s + ds, nsteps - 1) * (unsigned)(BK * sizeof(bf16_t));
+      ld.b_dst = stage(std::integral_constant<int, target>{});
+      ld.a_soff = (unsigned)min(s + 1, nsteps - 1) * (unsigned)(BK * sizeof(bf16_t));
+      ld.a_dst = par ? A0 : A1;
+    };
+    // prologue: the first kDist sub-steps' weight rows and the x rows of step 0 (weight rows first: they do not wait
+    // for the row indices)
 #pragma unroll
-    for (int q = 0; q < F::kBInstr; ++q) dma16_buf(ld.w_rsrc, ld.b_voff, q * ld.bstep, P + (q * 512 + wave * 64) * 8);
-    dma16_buf(ld.x_rsrc, a_voff[0], 0, A0 + (wave * 64) * 8);
-    dma16_buf(ld.x_rsrc, a_voff[1], 0, A0 + (512 + wave * 64) * 8);
+    for (int q = 0; q < F::kBInstr; ++q) dma16_buf(ld.w_rsrc, ld.b_voff, q * ld.bstep, S0 + (q * 512 + wave * 64) * 8);
+    dma16_buf(ld.x_rsrc, ld.a_voff[0], 0, A0 + (wave * 64) * 8);
+    dma16_buf(ld.x_rsrc, ld.a_voff[1], 0, A0 + (512 + wave * 64) * 8);
+    if constexpr (F::kDist == 2) {
+#pragma unroll
+      for (int q = 0; q < F::kBInstr; ++q)
+        dma16_buf(ld.w_rsrc, ld.b_voff, 32 * hb + q * ld.bstep, S1 + (q * 512 + wave * 64) * 8);   // sub-step (0, 1)
+    }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -159,29 +205,31 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
         for (int i = 0; i < 16; ++i) acc[mt][j][i] = 0.f;
     // fragment side: lane (n, h) reads logical granule 2*ss + h of rows congruent to n mod 32
     const int pos0 = ((lane >> 5) ^ ((n >> 1) & 7)) * 8;
-    auto frag_row = [&](int j) { return (wn * NT + j) * 32; };
-    // one K step: x rows in `Acur`, the next step's go to `Anext`
-    auto step = [&](const bf16_t* Acur, bf16_t* Anext, int k0, bool last) {
-      const unsigned kb = (unsigned)k0 * sizeof(bf16_t);
-      const unsigned kn = last ? kb : kb + BK * sizeof(bf16_t);                  // (the last step fetches its own x rows again: unused)
-      const bf16_t* a0 = Acur + (mbase + n) * BK + pos0;
-      // gate sub-step: multiplies P; the up rows of this step arrive in Q, rows 0..63 of the next x stage in Anext
-      wait_loads_and_sync();
-      ld.b_soff = up_off + kb; ld.b_dst = Q;
-      ld.a_soff = kn; ld.a_voff = a_voff[0]; ld.a_dst = Anext;
-      stripe_step<MT, NT, BK, true, 2 * NT, 0>(acc, a0, 32 * BK, P + n * BK, pos0, frag_row, ld, true, 0, nullptr);
-      // up sub-step: multiplies Q; the gate rows of the next step arrive in P, rows 64..127 of the next x stage
-      wait_loads_and_sync();
-      ld.b_soff = kn; ld.b_dst = P;
-      ld.a_voff = a_voff[1]; ld.a_dst = Anext + 512 * 8;
-      stripe_step<MT, NT, BK, true, 2 * NT, NT>(acc, a0, 32 * BK, Q + n * BK, pos0, frag_row, ld, !last, 0, nullptr);
+    auto frag_row = [&](int j) { return (wn * 2 + j) * 32; };
+    auto substep = [&](auto tc, auto pc, int s) {
+      constexpr int t = decltype(tc)::value, par = decltype(pc)::value;
+      constexpr int cur = NT == 1 ? par : t;
+      // loads still allowed in flight: those of the sub-steps after the one whose stage is read now
+      if constexpr (F::kDist == 1) sync_keep_loads<0>();
+      else if constexpr (t == 1) sync_keep_loads<F::kBInstr + 2>();     // the sub-step before (t = 0) also requested x rows
+      else sync_keep_loads<F::kBInstr>();
+      const bf16_t* a0 = (par ? A1 : A0) + (mbase + n) * BK + pos0;
+      const bf16_t* b0 = stage(std::integral_constant<int, cur>{}) + n * BK;
+      request(tc, pc, s);
+      const SubIssuer<F, t == 0> issuer{ld};
+      stripe_step<MT, 2, BK, true, 2 * NT, t, NT>(acc, a0, 32 * BK, b0, pos0, frag_row, issuer, true, 0, nullptr);
     };
-    for (int k0 = 0; k0 < H; k0 += 2 * BK) {                                     // H / BK is even
-      step(A0, A1, k0, false);
-      step(A1, A0, k0 + BK, k0 + 2 * BK >= H);
+    using std::integral_constant;
+    for (int s = 0; s < nsteps; s += 2) {                                         // H / BK is even
+      substep(integral_constant<int, 0>{}, integral_constant<int, 0>{}, s);
+      if constexpr (NT > 1) substep(integral_constant<int, 1>{}, integral_constant<int, 0>{}, s);
+      if constexpr (NT > 2) substep(integral_constant<int, 2>{}, integral_constant<int, 0>{}, s);
+      substep(integral_constant<int, 0>{}, integral_constant<int, 1>{}, s + 1);
+      if constexpr (NT > 1) substep(integral_constant<int, 1>{}, integral_constant<int, 1>{}, s + 1);
+      if constexpr (NT > 2) substep(integral_constant<int, 2>{}, integral_constant<int, 1>{}, s + 1);
     }
   }
-  __syncthreads();                         // every wave is done with the gate/up stages
+  wait_loads_and_sync();                   // every transfer has landed and every wave is done with the stages
 
   // ---- phase 2: Radial NormSiLU (moe.py:87-92), activations to LDS ----
   // The accumulators are transposed (lane = row mbase + 32*mt + n, register i = column acc_row(i, lane) of
@@ -210,17 +258,18 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
   }
   __syncthreads();
   {
-    bf16_t* hsel = wm ? Q : P;             // activations of this wave's M half, [64][I], granules swizzled
+    // stage t holds activation columns [128t, 128t + 128) of all 128 rows, [128][128], granules swizzled
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-      const int ml = mt * 32 + n;
-      const float rinv = rinv_s[mbase + ml];
-      const float nrl = -1.44269504f * rinv, rg = rinv * gain_s[mbase + ml];   // per-row constants folded once
-      bf16_t* hrow = hsel + ml * I + 4 * hh;
+      const int m = mbase + mt * 32 + n;
+      const float rinv = rinv_s[m];
+      const float nrl = -1.44269504f * rinv, rg = rinv * gain_s[m];            // per-row constants folded once
 #pragma unroll
-      for (int j = 0; j < NT; ++j)
+      for (int j = 0; j < NT; ++j) {
+        const int tile32 = wn * NT + j;      // 32-column tile of the activation row: slice tile32 / 4, granules (tile32 % 4) * 4 + q
+        bf16_t* hrow = ((tile32 >> 2) == 0 ? S0 : ((tile32 >> 2) == 1 ? S1 : S2)) + m * 128 + 4 * hh;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {        // columns (wn*NT + j)*32 + 8*q + 4*hh + 0..3: half of granule (wn*NT + j)*4 + q
+        for (int q = 0; q < 4; ++q) {        // columns tile32*32 + 8*q + 4*hh + 0..3: half of a granule
           bf16x4 hv;
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
@@ -228,9 +277,10 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
             const float sg = __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(g * nrl));   // sigmoid(g/r)
             hv[r] = (bf16_t)(g * rg * sg * acc[mt][NT + j][4 * q + r]);                // SiLU(g/r) r^p up
           }
-          const int c = (wn * NT + j) * 4 + q;
-          *reinterpret_cast<bf16x4*>(hrow + (c ^ (ml & 15)) * 8) = hv;
+          const int c = (tile32 & 3) * 4 + q;
+          *reinterpret_cast<bf16x4*>(hrow + (c ^ (m & 15)) * 8) = hv;
         }
+      }
     }
   }
   __syncthreads();                         // the activation tile is complete
@@ -240,7 +290,6 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
   constexpr int G = F::BN2 / 8;              // 16-byte granules per staged output row
   const int r16 = lane & 15, g4 = lane >> 4;
   const size_t tile_stride = (size_t)16 * I;
-  // activation fragment of row tile rt, K block kb, half s: granule (8*kb + 2*g4 + s) ^ r16 of row 16*rt + r16
   const int nblk = H / F::BN2;
   const bf16_t* wp = wd + ((size_t)e * H + wave * (16 * CT) + r16) * I + g4 * W3_LANE;
   constexpr int D = KB > 3 ? 3 : KB - 1;      // K blocks requested ahead of the one being multiplied
@@ -258,12 +307,10 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
     // Activation fragments are read a row tile ahead of the MFMAs that consume them (across K block
     // boundaries too).
     auto frag = [&](int kb, int rt, int s) {
-#ifdef BIBO_P3_OLD
-      const int gq = (((kb * 8 + 2 * g4) ^ r16) * 8) ^ (s * 8);
-#else
-      const int gq = (((kb * 8 + g4) ^ r16) * 8) ^ (s * 32);      // K elements 64 kb + 32 s + 8 g4 .. + 8 of the row
-#endif
-      return *reinterpret_cast<const bf16x8*>((rt < 4 ? P : Q) + ((rt & 3) * 16 + r16) * I + gq);
+      // K elements 64 kb + 32 s + 8 g4 .. + 8 of row 16 rt + r16: slice kb / 2, granule (kb % 2) * 8 + 4 s + g4
+      const int gq = ((((kb & 1) * 8 + g4) ^ r16) * 8) ^ (s * 32);
+      const bf16_t* slice = (kb >> 1) == 0 ? S0 : ((kb >> 1) == 1 ? S1 : S2);
+      return *reinterpret_cast<const bf16x8*>(slice + (rt * 16 + r16) * 128 + gq);
     };
     constexpr int AD = 1;                    // row tiles whose fragments are requested ahead (2 and 3 measured the same)
     bf16x8 xa[AD + 1][2];

@@ -139,7 +139,7 @@ __device__ __forceinline__ void issue_some(const Loader& ld, int k_next, bf16_t*
 // (if there is one): spreading the loads through the MFMAs keeps the waves from queueing up at the
 // texture-address unit before they start multiplying.  `a1` points at this lane's A fragment of the
 // second sub-step for M tile 0; tile mt is `astride` elements further.
-template <int Q, int MT, int NTW, int BK, bool TR, int NACC, int J0, typename Loader, typename FragRow>
+template <int Q, int MT, int NTW, int BK, bool TR, int NACC, int J0, int JS, typename Loader, typename FragRow>
 __device__ __forceinline__ void stripe_pair(floatx16 (&acc)[MT][NACC], bf16x8 (&a)[2][MT], bf16x8 (&b)[3],
                                             const bf16_t* a0, int astride, const bf16_t* bstage, int pos0,
                                             FragRow frag_row, const Loader& ld, bool prefetch, int k_next,
@@ -163,19 +163,19 @@ __device__ __forceinline__ void stripe_pair(floatx16 (&acc)[MT][NACC], bf16x8 (&
     a[(s + 1) & 1][mt] = *reinterpret_cast<const bf16x8*>(a0 + mt * astride + ((pos0 ^ ((s + 1) * 16)) - pos0));
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
-    acc[mt][J0 + j] = TR ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[Q % 3], a[s & 1][mt], acc[mt][J0 + j], 0, 0, 0)
-                         : __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[s & 1][mt], b[Q % 3], acc[mt][J0 + j], 0, 0, 0);
+    acc[mt][J0 + j * JS] = TR ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[Q % 3], a[s & 1][mt], acc[mt][J0 + j * JS], 0, 0, 0)
+                              : __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[s & 1][mt], b[Q % 3], acc[mt][J0 + j * JS], 0, 0, 0);
   constexpr int kReads = (Q + 2 < kPairs ? 1 : 0) + (kALast >= kAFirst ? kALast - kAFirst + 1 : 0);
   if constexpr (kReads > 0) __builtin_amdgcn_sched_group_barrier(0x100, kReads, 0);
   __builtin_amdgcn_sched_group_barrier(0x008, MT, 0);
 }
 
-template <int MT, int NTW, int BK, bool TR, int NACC, int J0, typename Loader, typename FragRow, int... Qs>
+template <int MT, int NTW, int BK, bool TR, int NACC, int J0, int JS, typename Loader, typename FragRow, int... Qs>
 __device__ __forceinline__ void stripe_pairs(floatx16 (&acc)[MT][NACC], bf16x8 (&a)[2][MT], bf16x8 (&b)[3],
                                              const bf16_t* a0, int astride, const bf16_t* bstage, int pos0,
                                              FragRow frag_row, const Loader& ld, bool prefetch, int k_next,
                                              bf16_t* next_stage, std::integer_sequence<int, Qs...>) {
-  (stripe_pair<Qs, MT, NTW, BK, TR, NACC, J0>(acc, a, b, a0, astride, bstage, pos0, frag_row, ld, prefetch, k_next, next_stage), ...);
+  (stripe_pair<Qs, MT, NTW, BK, TR, NACC, J0, JS>(acc, a, b, a0, astride, bstage, pos0, frag_row, ld, prefetch, k_next, next_stage), ...);
 }
 
 // Multiply one K step of BK into the accumulators while the load instructions of the next stage are
@@ -184,8 +184,8 @@ __device__ __forceinline__ void stripe_pairs(floatx16 (&acc)[MT][NACC], bf16x8 (
 // of the next sub-step are read while the current one is still multiplying.  a0: this lane's A
 // fragment of sub-step 0 for M tile 0 (position pos0 of its row; sub-step s sits at pos0 ^ 16s, M tile
 // mt `astride` elements further); bstage: this lane's row of the B stage (N tile 0).  The NTW tiles multiplied
-// here are columns J0 .. J0+NTW-1 of an accumulator array NACC tiles wide.
-template <int MT, int NTW, int BK, bool TR, int NACC = NTW, int J0 = 0, typename Loader, typename FragRow>
+// here are columns J0, J0+JS, .. of an accumulator array NACC tiles wide.
+template <int MT, int NTW, int BK, bool TR, int NACC = NTW, int J0 = 0, int JS = 1, typename Loader, typename FragRow>
 __device__ __forceinline__ void stripe_step(floatx16 (&acc)[MT][NACC], const bf16_t* a0, int astride, const bf16_t* bstage,
                                             int pos0, FragRow frag_row, const Loader& ld, bool prefetch, int k_next,
                                             bf16_t* next_stage) {
@@ -196,7 +196,7 @@ __device__ __forceinline__ void stripe_step(floatx16 (&acc)[MT][NACC], const bf1
   b[0] = *reinterpret_cast<const bf16x8*>(bstage + frag_row(0) * BK + pos0);
   b[1] = *reinterpret_cast<const bf16x8*>(bstage + frag_row(NTW > 1 ? 1 : 0) * BK + (NTW > 1 ? pos0 : (pos0 ^ 16)));
   __builtin_amdgcn_sched_group_barrier(0x100, MT + 2, 0);
-  stripe_pairs<MT, NTW, BK, TR, NACC, J0>(acc, a, b, a0, astride, bstage, pos0, frag_row, ld, prefetch, k_next, next_stage,
+  stripe_pairs<MT, NTW, BK, TR, NACC, J0, JS>(acc, a, b, a0, astride, bstage, pos0, frag_row, ld, prefetch, k_next, next_stage,
                                           std::make_integer_sequence<int, SS * NTW>{});
 }
 
