@@ -21,8 +21,8 @@
 // blocks ahead (the four lanes of a weight row fetch 64 contiguous bytes per instruction).  Keeping the
 // in-flight bytes in registers instead of LDS is what lets a CU cover the memory latency here: the
 // activations already fill most of the LDS.
-// Each block of columns is scaled by the routing weight, staged through LDS 32 rows at a time and
-// scattered to slot order as whole 16-byte row segments.
+// Each block of columns is scaled by the routing weight, staged through LDS 32 rows at a time (in the two x
+// buffers, which are idle by then) and scattered to slot order as 256-byte row segments.
 // Reference: BiBoFusedExperts.forward, src/modeling/ffn/moe.py:81-93.
 #include <type_traits>
 
@@ -43,6 +43,7 @@ struct FusedShape {
   static constexpr int kAElems = BM * BK;                          // x rows of one K step
   static constexpr int kOutRows = 32;                              // rows of a column block staged at a time
   static constexpr int kOutElems = kOutRows * BN2;
+  static constexpr int kXElems = kAElems > kOutElems ? kAElems : kOutElems;   // a buffer that serves as either
   static constexpr int kBInstr = kStageRows * (BK / 8) / 512;      // load instructions per thread and weight stage
   static_assert(kBInstr == 4 && BM * (BK / 8) == 2 * 512, "stage does not divide over the threads");
 };
@@ -97,7 +98,10 @@ struct SubIssuer {
   }
 };
 
-constexpr int W3_SECOND = 32, W3_LANE = 8;     // the four lanes of a row fetch 64 contiguous bytes per instruction
+// One 128-byte K block of a wave's 16*CT w_down rows as it comes from memory: lane l holds 16-byte piece l % 4 of
+// the first (s = 0) or second (s = 1) 64 bytes of row l / 4 of column tile ct.  The four lanes of a row are
+// ADJACENT, so the texture unit merges them into one 64-byte request; lanes that are 16 apart, as in the MFMA
+// operand layout, are not merged and move less than half the bytes per second.
 template <int CT>
 struct WBlock {
   bf16x8 w[CT][2];
@@ -109,8 +113,18 @@ __device__ __forceinline__ void load_wblock(WBlock<CT>& b, const bf16_t* __restr
   for (int ct = 0; ct < CT; ++ct) {
     const bf16_t* p = wp + ct * tile_stride + kb * 64;
     b.w[ct][0] = *reinterpret_cast<const bf16x8*>(p);
-    b.w[ct][1] = *reinterpret_cast<const bf16x8*>(p + W3_SECOND);
+    b.w[ct][1] = *reinterpret_cast<const bf16x8*>(p + 32);
   }
+}
+
+// Memory order -> MFMA operand order: lane r + 16 g takes the register of lane 4 r + g (row r, piece g).  sel is
+// 4 * (source lane); the exchange uses the LDS crossbar and no LDS memory.
+__device__ __forceinline__ bf16x8 to_operand_lanes(bf16x8 v, int sel) {
+  typedef int i32x4 __attribute__((ext_vector_type(4)));
+  i32x4 u = __builtin_bit_cast(i32x4, v);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) u[i] = __builtin_amdgcn_ds_bpermute(sel, u[i]);
+  return __builtin_bit_cast(bf16x8, u);
 }
 
 template <int NT, int CT>
@@ -129,9 +143,8 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
   __shared__ __attribute__((aligned(16))) bf16_t S0[F::kStageElems];  // weight stages, then the activations
   __shared__ __attribute__((aligned(16))) bf16_t S1[F::kStageElems];
   __shared__ __attribute__((aligned(16))) bf16_t S2[F::kRing == 3 ? F::kStageElems : 8];
-  __shared__ __attribute__((aligned(16))) bf16_t A0[F::kAElems];      // x rows of even K steps
-  __shared__ __attribute__((aligned(16))) bf16_t A1[F::kAElems];      // x rows of odd K steps
-  __shared__ __attribute__((aligned(16))) bf16_t O[F::kOutElems];     // output staging
+  __shared__ __attribute__((aligned(16))) bf16_t A0[F::kXElems];      // x rows of even K steps; then output staging,
+  __shared__ __attribute__((aligned(16))) bf16_t A1[F::kXElems];      // x rows of odd K steps;  alternating per 32 rows
   __shared__ float ssq[4 * BM];
   __shared__ float rinv_s[BM], gain_s[BM], w_s[BM];
   __shared__ int slot_s[BM];
@@ -287,11 +300,11 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
 
   // ---- phase 3: down projection, routing weight, scatter to slot order (moe.py:92-93) ----
   constexpr int KB = I / 64;                 // 128-byte K blocks
-  constexpr int G = F::BN2 / 8;              // 16-byte granules per staged output row
   const int r16 = lane & 15, g4 = lane >> 4;
   const size_t tile_stride = (size_t)16 * I;
   const int nblk = H / F::BN2;
-  const bf16_t* wp = wd + ((size_t)e * H + wave * (16 * CT) + r16) * I + g4 * W3_LANE;
+  const bf16_t* wp = wd + ((size_t)e * H + wave * (16 * CT) + (lane >> 2)) * I + (lane & 3) * 8;
+  const int sel = 4 * (4 * r16 + g4);
   constexpr int D = KB > 3 ? 3 : KB - 1;      // K blocks requested ahead of the one being multiplied
   constexpr int NB = D + 1;
   WBlock<CT> wb[NB];
@@ -312,31 +325,28 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
       const bf16_t* slice = (kb >> 1) == 0 ? S0 : ((kb >> 1) == 1 ? S1 : S2);
       return *reinterpret_cast<const bf16x8*>(slice + (rt * 16 + r16) * 128 + gq);
     };
-    constexpr int AD = 1;                    // row tiles whose fragments are requested ahead (2 and 3 measured the same)
-    bf16x8 xa[AD + 1][2];
+    // The multiply walks half K blocks (32 elements, one MFMA deep): while half hs is multiplied with all eight
+    // row tiles, the weights of half hs + 1 change lanes and the activation fragment of the next row tile is read.
+    bf16x8 wc[2][CT], xa[2];
 #pragma unroll
-    for (int g = 0; g < AD; ++g) {
-      xa[g][0] = frag(g / 8, g % 8, 0);
-      xa[g][1] = frag(g / 8, g % 8, 1);
-    }
+    for (int ct = 0; ct < CT; ++ct) wc[0][ct] = to_operand_lanes(wb[0].w[ct][0], sel);
+    xa[0] = frag(0, 0, 0);
 #pragma unroll
     for (int kb = 0; kb < KB; ++kb) {
       if (kb + D < KB) load_wblock<CT>(wb[(kb + D) % NB], wp, tile_stride, kb + D);
       __builtin_amdgcn_sched_barrier(0);     // keep the loads D blocks ahead of their use
 #pragma unroll
-      for (int rt = 0; rt < 8; ++rt) {
-        const int g = kb * 8 + rt;             // running (K block, row tile) index; fragments rotate through AD + 1 buffers
-        if (g + AD < KB * 8) {
-          xa[(g + AD) % (AD + 1)][0] = frag((g + AD) / 8, (g + AD) % 8, 0);
-          xa[(g + AD) % (AD + 1)][1] = frag((g + AD) / 8, (g + AD) % 8, 1);
-        }
+      for (int s = 0; s < 2; ++s) {
+        const int hs = 2 * kb + s;
 #pragma unroll
-        for (int s = 0; s < 2; ++s)
+        for (int rt = 0; rt < 8; ++rt) {
+          const int g = hs * 8 + rt;           // running (half K block, row tile) index
+          if (g + 1 < KB * 16) xa[(g + 1) & 1] = frag((g + 1) >> 4, (g + 1) & 7, ((g + 1) >> 3) & 1);
+          if (rt < CT && hs + 1 < 2 * KB) wc[(hs + 1) & 1][rt] = to_operand_lanes(wb[((hs + 1) >> 1) % NB].w[rt][(hs + 1) & 1], sel);
 #pragma unroll
           for (int ct = 0; ct < CT; ++ct)
-            acc2[ct][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb[kb % NB].w[ct][s], xa[g % (AD + 1)][s], acc2[ct][rt], 0, 0, 0);
-        if (g + AD < KB * 8) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, 2 * CT, 0);
+            acc2[ct][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[hs & 1][ct], xa[g & 1], acc2[ct][rt], 0, 0, 0);
+        }
       }
     }
     wp += (size_t)F::BN2 * I;                                  // next block of columns: in flight during the epilogue
@@ -345,16 +355,18 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
       for (int d = 0; d < D; ++d) load_wblock<CT>(wb[d], wp, tile_stride, d);
     }
     __builtin_amdgcn_sched_barrier(0);
-    // accumulator: lane holds row 16*rt + r16, columns wave*16*CT + 16*ct + 4*g4 + i.  Staged row r keeps
-    // granule c at position c ^ (r & 15): the 8-byte writes of a half wave then cover all banks.
+    // accumulator: lane holds row 16*rt + r16, columns wave*16*CT + 16*ct + 4*g4 + i.  The block leaves 32 rows at
+    // a time through the two x buffers in turn; between two barriers a wave stages the next 32 rows into one
+    // buffer and copies the previous 32 out of the other.  Staged row r keeps granule c at position c ^ (r & 15): the 8-byte writes of a half wave
+    // then cover all banks.  Copy-out: 16 consecutive threads move 256 contiguous bytes of one row.
     // (The thread index goes through an empty asm so the staging addresses are formed here, per block,
     // instead of being hoisted out of the loop and kept alive across the multiply.)
     int tid_o = tid;
     asm volatile("" : "+v"(tid_o));
     const int r16o = tid_o & 15, g4o = (tid_o >> 4) & 3;
-#pragma unroll
-    for (int hf = 0; hf < BM / F::kOutRows; ++hf) {
-      __syncthreads();                       // the previous copy-out is done with O
+    const int ro = tid_o >> 4, pco = tid_o & 15;             // copy-out: staged row, first granule position
+    auto stage_rows = [&](int hf) {          // rows 32 hf .. + 32 of the block into buffer hf % 2
+      bf16_t* const O = (hf & 1) ? A1 : A0;
 #pragma unroll
       for (int rq = 0; rq < F::kOutRows / 16; ++rq) {
         const int rt = hf * (F::kOutRows / 16) + rq;
@@ -369,16 +381,27 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
           *reinterpret_cast<bf16x4*>(orow + (c ^ r16o) * 8) = v;
         }
       }
-      __syncthreads();
+    };
+    auto copy_out = [&](int hf) {
+      const bf16_t* const O = (hf & 1) ? A1 : A0;
+      const int m = hf * F::kOutRows + ro;
+      if (m < rows) {
+        bf16_t* dst = yw + (size_t)slot_s[m] * H + n0;
+        const bf16_t* src = O + ro * F::BN2;
 #pragma unroll
-      for (int q = 0; q < F::kOutRows * G / 512; ++q) {
-        const int idx = q * 512 + tid_o;
-        const int r = idx / G, pc = idx - r * G;
-        const int m = hf * F::kOutRows + r;
-        if (m < rows)
-          *reinterpret_cast<u32x4*>(yw + (size_t)slot_s[m] * H + n0 + (pc ^ (r & 15)) * 8) =
-              *reinterpret_cast<const u32x4*>(O + r * F::BN2 + pc * 8);
+        for (int q = 0; q < CT; ++q) {                         // 16 CT granules per row, 16 threads per row
+          const int pc = pco + 16 * q;
+          *reinterpret_cast<u32x4*>(dst + (pc ^ (ro & 15)) * 8) = *reinterpret_cast<const u32x4*>(src + pc * 8);
+        }
       }
+    };
+    constexpr int NR = BM / F::kOutRows;
+    stage_rows(0);
+#pragma unroll
+    for (int hf = 0; hf < NR; ++hf) {
+      __syncthreads();                       // rows of round hf are staged; round hf - 1 has left its buffer
+      if (hf + 1 < NR) stage_rows(hf + 1);
+      copy_out(hf);
     }
   }
 }
