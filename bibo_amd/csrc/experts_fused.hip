@@ -80,6 +80,8 @@ struct SubLoader {
   unsigned a_voff[2];      // byte offsets of this thread's two token rows and granule
   unsigned a_soff;         // K offset in bytes (uniform)
   bf16_t* a_dst;           // LDS x stage
+  int wave_elems;          // this wave's place in an instruction's LDS block, in elements (uniform: a scalar register,
+                           // so that the LDS base of every transfer is formed by scalar instructions alone)
 };
 
 // The load instructions of one sub-step: the weight stage kDist sub-steps ahead and, in the first sub-step of a K
@@ -91,10 +93,9 @@ struct SubIssuer {
   static constexpr int kInstr = F::kBInstr + (WITH_A ? 2 : 0);
   template <int Q>
   __device__ __forceinline__ void issue(int, bf16_t*) const {
-    const int wave = threadIdx.x >> 6;
-    if constexpr (Q < F::kBInstr) dma16_buf(d.w_rsrc, d.b_voff, d.b_soff + Q * d.bstep, d.b_dst + (Q * 512 + wave * 64) * 8);
+    if constexpr (Q < F::kBInstr) dma16_buf(d.w_rsrc, d.b_voff, d.b_soff + Q * d.bstep, d.b_dst + Q * 512 * 8 + d.wave_elems);
     else if constexpr (WITH_A && Q < F::kBInstr + 2)
-      dma16_buf(d.x_rsrc, d.a_voff[Q - F::kBInstr], d.a_soff, d.a_dst + ((Q - F::kBInstr) * 512 + wave * 64) * 8);
+      dma16_buf(d.x_rsrc, d.a_voff[Q - F::kBInstr], d.a_soff, d.a_dst + (Q - F::kBInstr) * 512 * 8 + d.wave_elems);
   }
 };
 
@@ -182,6 +183,7 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
     ld.x_rsrc = make_rsrc(x, x_bytes);
     ld.b_voff = ((unsigned)((drow >> 5) * I + (drow & 31))) * hb + chunk * 16;
     ld.bstep = (unsigned)NT * 32 * hb;
+    ld.wave_elems = __builtin_amdgcn_readfirstlane(wave) * 64 * 8;
 #pragma unroll
     for (int a = 0; a < 2; ++a) {
       const int m = min(a * 64 + drow, rows - 1);                                // rows past the end re-read the last valid row
@@ -202,13 +204,13 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
     // prologue: the first kDist sub-steps' weight rows and the x rows of step 0 (weight rows first: they do not wait
     // for the row indices)
 #pragma unroll
-    for (int q = 0; q < F::kBInstr; ++q) dma16_buf(ld.w_rsrc, ld.b_voff, q * ld.bstep, S0 + (q * 512 + wave * 64) * 8);
-    dma16_buf(ld.x_rsrc, ld.a_voff[0], 0, A0 + (wave * 64) * 8);
-    dma16_buf(ld.x_rsrc, ld.a_voff[1], 0, A0 + (512 + wave * 64) * 8);
+    for (int q = 0; q < F::kBInstr; ++q) dma16_buf(ld.w_rsrc, ld.b_voff, q * ld.bstep, S0 + q * 512 * 8 + ld.wave_elems);
+    dma16_buf(ld.x_rsrc, ld.a_voff[0], 0, A0 + ld.wave_elems);
+    dma16_buf(ld.x_rsrc, ld.a_voff[1], 0, A0 + 512 * 8 + ld.wave_elems);
     if constexpr (F::kDist == 2) {
 #pragma unroll
       for (int q = 0; q < F::kBInstr; ++q)
-        dma16_buf(ld.w_rsrc, ld.b_voff, 32 * hb + q * ld.bstep, S1 + (q * 512 + wave * 64) * 8);   // sub-step (0, 1)
+        dma16_buf(ld.w_rsrc, ld.b_voff, 32 * hb + q * ld.bstep, S1 + q * 512 * 8 + ld.wave_elems);   // sub-step (0, 1)
     }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
