@@ -211,6 +211,39 @@ def moe_forward(x, w_router, bias, w_gate_up, w_down, theta, k, dtype=torch.floa
     return out, idx, w
 
 
+# --------------------------------------------------------------------------------------
+# backward pass: what torch.autograd computes for the reference's eager layer
+# --------------------------------------------------------------------------------------
+def route_weights(logits: torch.Tensor, idx, norm="sum") -> torch.Tensor:
+    """Combine weights as a differentiable function of the logits for a FIXED selection `idx` [T,k]
+    (router.py:31,41-47): the selection itself (router.py:38-39, with the bias) has no gradient."""
+    idx_t = torch.as_tensor(np.asarray(idx), dtype=torch.int64)
+    raw = torch.sigmoid(logits).gather(-1, idx_t)                             # router.py:31,41
+    if idx_t.shape[1] > 1 and norm == "softmax":
+        return F.softmax(raw, dim=-1)                                         # router.py:42-43
+    if idx_t.shape[1] > 1 and norm:
+        return raw / (raw.sum(-1, keepdim=True) + SUM_NORM_EPS)               # router.py:44-45
+    return raw                                                                # router.py:46-47
+
+
+def moe_backward(x, w_router, w_gate_up, w_down, theta, idx, d_out, norm="sum", act="radial", dtype=torch.float64,
+                 n_pos=0, n_neg=0):
+    """Gradients of sum(out * d_out) for out = BiBoMoELayer.forward(x) (moe.py:157-183, no shared expert) with the
+    selection `idx` held fixed, as torch.autograd derives them from the restated forward evaluated in `dtype`:
+    through the combine weights into the router weight (router.py:25-47), through each expert's down projection,
+    Radial NormSiLU (theta included) and gate/up projection (moe.py:81-93).  The balancing bias gets none: it only
+    enters the selection (router.py:38).  Returns a dict: x [T,H], w_router [E,H], w_gate_up, w_down, theta, and
+    `w` [T,k], the gradient with respect to the combine weights."""
+    leaf = lambda t: t.detach().to(dtype).clone().requires_grad_(True)
+    xl, wr, gu, dn, th = leaf(x), leaf(w_router), leaf(w_gate_up), leaf(w_down), leaf(theta)
+    logits = xl @ wr.t()                                                      # router.py:25-26
+    w = route_weights(logits, idx, norm)
+    w.retain_grad()
+    out = experts_forward(xl, idx, w, gu, dn, th, dtype=dtype, n_pos=n_pos, n_neg=n_neg, act=act)
+    (out * d_out.to(dtype)).sum().backward()
+    return {"x": xl.grad, "w_router": wr.grad, "w_gate_up": gu.grad, "w_down": dn.grad, "theta": th.grad, "w": w.grad}
+
+
 def shared_mlp(x, w_gate, w_up, w_down):
     """The shared expert, BiBoMLP.forward (src/modeling/ffn/mlp.py:34-35) with hidden_act = silu:
     down(silu(gate(x)) * up(x)); added to the routed output by the layer (moe.py:174-176).  fp32."""

@@ -346,3 +346,99 @@ def test_shared_mlp_is_a_swiglu():
     a = x.double() @ wg.double().t()
     want = ((a / (1 + torch.exp(-a))) * (x.double() @ wu.double().t())) @ wd.double().t()
     assert torch.allclose(got.double(), want, rtol=1e-4, atol=1e-4)
+
+
+# --------------------------------------------------------------------------------------
+# backward pass of the oracle: pinned by central differences and by hand-derived closed forms
+# --------------------------------------------------------------------------------------
+def _bwd_case(seed=11, T=24, H=32, E=6, k=3, I=16, act="radial", norm="sum"):
+    p = O.make_inputs(T=T, H=H, E=E, k=k, I=I, bias="uniform", theta="normal", seed=seed, dtype=torch.float64)
+    g = torch.Generator().manual_seed(seed + 1)
+    p["x"] = torch.randn(T, H, generator=g, dtype=torch.float64)
+    p["w_gate_up"] = torch.randn(E, 2 * I, H, generator=g, dtype=torch.float64) * 0.3
+    p["w_down"] = torch.randn(E, H, I, generator=g, dtype=torch.float64) * 0.3
+    p["w_router"] = torch.randn(E, H, generator=g, dtype=torch.float64) * 0.2
+    logits = (p["x"] @ p["w_router"].t()).float().numpy()
+    idx, _, _ = O.route_from_logits(logits, p["bias"].float().numpy(), k, norm)
+    d_out = torch.randn(T, H, generator=g, dtype=torch.float64)
+    return p, idx, d_out
+
+
+def _loss(p, idx, d_out, norm, act):
+    w = O.route_weights(p["x"] @ p["w_router"].t(), idx, norm)
+    return float((O.experts_forward(p["x"], idx, w, p["w_gate_up"], p["w_down"], p["theta"], dtype=torch.float64, act=act)
+                  * d_out).sum())
+
+
+@pytest.mark.parametrize("act,norm", [("radial", "sum"), ("tanh", "softmax"), ("silu", False)])
+def test_backward_matches_central_differences(act, norm):
+    """The gradient of every operand agrees with (L(v + h d) - L(v - h d)) / 2h along random directions d: pins the
+    autograd oracle against a dropped path (router, theta, norm) without retyping any derivative."""
+    p, idx, d_out = _bwd_case(act=act, norm=norm)
+    grads = O.moe_backward(p["x"], p["w_router"], p["w_gate_up"], p["w_down"], p["theta"], idx, d_out, norm=norm, act=act)
+    g = torch.Generator().manual_seed(5)
+    for name in ("x", "w_router", "w_gate_up", "w_down", "theta"):
+        if act == "silu" and name == "theta":
+            assert grads[name] is None or float(grads[name].abs().max()) == 0.0   # plain SiLU has no radial gain
+            continue
+        d = torch.randn(p[name].shape, generator=g, dtype=torch.float64)
+        h = 1e-6
+        base = p[name].clone()
+        p[name] = base + h * d
+        lp = _loss(p, idx, d_out, norm, act)
+        p[name] = base - h * d
+        lm = _loss(p, idx, d_out, norm, act)
+        p[name] = base
+        fd, an = (lp - lm) / (2 * h), float((grads[name] * d).sum())
+        assert abs(fd - an) <= 1e-6 * max(1.0, abs(an)), (name, fd, an)
+
+
+def test_radial_backward_closed_form():
+    """h = r^p SiLU(g/r) u, r = sqrt(mean(g^2) + eps), p = sigmoid(theta).  With a = SiLU(z), a' = s (1 + z (1 - s)),
+    s = sigmoid(z), z = g / r and q = dh u (all per element):
+      du = dh r^p a;   dg = q r^(p-1) a' + g / (I r) * sum_i q_i (p r^(p-1) a_i - r^(p-2) a'_i g_i);
+      dtheta = p (1 - p) ln(r) sum_i q_i r^p a_i."""
+    g0 = torch.Generator().manual_seed(2)
+    I = 24
+    gate = torch.randn(5, I, generator=g0, dtype=torch.float64, requires_grad=True)
+    up = torch.randn(5, I, generator=g0, dtype=torch.float64, requires_grad=True)
+    theta = torch.tensor(0.7, dtype=torch.float64, requires_grad=True)
+    dh = torch.randn(5, I, generator=g0, dtype=torch.float64)
+    (O.radial_normsilu(gate, theta) * up * dh).sum().backward()
+    with torch.no_grad():
+        r = torch.sqrt(gate.square().mean(-1, keepdim=True) + O.NORMSILU_EPS)
+        p = torch.sigmoid(theta)
+        z = gate / r
+        s = torch.sigmoid(z)
+        a, ad = z * s, s * (1 + z * (1 - s))
+        q = dh * up
+        du = dh * r.pow(p) * a
+        inner = (q * (p * r.pow(p - 1) * a - r.pow(p - 2) * ad * gate)).sum(-1, keepdim=True)
+        dg = q * r.pow(p - 1) * ad + gate / (I * r) * inner
+        dth = (p * (1 - p) * torch.log(r) * (q * r.pow(p) * a).sum(-1, keepdim=True)).sum()
+    assert torch.allclose(up.grad, du, rtol=1e-12, atol=1e-14)
+    assert torch.allclose(gate.grad, dg, rtol=1e-10, atol=1e-13)
+    assert abs(float(theta.grad) - float(dth)) <= 1e-12 * max(1.0, abs(float(dth)))
+
+
+@pytest.mark.parametrize("norm", ["sum", "softmax", False])
+def test_route_weight_backward_closed_form(norm):
+    """sum: w = s / (S + eps), S = sum of the selected scores: ds_j = (dw_j - sum_i dw_i w_i) / (S + eps);
+    softmax over the selected scores: ds_j = w_j (dw_j - sum_i dw_i w_i); none: ds = dw; dlogit = ds s (1 - s)."""
+    g0 = torch.Generator().manual_seed(4)
+    logits = torch.randn(7, 10, generator=g0, dtype=torch.float64, requires_grad=True)
+    idx = np.stack([np.sort(np.random.default_rng(i).choice(10, 4, replace=False)) for i in range(7)])
+    dw = torch.randn(7, 4, generator=g0, dtype=torch.float64)
+    w = O.route_weights(logits, idx, norm)
+    (w * dw).sum().backward()
+    with torch.no_grad():
+        s = torch.sigmoid(logits).gather(-1, torch.from_numpy(idx))
+        dot = (dw * w).sum(-1, keepdim=True)
+        if norm == "sum":
+            ds = (dw - dot) / (s.sum(-1, keepdim=True) + O.SUM_NORM_EPS)
+        elif norm == "softmax":
+            ds = w * (dw - dot)
+        else:
+            ds = dw
+        dl = torch.zeros_like(logits).scatter_(-1, torch.from_numpy(idx), ds * s * (1 - s))
+    assert torch.allclose(logits.grad, dl, rtol=1e-12, atol=1e-15)
