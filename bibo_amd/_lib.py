@@ -22,7 +22,7 @@ SYMBOLS = (
     "bibo_moe_abi_version", "bibo_moe_strerror", "bibo_moe_workspace_bytes", "bibo_moe_select_algo", "bibo_moe_router_fwd",
     "bibo_moe_permute", "bibo_moe_gateup_fwd", "bibo_moe_down_combine_fwd", "bibo_moe_gateup_down_fwd",
     "bibo_moe_combine_fwd", "bibo_moe_combine_ex_fwd", "bibo_moe_experts_fwd", "bibo_moe_forward", "bibo_moe_rmsnorm_fwd",
-    "bibo_moe_ffn_workspace_bytes", "bibo_moe_ffn_forward", "bibo_moe_forward_static",
+    "bibo_moe_ffn_workspace_bytes", "bibo_moe_ffn_forward", "bibo_moe_forward_static", "bibo_moe_backward_workspace_bytes", "bibo_moe_backward",
 )
 STATIC_SCRATCH_BYTES = 16 << 20
 
@@ -71,6 +71,10 @@ def _declare(l):
     l.bibo_moe_ffn_forward.argtypes = [vp, vp, ctypes.c_float, vp, vp, vp, vp, vp, vp, ctypes.POINTER(Shape), ci, ci, vp, vp,
                                        vp, vp, vp, sz, vp]
     l.bibo_moe_forward_static.restype = ci
+    l.bibo_moe_backward_workspace_bytes.restype = ci
+    l.bibo_moe_backward_workspace_bytes.argtypes = [ctypes.POINTER(Shape), ctypes.POINTER(sz)]
+    l.bibo_moe_backward.restype = ci
+    l.bibo_moe_backward.argtypes = [vp, vp, vp, vp, vp, vp, vp, ctypes.POINTER(Shape), ci, vp, vp, vp, vp, vp, vp, vp, sz, vp]
     l.bibo_moe_forward_static.argtypes = [vp, vp, vp, vp, vp, vp, ctypes.POINTER(Shape), ci, ci, vp, vp, vp, vp, vp, vp]
     l.bibo_moe_forward.restype = ci
     l.bibo_moe_forward.argtypes = [vp, vp, vp, vp, vp, vp, ctypes.POINTER(Shape), ci, ci, vp, vp, vp, vp, vp, vp, sz, vp]

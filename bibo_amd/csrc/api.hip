@@ -246,6 +246,52 @@ int forward_impl(const void* x, const void* w_router, const float* bias, const v
 }
 
 
+struct BackwardWorkspace {
+  size_t hist, idx, w, logits, counts, offsets, perm_slot, perm_token, pad_off, dw_slot, dl, dtheta_row, wd_t, wgu_t, gu, dhp, dgu,
+      hidden, dxs, p_t, q_t, total;
+};
+
+BackwardWorkspace carve_backward(int T, int H, int E, int k, int I) {
+  const size_t S = (size_t)T * k, ld = backward_padded_rows(T, E, k), b = sizeof(bf16_t);
+  BackwardWorkspace ws;
+  size_t o = 0;
+  ws.hist = o;       o += align_up(permute_workspace_bytes(T) > router_hist_bytes(T) ? permute_workspace_bytes(T)
+                                                                                    : router_hist_bytes(T));
+  ws.idx = o;        o += align_up(S * sizeof(int32_t));
+  ws.w = o;          o += align_up(S * sizeof(float));
+  ws.logits = o;     o += align_up((size_t)T * E * sizeof(float));
+  ws.counts = o;     o += align_up(kMaxE * sizeof(int32_t));
+  ws.offsets = o;    o += align_up((kMaxE + 1) * sizeof(int32_t));
+  ws.perm_slot = o;  o += align_up(S * sizeof(int32_t));
+  ws.perm_token = o; o += align_up(S * sizeof(int32_t));
+  ws.pad_off = o;    o += align_up((kMaxE + 1) * sizeof(int32_t));
+  ws.dw_slot = o;    o += align_up(S * sizeof(float));
+  ws.dl = o;         o += align_up(S * sizeof(float));
+  ws.dtheta_row = o; o += align_up(S * sizeof(float));
+  ws.wd_t = o;       o += align_up((size_t)E * I * H * b);
+  ws.wgu_t = o;      o += align_up((size_t)E * H * 2 * I * b);
+  ws.gu = o;         o += align_up(S * 2 * I * b);
+  ws.dhp = o;        o += align_up(S * I * b);
+  ws.dgu = o;        o += align_up(S * 2 * I * b);
+  ws.hidden = o;     o += align_up(S * I * b);
+  ws.dxs = o;        o += align_up(S * H * b);
+  ws.p_t = o;        o += align_up((size_t)(H > 2 * I ? H : 2 * I) * ld * b);
+  ws.q_t = o;        o += align_up((size_t)(H > I ? H : I) * ld * b);
+  ws.total = o;
+  return ws;
+}
+
+int backward_check(const bibo_moe_shape* sh, int norm_mode) {
+  if (sh == nullptr) return BIBO_ERR_NULL_POINTER;
+  const int rc = check_dims(sh->T, sh->H, sh->E, sh->k, sh->I, sh->dtype, sh->n_pos, sh->n_neg);
+  if (rc != BIBO_OK) return rc;
+  if (norm_mode < BIBO_NORM_NONE || norm_mode > BIBO_NORM_SOFTMAX || !act_ok(sh->act)) return BIBO_ERR_UNSUPPORTED;
+  // bf16, GLU experts only, dimensions the MFMA tiles divide
+  if (sh->n_pos + sh->n_neg > 0 || !backward_supported(sh->H, sh->I, sh->k, sh->dtype)) return BIBO_ERR_UNSUPPORTED;
+  return BIBO_OK;
+}
+
+
 }  // namespace
 
 extern "C" {
@@ -474,6 +520,57 @@ int bibo_moe_ffn_forward(const void* h, const float* norm_weight, float eps, con
   if (e != hipSuccess) return (int)e;
   return forward_impl(xn, w_router, bias, w_gate_up, w_down, theta, sh, norm_mode, algo, res, out, idx_out, w_out,
                       counts_out, nullptr, workspace, inner, stream);
+}
+
+int bibo_moe_backward_workspace_bytes(const bibo_moe_shape* sh, size_t* bytes) {
+  if (bytes == nullptr) return BIBO_ERR_NULL_POINTER;
+  const int rc = backward_check(sh, BIBO_NORM_SUM);
+  if (rc != BIBO_OK) return rc;
+  *bytes = carve_backward(sh->T, sh->H, sh->E, sh->k, sh->I).total;
+  return BIBO_OK;
+}
+
+int bibo_moe_backward(const void* x, const void* d_out, const void* w_router, const float* bias, const void* w_gate_up,
+                      const void* w_down, const float* theta, const bibo_moe_shape* sh, int norm_mode, void* d_x,
+                      void* d_w_router, void* d_w_gate_up, void* d_w_down, float* d_theta, float* d_w_out,
+                      void* workspace, size_t workspace_bytes, void* stream) {
+  int rc = backward_check(sh, norm_mode);
+  if (rc != BIBO_OK) return rc;
+  const int T = sh->T, H = sh->H, E = sh->E, k = sh->k, I = sh->I;
+  if (!workspace) return BIBO_ERR_NULL_POINTER;
+  if (!aligned_ws(workspace)) return BIBO_ERR_MISALIGNED;
+  if (!d_w_router || !d_w_gate_up || !d_w_down || !d_theta) return BIBO_ERR_NULL_POINTER;
+  if (T > 0 && (!x || !d_out || !w_router || !bias || !w_gate_up || !w_down || !d_x)) return BIBO_ERR_NULL_POINTER;
+  if (T > 0 && !theta && sh->act != BIBO_ACT_SILU) return BIBO_ERR_NULL_POINTER;
+  if (!aligned16(x) || !aligned16(d_out) || !aligned16(w_router) || !aligned16(w_gate_up) || !aligned16(w_down) ||
+      !aligned16(d_x) || !aligned16(d_w_gate_up) || !aligned16(d_w_down))
+    return BIBO_ERR_MISALIGNED;
+  const BackwardWorkspace ws = carve_backward(T, H, E, k, I);
+  if (workspace_bytes < ws.total) return BIBO_ERR_WORKSPACE_TOO_SMALL;
+  char* base = static_cast<char*>(workspace);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  int32_t* idx = reinterpret_cast<int32_t*>(base + ws.idx);
+  float* w = reinterpret_cast<float*>(base + ws.w);
+  float* logits = reinterpret_cast<float*>(base + ws.logits);
+  int32_t* counts = reinterpret_cast<int32_t*>(base + ws.counts);
+  int32_t* offsets = reinterpret_cast<int32_t*>(base + ws.offsets);
+  int32_t* perm_slot = reinterpret_cast<int32_t*>(base + ws.perm_slot);
+  int32_t* perm_token = reinterpret_cast<int32_t*>(base + ws.perm_token);
+  // the routing of the forward pass again: same kernel, same inputs, hence the same selection and weights
+  if (T > 0 && (rc = hip_rc(launch_router(x, w_router, bias, T, H, E, k, sh->dtype, norm_mode, logits, idx, w, nullptr,
+                                          nullptr, nullptr, s))) != BIBO_OK)
+    return rc;
+  if ((rc = hip_rc(launch_permute(idx, T, E, k, counts, offsets, perm_slot, perm_token, base + ws.hist, s))) != BIBO_OK)
+    return rc;
+  BackwardBuffers b;
+  b.wd_t = base + ws.wd_t; b.wgu_t = base + ws.wgu_t; b.gu = base + ws.gu; b.dhp = base + ws.dhp; b.dgu = base + ws.dgu;
+  b.hidden = base + ws.hidden; b.dxs = base + ws.dxs; b.p_t = base + ws.p_t; b.q_t = base + ws.q_t;
+  b.dw_slot = d_w_out ? d_w_out : reinterpret_cast<float*>(base + ws.dw_slot);
+  b.dl = reinterpret_cast<float*>(base + ws.dl);
+  b.dtheta_row = reinterpret_cast<float*>(base + ws.dtheta_row);
+  b.pad_off = reinterpret_cast<int32_t*>(base + ws.pad_off);
+  return hip_rc(launch_backward(x, d_out, w_router, w_gate_up, w_down, theta, logits, idx, w, offsets, perm_slot, perm_token,
+                                T, H, E, k, I, norm_mode, sh->act, b, d_x, d_w_router, d_w_gate_up, d_w_down, d_theta, s));
 }
 
 }  // extern "C"

@@ -179,4 +179,18 @@ hipError_t launch_gateup_stream(const void* x, const void* wgu, const int32_t* i
 hipError_t launch_down_stream(const void* gu, const void* wd, const float* theta, const float* w, const int32_t* idx,
                               int T, int H, int E, int k, int I, int act, void* hidden, float* yw, hipStream_t s);
 
+// ---- backward pass (backward.hip) ----
+struct BackwardBuffers {
+  void *wd_t, *wgu_t, *gu, *dhp, *dgu, *hidden, *dxs, *p_t, *q_t;   // bf16 device buffers, sizes in launch_backward's comment
+  float *dw_slot, *dl, *dtheta_row;                                 // [T*k] each
+  int32_t* pad_off;                                                 // [E + 1]
+};
+bool backward_supported(int H, int I, int k, int dtype);
+size_t backward_padded_rows(int T, int E, int k);
+hipError_t launch_backward(const void* x, const void* d_out, const void* w_router, const void* wgu, const void* wd,
+                           const float* theta, const float* logits, const int32_t* idx, const float* w,
+                           const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token, int T, int H, int E,
+                           int k, int I, int norm_mode, int act, const BackwardBuffers& b, void* dx, void* d_w_router,
+                           void* d_wgu, void* d_wd, float* d_theta, hipStream_t s);
+
 }  // namespace bibo

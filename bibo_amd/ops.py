@@ -288,6 +288,34 @@ def moe_forward_static(x, w_router, bias, w_gate_up, w_down, theta, k, out, norm
     return out
 
 
+def moe_backward(x, d_out, w_router, bias, w_gate_up, w_down, theta, k, norm="sum", act="radial", want_dw=False):
+    """Gradients of the layer (bibo_moe_backward) for the upstream gradient d_out [T,H] of its output: what autograd
+    derives for BiBoMoELayer.forward (moe.py:157-183) with the selection held fixed.
+    -> d_x [T,H], d_w_router [E,H], d_w_gate_up [E,2I,H], d_w_down [E,H,I] (x.dtype), d_theta fp32 [E], d_w fp32 [T,k]|None."""
+    T, H = x.shape
+    E, two_i, _ = w_gate_up.shape
+    I = two_i // 2
+    dc = _dtype_code(x)
+    _chk(x, "x"); _chk(d_out, "d_out", x.dtype, (T, H)); _chk(w_router, "w_router", x.dtype, (E, H))
+    _chk(bias, "bias", torch.float32, (E,)); _chk(w_gate_up, "w_gate_up", x.dtype, (E, 2 * I, H))
+    _chk(w_down, "w_down", x.dtype, (E, H, I)); _chk(theta, "theta", torch.float32, (E,))
+    dev = x.device
+    d_x = torch.empty_like(x)
+    d_wr, d_gu, d_dn = torch.empty_like(w_router), torch.empty_like(w_gate_up), torch.empty_like(w_down)
+    d_theta = torch.empty(E, dtype=torch.float32, device=dev)
+    d_w = torch.empty(T, k, dtype=torch.float32, device=dev) if want_dw else None
+    sh = L.Shape(T, H, E, k, I, dc, 0, 0, act_code(act), 0)
+    nbytes = ctypes.c_size_t(0)
+    L.check(L.lib().bibo_moe_backward_workspace_bytes(ctypes.byref(sh), ctypes.byref(nbytes)), "bibo_moe_backward_workspace_bytes")
+    ws = workspace(dev, nbytes.value)
+    with torch.cuda.device(dev):
+        L.check(L.lib().bibo_moe_backward(_ptr(x), _ptr(d_out), _ptr(w_router), _ptr(bias), _ptr(w_gate_up), _ptr(w_down),
+                                          _ptr(theta), ctypes.byref(sh), norm_mode(norm), _ptr(d_x), _ptr(d_wr), _ptr(d_gu),
+                                          _ptr(d_dn), _ptr(d_theta), _ptr(d_w), _ptr(ws), ws.numel(), _stream(dev)),
+                "bibo_moe_backward")
+    return d_x, d_wr, d_gu, d_dn, d_theta, d_w
+
+
 def rmsnorm_fwd(x, norm_weight, eps):
     """out = norm_weight * round(x * rsqrt(mean(x^2) + eps)) in x.dtype (the block's input norm, norm.py:19-24)."""
     T, H = x.shape

@@ -260,6 +260,27 @@ int bibo_moe_ffn_forward(const void* h, const float* norm_weight, float eps, con
                          int norm_mode, int algo, void* out, int32_t* idx_out, float* w_out, int32_t* counts_out,
                          void* workspace, size_t workspace_bytes, void* stream);
 
+/*
+ * Backward pass of the layer: the gradients torch.autograd derives for BiBoMoELayer.forward in training
+ * (src/modeling/ffn/moe.py:157-183 with the experts of moe.py:46-101 and the router of router.py:25-47) for the
+ * upstream gradient d_out [T,H] of the layer's output, with the selection held fixed (the balancing bias only enters
+ * the selection, router.py:38, and gets no gradient; nor does anything flow through which experts were chosen).
+ * x is the block's input as in bibo_moe_forward; the routing is recomputed from it by the forward's router kernel,
+ * so the selection and the combine weights are those of the forward call on the same operands.
+ *   d_x [T,H], d_w_router [E,H], d_w_gate_up [E,2I,H], d_w_down [E,H,I] in `dtype`; d_theta fp32 [E]
+ *   (reference pins: theta receives gradient, tests/test_moe.py:53-63, ablate/common/test_eager_radial.py:63-69);
+ *   d_w_out fp32 [T,k] or NULL: gradient with respect to the combine weights (router.py:47), for inspection.
+ * bf16 only, H and I multiples of 128, I <= 512, no +/-Identity experts (BIBO_ERR_UNSUPPORTED otherwise); the
+ * intermediate activations are recomputed, nothing has to be kept from the forward call.  All gradients are
+ * overwritten, not accumulated.  Workspace: bibo_moe_backward_workspace_bytes (about 14 bytes per routed slot and
+ * column plus one transposed copy of the expert weights).
+ */
+int bibo_moe_backward_workspace_bytes(const bibo_moe_shape* shape, size_t* bytes);
+int bibo_moe_backward(const void* x, const void* d_out, const void* w_router, const float* bias, const void* w_gate_up,
+                      const void* w_down, const float* theta, const bibo_moe_shape* shape, int norm_mode, void* d_x,
+                      void* d_w_router, void* d_w_gate_up, void* d_w_down, float* d_theta, float* d_w_out,
+                      void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

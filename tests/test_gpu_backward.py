@@ -1,0 +1,95 @@
+"""Backward pass of the layer through the C ABI (bibo_moe_backward) against the oracle's autograd gradients, which
+are pinned on the CPU by central differences and closed forms (tests/test_oracle.py).  The oracle differentiates the
+fp64 forward with the selection the kernel made; the kernel works in bf16 with fp32 accumulation, so gradients are
+compared by max |difference| relative to max |reference| per tensor."""
+import numpy as np
+import pytest
+import torch
+
+from bibo_amd import ops
+from oracle import bibo_moe_oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+TOL = 2e-2          # bf16 operands, fp32 accumulation, bf16 results
+
+
+def _rel(a, ref):
+    return float((a.double().cpu() - ref.double()).abs().max() / ref.double().abs().max().clamp_min(1e-30))
+
+
+def _run(T, H, E, k, I, norm="sum", act="radial", seed=0, theta="normal", scale=1.0):
+    p = O.make_inputs(T=T, H=H, E=E, k=k, I=I, bias="uniform", theta=theta, seed=seed)
+    g = torch.Generator().manual_seed(seed + 100)
+    d_out = (torch.randn(T, H, generator=g) * scale).to(torch.bfloat16)
+    dev = lambda t: t.to(DEV)
+    _, idx, w, _, logits = ops.moe_forward(dev(p["x"]), dev(p["w_router"]), dev(p["bias"]), dev(p["w_gate_up"]),
+                                           dev(p["w_down"]), dev(p["theta"]), k, norm=norm, act=act, want_routing=True,
+                                           want_logits=True)
+    got = ops.moe_backward(dev(p["x"]), dev(d_out), dev(p["w_router"]), dev(p["bias"]), dev(p["w_gate_up"]), dev(p["w_down"]),
+                           dev(p["theta"]), k, norm=norm, act=act, want_dw=True)
+    torch.cuda.synchronize()
+    ref = O.moe_backward(p["x"], p["w_router"], p["w_gate_up"], p["w_down"], p["theta"], idx.cpu().numpy(), d_out, norm=norm,
+                         act=act)
+    return dict(zip(("x", "w_router", "w_gate_up", "w_down", "theta", "w"), got)), ref, idx.cpu().numpy()
+
+
+@pytest.mark.parametrize("T,H,E,k,I", [(300, 256, 16, 4, 128), (512, 512, 64, 6, 256), (64, 384, 8, 2, 384), (1000, 768, 64, 6, 384)])
+def test_backward_matches_oracle(T, H, E, k, I):
+    got, ref, _ = _run(T, H, E, k, I, seed=T)
+    for name in ("w", "x", "w_down", "w_gate_up", "w_router", "theta"):
+        assert _rel(got[name], ref[name]) <= TOL, (name, _rel(got[name], ref[name]))
+
+
+@pytest.mark.parametrize("norm,act", [("softmax", "radial"), (False, "tanh"), ("sum", "silu"), ("sum", "tanh")])
+def test_backward_norm_modes_and_activations(norm, act):
+    got, ref, _ = _run(320, 256, 16, 3, 128, norm=norm, act=act, seed=7)
+    for name in ("w", "x", "w_down", "w_gate_up", "w_router"):
+        assert _rel(got[name], ref[name]) <= TOL, (name, _rel(got[name], ref[name]))
+    if act == "silu":
+        assert float(got["theta"].abs().max()) == 0.0            # plain SwiGLU: theta is not read
+    else:
+        assert _rel(got["theta"], ref["theta"]) <= TOL
+
+
+def test_backward_idle_experts_and_ragged_rows():
+    """Experts that get no row have zero weight gradients; row counts that are no multiple of any tile size."""
+    T, H, E, k, I = 37, 256, 64, 2, 128
+    got, ref, idx = _run(T, H, E, k, I, seed=5)
+    idle = np.setdiff1d(np.arange(E), np.unique(idx))
+    assert idle.size > 0
+    for name in ("w_down", "w_gate_up", "w_router"):
+        assert float(got[name][torch.from_numpy(idle).to(DEV)].abs().max()) == 0.0
+        assert _rel(got[name], ref[name]) <= TOL, name
+    assert _rel(got["x"], ref["x"]) <= TOL and _rel(got["theta"], ref["theta"]) <= TOL
+
+
+def test_backward_is_linear_in_the_upstream_gradient():
+    """Size-independent property at the full c2 shape: the gradients of 2 d are twice those of d (every path is linear
+    in d_out), to bf16 rounding; and nothing is accumulated between calls."""
+    T, H, E, k, I = 8192, 768, 64, 6, 384
+    p = O.make_inputs(T=T, H=H, E=E, k=k, I=I, bias="uniform", theta="normal", seed=20262)
+    g = torch.Generator().manual_seed(1)
+    d = torch.randn(T, H, generator=g).to(torch.bfloat16).to(DEV)
+    args = [p[n].to(DEV) for n in ("w_router", "bias", "w_gate_up", "w_down", "theta")]
+    x = p["x"].to(DEV)
+    a = ops.moe_backward(x, d, *args, k)
+    b = ops.moe_backward(x, (2 * d.float()).to(torch.bfloat16), *args, k)
+    a2 = ops.moe_backward(x, d, *args, k)
+    torch.cuda.synchronize()
+    for u, v, u2 in zip(a[:5], b[:5], a2[:5]):
+        assert torch.equal(u, u2)
+        assert _rel(v.float(), 2 * u.float().cpu()) <= 1e-2
+    assert all(bool(torch.isfinite(t.float()).all()) for t in a[:5])
+
+
+def test_backward_rejects_what_it_does_not_cover():
+    from bibo_amd import _lib as L
+    import ctypes
+    sh = L.Shape(64, 200, 8, 2, 128, L.DTYPE_BF16)                  # H no multiple of 128
+    n = ctypes.c_size_t(0)
+    assert L.lib().bibo_moe_backward_workspace_bytes(ctypes.byref(sh), ctypes.byref(n)) == -6
+    sh = L.Shape(64, 256, 8, 2, 128, L.DTYPE_BF16, 1, 1)            # +/-Identity experts
+    assert L.lib().bibo_moe_backward_workspace_bytes(ctypes.byref(sh), ctypes.byref(n)) == -6
+    sh = L.Shape(64, 256, 8, 2, 128, L.DTYPE_F32)
+    assert L.lib().bibo_moe_backward_workspace_bytes(ctypes.byref(sh), ctypes.byref(n)) == -6
