@@ -3,7 +3,8 @@
 Class names, constructor argument, attribute names, parameter shapes and state_dict keys follow
 src/modeling/ffn/router.py and src/modeling/ffn/moe.py of the reference, so a reference checkpoint
 loads with strict=True and code that pokes at `layer.gate.bias` or `layer.experts.radial_theta`
-keeps working.  Forward only: outputs carry no autograd graph."""
+keeps working.  `BiBoMoELayer.forward` is differentiable (its backward is the library's bibo_moe_backward) for bf16
+compute without hooks; `BiBoMoERouter` and `BiBoFusedExperts` called on their own are forward only."""
 from __future__ import annotations
 
 import torch
@@ -20,11 +21,46 @@ except AttributeError:                                    # older torch
     _no_compile = torch._dynamo.disable
 
 
+def _wants_grad(*tensors) -> bool:
+    return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors)
+
+
 def _forward_only_guard(*tensors):
-    if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors):
+    if _wants_grad(*tensors):
         raise RuntimeError(
-            "bibo_amd implements the forward pass only; call it under torch.no_grad() or torch.inference_mode() "
-            "(an input or parameter requires grad and autograd is enabled, so gradients would silently be lost)")
+            "this bibo_amd entry point implements the forward pass only; call it under torch.no_grad() or "
+            "torch.inference_mode() (an input or parameter requires grad and autograd is enabled, so gradients would "
+            "silently be lost).  BiBoMoELayer.forward without hooks is the differentiable path")
+
+
+class _MoELayerFn(torch.autograd.Function):
+    """The whole layer as one autograd node: forward = bibo_moe_forward, backward = bibo_moe_backward, which recomputes
+    the routing and the activations from the saved input, so nothing but the input rows is kept.  Gradients are what
+    autograd gives the reference's eager layer with the selection held fixed (moe.py:157-183); the balancing bias
+    gets none (router.py:38).  The per-expert row counts come out as a second, non-differentiable result."""
+
+    @staticmethod
+    def forward(ctx, x, w_router, w_gate_up, w_down, theta, bias, k, norm, act, algo, want_counts):
+        cd = torch.bfloat16
+        cast = lambda t, d: (t if t.dtype == d else t.to(d)).contiguous()
+        xb, wr, gu, dn = cast(x.detach(), cd), cast(w_router.detach(), cd), cast(w_gate_up.detach(), cd), cast(w_down.detach(), cd)
+        th, b = cast(theta.detach(), torch.float32), cast(bias.detach(), torch.float32)
+        out, _, _, counts, _ = ops.moe_forward(xb, wr, b, gu, dn, th, k, norm=norm, algo=algo, want_counts=want_counts, act=act)
+        ctx.save_for_backward(xb, wr, gu, dn, th, b)
+        ctx.conf = (k, norm, act)
+        ctx.in_dtypes = (x.dtype, w_router.dtype, w_gate_up.dtype, w_down.dtype, theta.dtype)
+        if counts is None:
+            counts = torch.empty(0, dtype=torch.int32, device=x.device)
+        ctx.mark_non_differentiable(counts)
+        return out, counts
+
+    @staticmethod
+    def backward(ctx, d_out, _d_counts):
+        xb, wr, gu, dn, th, b = ctx.saved_tensors
+        k, norm, act = ctx.conf
+        d = d_out.to(torch.bfloat16).contiguous()
+        grads = ops.moe_backward(xb, d, wr, b, gu, dn, th, k, norm=norm, act=act)[:5]
+        return tuple(g.to(dt) for g, dt in zip(grads, ctx.in_dtypes)) + (None,) * 6
 
 
 class _CastCache:
@@ -308,8 +344,12 @@ class BiBoMoELayer(nn.Module):
             res = self.experts(hidden_states.reshape(num_tokens, hdim), top_idx.view(num_tokens, -1),
                                top_w.view(num_tokens, -1), _want_counts=balancing)
             out, counts = res if balancing else (res, None)
+        elif _wants_grad(hidden_states, self.gate.gate_proj.weight, self.experts.gate_up_proj, self.experts.down_proj,
+                         self.experts.radial_theta):
+            out, counts = self._differentiable_forward(hidden_states.reshape(num_tokens, hdim), balancing)
+            out = out if out.dtype == hidden_states.dtype else out.to(hidden_states.dtype)
+            top_idx = None
         else:
-            _forward_only_guard(hidden_states, self.gate.gate_proj.weight, self.experts.gate_up_proj)
             cd = _compute_dtype(hidden_states)
             x = hidden_states.detach().reshape(num_tokens, hdim)
             x = (x.to(cd) if x.dtype != cd else x).contiguous()
@@ -331,6 +371,22 @@ class BiBoMoELayer(nn.Module):
                 self.update_bias(tpe)
         return out
 
+    def _differentiable_forward(self, x: torch.Tensor, want_counts: bool):
+        """x [T,H] -> (out [T,H] bf16 with an autograd graph, counts|None).  bf16 compute only (bf16 activations, or
+        fp32 activations under bf16 autocast), GLU experts only, H and I multiples of 128 and I <= 512: what
+        bibo_moe_backward covers."""
+        e = self.experts
+        if _compute_dtype(x) != torch.bfloat16:
+            raise RuntimeError("the backward pass runs in bf16: use bf16 activations or bf16 autocast, or call the layer "
+                               "under torch.no_grad()")
+        if e.num_pos + e.num_neg > 0 or self.hidden_size % 128 or e.intermediate_size % 128 or e.intermediate_size > 512:
+            raise NotImplementedError("the backward pass covers GLU experts only (no +/-Identity experts), hidden and "
+                                      "expert sizes that are multiples of 128 and expert size <= 512")
+        out, counts = _MoELayerFn.apply(x, self.gate.gate_proj.weight, e.gate_up_proj, e.down_proj, e.radial_theta,
+                                        self.gate.bias, self.num_experts_per_tok, self.gate.norm_topk_prob, e.act, e.algo,
+                                        want_counts)
+        return out, (counts if want_counts else None)
+
     @_no_compile
     def ffn_forward(self, hidden_states: torch.Tensor, norm_weight: torch.Tensor, eps: float,
                     bf16_stream: bool = False, bf16_moe_out: bool = False, residual=None) -> torch.Tensor:
@@ -346,17 +402,19 @@ class BiBoMoELayer(nn.Module):
         bsz, seq, hdim = hidden_states.shape
         num_tokens = bsz * seq
         if (self._hooks_present() or self.use_shared_expert or hidden_states.dtype != _compute_dtype(hidden_states)
-                or (bf16_moe_out and hidden_states.dtype != torch.bfloat16)):
-            # (an fp32 residual stream under bf16 autocast keeps its fp32 norm and fp32 residual add)
+                or (bf16_moe_out and hidden_states.dtype != torch.bfloat16)
+                or _wants_grad(hidden_states, norm_weight, self.gate.gate_proj.weight, self.experts.gate_up_proj,
+                               self.experts.down_proj, self.experts.radial_theta)):
+            # (an fp32 residual stream under bf16 autocast keeps its fp32 norm and fp32 residual add; with autograd
+            # on, norm and residual are ordinary differentiable operations around the differentiable block)
             xf = hidden_states.float()
             xn = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)).to(hidden_states.dtype)    # norm.py:21-24
-            blk = self.forward(norm_weight * xn)                                                       # layers.py:60-61
+            blk = self.forward((norm_weight * xn).to(hidden_states.dtype))                             # layers.py:60-61
             blk = blk.to(torch.bfloat16) if bf16_moe_out else blk                                      # layers.py:62-63
             base = hidden_states if residual is None else residual
             out = blk.to(hidden_states.dtype) if residual is False else base + blk.to(hidden_states.dtype)   # layers.py:64
             return out.to(torch.bfloat16) if bf16_stream else out
         balancing = self.training and self.bias_update_factor > 0
-        _forward_only_guard(hidden_states, self.gate.gate_proj.weight, self.experts.gate_up_proj)
         cd = _compute_dtype(hidden_states)
         h = hidden_states.detach().reshape(num_tokens, hdim)
         h = (h.to(cd) if h.dtype != cd else h).contiguous()

@@ -93,3 +93,85 @@ def test_backward_rejects_what_it_does_not_cover():
     assert L.lib().bibo_moe_backward_workspace_bytes(ctypes.byref(sh), ctypes.byref(n)) == -6
     sh = L.Shape(64, 256, 8, 2, 128, L.DTYPE_F32)
     assert L.lib().bibo_moe_backward_workspace_bytes(ctypes.byref(sh), ctypes.byref(n)) == -6
+
+
+# ---- the module: BiBoMoELayer.forward under autograd ----
+def _layer(H=256, I=128, E=8, k=2, **kw):
+    from bibo_amd.config import BiBoMoEConfig
+    from bibo_amd.moe import BiBoMoELayer
+    cfg = BiBoMoEConfig(hidden_size=H, moe_intermediate_size=I, num_routed_experts=E, num_experts_per_tok=k,
+                        special_expert_pairs=0, **kw)
+    torch.manual_seed(0)
+    return BiBoMoELayer(cfg).to(DEV).bfloat16()
+
+
+def test_radial_theta_is_a_real_learnable_parameter():
+    """The reference's regression test (tests/test_moe.py:53-63): theta requires grad, starts at 0, and a backward
+    through the layer leaves a non-zero gradient in it."""
+    layer = _layer()
+    th = layer.experts.radial_theta
+    assert th.requires_grad and float(th.detach().abs().max()) == 0.0
+    x = torch.randn(2, 6, 256, device=DEV, dtype=torch.bfloat16)
+    (layer(x) * torch.randn(2, 6, 256, device=DEV, dtype=torch.bfloat16)).sum().backward()
+    assert th.grad is not None and float(th.grad.abs().max()) > 0
+
+
+def test_layer_gradients_match_oracle():
+    layer = _layer(H=256, I=128, E=16, k=4)
+    with torch.no_grad():
+        layer.experts.radial_theta.copy_(torch.linspace(-2, 3, 16))
+        layer.gate.bias.copy_(torch.linspace(-0.01, 0.01, 16))
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(3, 50, 256, generator=g).to(torch.bfloat16).to(DEV).requires_grad_(True)
+    d = torch.randn(3, 50, 256, generator=g).to(torch.bfloat16).to(DEV)
+    layer.train()
+    out = layer(x)
+    out.backward(d)
+    torch.cuda.synchronize()
+    p = {n: v.detach().cpu() for n, v in (("wr", layer.gate.gate_proj.weight), ("b", layer.gate.bias),
+                                          ("gu", layer.experts.gate_up_proj), ("dn", layer.experts.down_proj),
+                                          ("th", layer.experts.radial_theta))}
+    x2 = x.detach().cpu().reshape(150, 256)
+    _, idx, _, _, _ = ops.moe_forward(x.detach().reshape(150, 256), layer.gate.gate_proj.weight.detach(), layer.gate.bias.detach().float(),
+                                      layer.experts.gate_up_proj.detach(), layer.experts.down_proj.detach(),
+                                      layer.experts.radial_theta.detach().float(), 4, want_routing=True)
+    ref = O.moe_backward(x2, p["wr"], p["gu"], p["dn"], p["th"].float(), idx.cpu().numpy(), d.cpu().reshape(150, 256))
+    assert _rel(x.grad.reshape(150, 256), ref["x"]) <= TOL
+    assert _rel(layer.gate.gate_proj.weight.grad, ref["w_router"]) <= TOL
+    assert _rel(layer.experts.gate_up_proj.grad, ref["w_gate_up"]) <= TOL
+    assert _rel(layer.experts.down_proj.grad, ref["w_down"]) <= TOL
+    assert _rel(layer.experts.radial_theta.grad, ref["theta"]) <= TOL
+    assert layer.gate.bias.grad is None                          # selection only (router.py:38)
+    assert float(layer.accumulated_tpe.sum()) == 150 * 4        # the training forward still feeds the balancing state
+
+
+def test_seam_and_shared_expert_under_autograd():
+    """ffn_forward with autograd on: norm and residual become ordinary differentiable operations around the block, and
+    the shared expert's parameters get gradients as well."""
+    layer = _layer(H=256, I=128, E=8, k=2, use_shared_expert=True)
+    nw = torch.ones(256, device=DEV, requires_grad=True)
+    h = torch.randn(2, 20, 256, device=DEV, dtype=torch.bfloat16, requires_grad=True)
+    out = layer.ffn_forward(h, nw, 1e-6)
+    out.float().square().sum().backward()
+    assert h.grad is not None and nw.grad is not None and float(nw.grad.abs().max()) > 0
+    for prm in layer.parameters():
+        if prm.requires_grad:
+            assert prm.grad is not None and bool(torch.isfinite(prm.grad.float()).all())
+
+
+def test_what_the_backward_does_not_cover_is_refused():
+    from bibo_amd.config import BiBoMoEConfig
+    from bibo_amd.moe import BiBoMoELayer
+    layer = BiBoMoELayer(BiBoMoEConfig(hidden_size=256, moe_intermediate_size=128, num_routed_experts=8,
+                                       num_experts_per_tok=2, special_expert_pairs=1)).to(DEV).bfloat16()
+    x = torch.randn(1, 8, 256, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(NotImplementedError):
+        layer(x)                                                   # +/-Identity experts: forward only
+    with torch.no_grad():
+        layer(x)
+    fp32 = _layer().float()
+    with pytest.raises(RuntimeError):
+        fp32(torch.randn(1, 8, 256, device=DEV))                   # fp32 compute: forward only
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        fp32(torch.randn(1, 8, 256, device=DEV)).sum().backward()  # fp32 master weights under bf16 autocast train
+    assert fp32.experts.gate_up_proj.grad is not None and fp32.experts.gate_up_proj.grad.dtype == torch.float32
