@@ -247,7 +247,7 @@ int forward_impl(const void* x, const void* w_router, const float* bias, const v
 
 
 struct BackwardWorkspace {
-  size_t hist, idx, w, logits, counts, offsets, perm_slot, perm_token, pad_off, dw_slot, dl, dtheta_row, wd_t, wgu_t, gu, dhp, dgu,
+  size_t hist, idx, w, logits, counts, offsets, perm_slot, perm_token, pad_off, dw_slot, dl, dtheta_row, dwr_part, wd_t, wgu_t, gu, dhp, dgu,
       hidden, dxs, p_t, q_t, total;
 };
 
@@ -268,6 +268,7 @@ BackwardWorkspace carve_backward(int T, int H, int E, int k, int I) {
   ws.dw_slot = o;    o += align_up(S * sizeof(float));
   ws.dl = o;         o += align_up(S * sizeof(float));
   ws.dtheta_row = o; o += align_up(S * sizeof(float));
+  ws.dwr_part = o;   o += align_up((size_t)E * backward_dwr_split() * H * sizeof(float));
   ws.wd_t = o;       o += align_up((size_t)E * I * H * b);
   ws.wgu_t = o;      o += align_up((size_t)E * H * 2 * I * b);
   ws.gu = o;         o += align_up(S * 2 * I * b);
@@ -568,6 +569,7 @@ int bibo_moe_backward(const void* x, const void* d_out, const void* w_router, co
   b.dw_slot = d_w_out ? d_w_out : reinterpret_cast<float*>(base + ws.dw_slot);
   b.dl = reinterpret_cast<float*>(base + ws.dl);
   b.dtheta_row = reinterpret_cast<float*>(base + ws.dtheta_row);
+  b.dwr_part = reinterpret_cast<float*>(base + ws.dwr_part);
   b.pad_off = reinterpret_cast<int32_t*>(base + ws.pad_off);
   return hip_rc(launch_backward(x, d_out, w_router, w_gate_up, w_down, theta, logits, idx, w, offsets, perm_slot, perm_token,
                                 T, H, E, k, I, norm_mode, sh->act, b, d_x, d_w_router, d_w_gate_up, d_w_down, d_theta, s));

@@ -20,6 +20,10 @@ namespace bibo {
 namespace {
 
 constexpr int kPad = 64;     // an expert's rows start at a multiple of this in the transposed buffers
+#ifndef BIBO_BWD_BK
+#define BIBO_BWD_BK 64
+#endif
+constexpr int kBwdBK = BIBO_BWD_BK;   // K elements per LDS stage of the GEMMs here: 64 = whole 128-byte lines per row
 
 // ---- grouped GEMM: out[dst(r), n] = sum_k A[src(r), k] W[e][n, k] for the rows r of expert e ------------------
 // src(r) = a_index[r] (GATHER) or r; dst(r) = out_index[r] (SCATTER) or r.  r runs over permuted rows.
@@ -29,7 +33,7 @@ __global__ __launch_bounds__(256 * WM) void ggemm_kernel(const bf16_t* __restric
                                                          const int32_t* __restrict__ offsets,
                                                          const int32_t* __restrict__ out_index, int K, int N, int E,
                                                          int nblk_n, bf16_t* __restrict__ out) {
-  using S = Stripe<MT, NTW, WM, kBK>;
+  using S = Stripe<MT, NTW, WM, kBwdBK>;
   constexpr int BM = S::BM;
   constexpr int BN = S::BN;
   __shared__ __attribute__((aligned(16))) bf16_t st0[S::kStageElems];
@@ -112,7 +116,7 @@ template <int NTW, bool GATHER, bool SCATTER>
 hipError_t launch_ggemm_t(const bf16_t* A, const int32_t* a_index, const bf16_t* W, const int32_t* offsets,
                           const int32_t* out_index, int S_rows, int K, int N, int E, bf16_t* out, hipStream_t s) {
   constexpr int MT = 2, WM = 2;
-  using St = Stripe<MT, NTW, WM, kBK>;
+  using St = Stripe<MT, NTW, WM, kBwdBK>;
   const int nblk_n = N / St::BN;
   const int tiles = (S_rows / St::BM + E) * nblk_n;
   const int grid = ((tiles + 7) & ~7) + 8;
@@ -130,25 +134,59 @@ hipError_t launch_ggemm(const bf16_t* A, const int32_t* a_index, const bf16_t* W
 }
 
 // ---- transposes ---------------------------------------------------------------------------------------------
-// out[b][c][r] = in[b][r][c] for b < batch: 64 x 64 tiles through LDS (row stride 66 elements: the column reads of
-// a wave then touch 32 different banks).  grid = (C / 64, R / 64, batch), 256 threads.
+// A 64 x 64 tile goes through LDS (row stride 66 elements: the eight column reads behind one 16-byte store touch
+// different banks); global memory is read and written 16 bytes per thread, 128 contiguous bytes per row.
+constexpr int kTS = 66;
+
+// rows j = t / 8 and j + 32 of the tile, columns 8 (t % 8) .. + 8: row j of the tile is in[src(j)], scaled; src < 0: zeros
+template <typename RowPtr, typename Scale>
+__device__ __forceinline__ void tile_load(bf16_t (&tile)[64][kTS], RowPtr row_ptr, Scale scale) {
+  const int t = threadIdx.x, cg = (t & 7) * 8;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int j = (t >> 3) + 32 * h;
+    const bf16_t* src = row_ptr(j);
+    bf16x8 v;
+    if (src != nullptr) {
+      v = *reinterpret_cast<const bf16x8*>(src + cg);
+      const float sc = scale(j);
+      if (sc != 1.f) {
+#pragma unroll
+        for (int q = 0; q < 8; ++q) v[q] = (bf16_t)(sc * (float)v[q]);
+      }
+    } else {
+#pragma unroll
+      for (int q = 0; q < 8; ++q) v[q] = (bf16_t)0.f;
+    }
+#pragma unroll
+    for (int q = 0; q < 8; q += 2)          // 4-byte LDS writes (the row stride is not a multiple of 16 bytes)
+      *reinterpret_cast<bf16x2*>(&tile[j][cg + q]) = bf16x2{v[q], v[q + 1]};
+  }
+}
+
+// column c = t / 8 and c + 32 of the tile, rows 8 (t % 8) .. + 8, to out_row(c) + 8 (t % 8)
+template <typename OutPtr>
+__device__ __forceinline__ void tile_store_transposed(const bf16_t (&tile)[64][kTS], OutPtr out_row) {
+  const int t = threadIdx.x, pg = (t & 7) * 8;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int c = (t >> 3) + 32 * h;
+    bf16x8 v;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) v[q] = tile[pg + q][c];
+    *reinterpret_cast<bf16x8*>(out_row(c) + pg) = v;
+  }
+}
+
+// out[b][c][r] = in[b][r][c] for b < batch.  grid = (C / 64, R / 64, batch), 256 threads.
 __global__ __launch_bounds__(256) void transpose_batched_kernel(const bf16_t* __restrict__ in, int R, int C,
                                                                 bf16_t* __restrict__ out) {
-  __shared__ bf16_t tile[64][66];
+  __shared__ __attribute__((aligned(16))) bf16_t tile[64][kTS];
   const size_t base = (size_t)blockIdx.z * R * C;
   const int c0 = blockIdx.x * 64, r0 = blockIdx.y * 64;
-  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-#pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    const int r = ty * 16 + i;
-    tile[r][tx] = in[base + (size_t)(r0 + r) * C + c0 + tx];
-  }
+  tile_load(tile, [&](int j) { return in + base + (size_t)(r0 + j) * C + c0; }, [](int) { return 1.f; });
   __syncthreads();
-#pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    const int c = ty * 16 + i;
-    out[base + (size_t)(c0 + c) * R + r0 + tx] = tile[tx][c];
-  }
+  tile_store_transposed(tile, [&](int c) { return out + base + (size_t)(c0 + c) * R + r0; });
 }
 
 // pad_off[e] = sum over e' < e of the rows of e' rounded up to kPad (one wave; E <= 64)
@@ -171,14 +209,13 @@ __global__ __launch_bounds__(256) void transpose_rows_kernel(const bf16_t* __res
                                                              const int32_t* __restrict__ offsets,
                                                              const int32_t* __restrict__ pad_off, int E, int C, int ld,
                                                              bf16_t* __restrict__ outT) {
-  __shared__ bf16_t tile[64][66];
+  __shared__ __attribute__((aligned(16))) bf16_t tile[64][kTS];
   __shared__ int src_s[64];
   __shared__ float scale_s[64];
   const int p0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
   if (p0 >= pad_off[E]) return;
   int e = 0;
   while (pad_off[e + 1] <= p0) ++e;                            // E <= 64 steps, uniform
-  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
   if (threadIdx.x < 64) {
     const int r = offsets[e] + (p0 - pad_off[e]) + threadIdx.x;
     const bool live = r < offsets[e + 1];
@@ -186,18 +223,10 @@ __global__ __launch_bounds__(256) void transpose_rows_kernel(const bf16_t* __res
     scale_s[threadIdx.x] = (live && scale_by_slot) ? scale_by_slot[slot_of_row[r]] : 1.f;
   }
   __syncthreads();
-#pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    const int j = ty * 16 + i;
-    const int src = src_s[j];
-    tile[j][tx] = src >= 0 ? (bf16_t)(scale_s[j] * (float)in[(size_t)src * C + c0 + tx]) : (bf16_t)0.f;
-  }
+  tile_load(tile, [&](int j) { return src_s[j] >= 0 ? in + (size_t)src_s[j] * C + c0 : nullptr; },
+            [&](int j) { return scale_s[j]; });
   __syncthreads();
-#pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    const int c = ty * 16 + i;
-    outT[(size_t)(c0 + c) * ld + p0 + tx] = tile[tx][c];
-  }
+  tile_store_transposed(tile, [&](int c) { return outT + (size_t)(c0 + c) * ld + p0; });
 }
 
 // ---- weight gradients: dW[e][n][m] = sum over the padded rows kc of expert e of PT[n][kc] QT[m][kc] --------------
@@ -206,7 +235,7 @@ template <int MT, int NTW, int WM>
 __global__ __launch_bounds__(256 * WM) void wgrad_kernel(const bf16_t* __restrict__ PT, const bf16_t* __restrict__ QT,
                                                          const int32_t* __restrict__ pad_off, int N, int M, int ld,
                                                          bf16_t* __restrict__ dW) {
-  using S = Stripe<MT, NTW, WM, kBK>;
+  using S = Stripe<MT, NTW, WM, kBwdBK>;
   constexpr int BM = S::BM, BN = S::BN;
   __shared__ __attribute__((aligned(16))) bf16_t st0[S::kStageElems];
   __shared__ __attribute__((aligned(16))) bf16_t st1[S::kStageElems];
@@ -255,7 +284,7 @@ template <int NTW>
 hipError_t launch_wgrad_t(const bf16_t* PT, const bf16_t* QT, const int32_t* pad_off, int N, int M, int ld, int E,
                           bf16_t* dW, hipStream_t s) {
   constexpr int MT = 2, WM = 2;
-  using St = Stripe<MT, NTW, WM, kBK>;
+  using St = Stripe<MT, NTW, WM, kBwdBK>;
   hipLaunchKernelGGL((wgrad_kernel<MT, NTW, WM>), dim3(N / St::BM, M / St::BN, E), dim3(256 * WM), 0, s, PT, QT, pad_off, N,
                      M, ld, dW);
   return hipGetLastError();
@@ -272,8 +301,8 @@ hipError_t launch_wgrad(const bf16_t* PT, const bf16_t* QT, const int32_t* pad_o
 // h = r^p a u, a = SiLU(z) = z s, s = sigmoid(z), z = g / r, a' = s (1 + z (1 - s)); with q = dh u:
 //   du = dh r^p a;  dg = q r^(p-1) a' + g / (I r) sum_i q_i (p r^(p-1) a_i - r^(p-2) a'_i g_i);
 //   dtheta (the row's share) = p'(theta) ln r sum_i q_i r^p a_i;  dw = <dh', h>, dh = w dh'.
-// act = SiLU: h = SiLU(g) u, dg = q a'(g), no theta.  Rows of I <= 64 * kActPer elements.
-constexpr int kActPer = 8;
+// act = SiLU: h = SiLU(g) u, dg = q a'(g), no theta.  Rows of I <= kActMaxI elements.
+constexpr int kActMaxI = 512;   // one 16-byte granule of the row per lane
 
 __global__ __launch_bounds__(256) void act_bwd_kernel(const bf16_t* __restrict__ gu, const bf16_t* __restrict__ dhp,
                                                       const float* __restrict__ w, const float* __restrict__ theta,
@@ -295,20 +324,21 @@ __global__ __launch_bounds__(256) void act_bwd_kernel(const bf16_t* __restrict__
   }
   const int slot = perm_slot[row];
   const float ws = w[slot];
-  const bf16_t* grow = gu + (size_t)row * 2 * I;
-  const bf16_t* drow = dhp + (size_t)row * I;
-  float g[kActPer], u[kActPer], d[kActPer];
+  const bool live = lane * 8 < I;
+  bf16x8 gv, uv, dv;
+#pragma unroll
+  for (int q = 0; q < 8; ++q) gv[q] = uv[q] = dv[q] = (bf16_t)0.f;
+  if (live) {
+    gv = *reinterpret_cast<const bf16x8*>(gu + (size_t)row * 2 * I + lane * 8);
+    uv = *reinterpret_cast<const bf16x8*>(gu + (size_t)row * 2 * I + I + lane * 8);
+    dv = *reinterpret_cast<const bf16x8*>(dhp + (size_t)row * I + lane * 8);
+  }
+  float g[8], u[8], d[8];
   float ss = 0.f;
 #pragma unroll
-  for (int j = 0; j < kActPer; ++j) {
-    const int i = lane + 64 * j;
-    g[j] = u[j] = d[j] = 0.f;
-    if (i < I) {
-      g[j] = (float)grow[i];
-      u[j] = (float)grow[I + i];
-      d[j] = (float)drow[i];
-      ss = fmaf(g[j], g[j], ss);
-    }
+  for (int q = 0; q < 8; ++q) {
+    g[q] = (float)gv[q]; u[q] = (float)uv[q]; d[q] = (float)dv[q];
+    ss = fmaf(g[q], g[q], ss);
   }
   ss = wave_sum(ss);
   const bool radial = act != BIBO_ACT_SILU;
@@ -319,37 +349,35 @@ __global__ __launch_bounds__(256) void act_bwd_kernel(const bf16_t* __restrict__
   }
   const float r = 1.f / rinv;
   float dot_h = 0.f, sum_qa = 0.f, inner = 0.f;
-  float a_[kActPer], ad_[kActPer];
+  float a_[8], ad_[8];
 #pragma unroll
-  for (int j = 0; j < kActPer; ++j) {
-    const float z = g[j] * rinv;
+  for (int q = 0; q < 8; ++q) {
+    const float z = g[q] * rinv;
     const float s = 1.f / (1.f + __expf(-z));
-    a_[j] = z * s;
-    ad_[j] = s * (1.f + z * (1.f - s));
-    const float h = gain * a_[j] * u[j];
-    dot_h = fmaf(d[j], h, dot_h);
-    const float q = ws * d[j] * u[j];
-    sum_qa = fmaf(q, a_[j], sum_qa);
-    // p r^(p-1) a - r^(p-2) a' g = r^p / r (p a - a' z)
-    inner = fmaf(q, gain * rinv * (p * a_[j] - ad_[j] * z), inner);
+    a_[q] = z * s;
+    ad_[q] = s * (1.f + z * (1.f - s));
+    dot_h = fmaf(d[q], gain * a_[q] * u[q], dot_h);
+    const float qq = ws * d[q] * u[q];
+    sum_qa = fmaf(qq, a_[q], sum_qa);
+    inner = fmaf(qq, gain * rinv * (p * a_[q] - ad_[q] * z), inner);    // p r^(p-1) a - r^(p-2) a' g = r^(p-1) (p a - a' z)
   }
   dot_h = wave_sum(dot_h);
   sum_qa = wave_sum(sum_qa);
   inner = wave_sum(inner);
-  bf16_t* orow = dgu + (size_t)row * 2 * I;
-  bf16_t* hrow = hidden + (size_t)row * I;
+  if (live) {
+    bf16x8 og, ou, oh;
 #pragma unroll
-  for (int j = 0; j < kActPer; ++j) {
-    const int i = lane + 64 * j;
-    if (i < I) {
-      const float dh = ws * d[j];
-      const float q = dh * u[j];
-      float dg = q * gain * rinv * ad_[j];
-      if (radial) dg = fmaf(g[j] * rinv / (float)I, inner, dg);
-      orow[i] = (bf16_t)dg;
-      orow[I + i] = (bf16_t)(dh * gain * a_[j]);
-      hrow[i] = (bf16_t)(gain * a_[j] * u[j]);
+    for (int q = 0; q < 8; ++q) {
+      const float dh = ws * d[q];
+      float dg = dh * u[q] * gain * rinv * ad_[q];
+      if (radial) dg = fmaf(g[q] * rinv / (float)I, inner, dg);
+      og[q] = (bf16_t)dg;
+      ou[q] = (bf16_t)(dh * gain * a_[q]);
+      oh[q] = (bf16_t)(gain * a_[q] * u[q]);
     }
+    *reinterpret_cast<bf16x8*>(dgu + (size_t)row * 2 * I + lane * 8) = og;
+    *reinterpret_cast<bf16x8*>(dgu + (size_t)row * 2 * I + I + lane * 8) = ou;
+    *reinterpret_cast<bf16x8*>(hidden + (size_t)row * I + lane * 8) = oh;
   }
   if (lane == 0) {
     dw_slot[slot] = dot_h;
@@ -416,24 +444,50 @@ __global__ __launch_bounds__(256) void dx_combine_kernel(const bf16_t* __restric
   *reinterpret_cast<bf16x8*>(dx + (size_t)t * H + c) = o;
 }
 
-// dW_router[e, c] = sum over the rows r of expert e of dl[slot(r)] x[token(r), c]; grid = (H / 256, E), the rows of
-// an expert in eight interleaved partial sums per thread.
-__global__ __launch_bounds__(256) void dwr_kernel(const bf16_t* __restrict__ x, const float* __restrict__ dl,
-                                                  const int32_t* __restrict__ offsets,
-                                                  const int32_t* __restrict__ perm_slot,
-                                                  const int32_t* __restrict__ perm_token, int H,
-                                                  bf16_t* __restrict__ dwr) {
-  const int e = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
-  if (c >= H) return;
-  const int lo = offsets[e], hi = offsets[e + 1];
+// dW_router[e, c] = sum over the rows r of expert e of dl[slot(r)] x[token(r), c], in two steps.  Step 1, grid =
+// (H / 256, E, kDwrSplit): block z takes the z-th of kDwrSplit equal row ranges of the expert; thread (rl = t / 32,
+// cg = t % 32) adds up rows rl, rl + 8, .. of the range for columns 8 cg .. + 8 of the block's 256, the eight partial
+// sums meet in LDS in a fixed order -> part[e][z][c] fp32.  Step 2 adds the kDwrSplit ranges in order.
+constexpr int kDwrSplit = 8;
+
+__global__ __launch_bounds__(256) void dwr_partial_kernel(const bf16_t* __restrict__ x, const float* __restrict__ dl,
+                                                          const int32_t* __restrict__ offsets,
+                                                          const int32_t* __restrict__ perm_slot,
+                                                          const int32_t* __restrict__ perm_token, int H,
+                                                          float* __restrict__ part) {
+  __shared__ float red[8][256];
+  const int e = blockIdx.y, z = blockIdx.z, cg = threadIdx.x & 31, rl = threadIdx.x >> 5;
+  const int c = blockIdx.x * 256 + cg * 8;
+  const int lo_e = offsets[e], n = offsets[e + 1] - lo_e;
+  const int per = (n + kDwrSplit - 1) / kDwrSplit;
+  const int lo = lo_e + min(z * per, n), hi = lo_e + min((z + 1) * per, n);
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  int r = lo;
-  for (; r + 8 <= hi; r += 8) {
+  if (c < H)
+    for (int r = lo + rl; r < hi; r += 8) {
+      const float d = dl[perm_slot[r]];
+      const bf16x8 v = *reinterpret_cast<const bf16x8*>(x + (size_t)perm_token[r] * H + c);
 #pragma unroll
-    for (int q = 0; q < 8; ++q) acc[q] = fmaf(dl[perm_slot[r + q]], (float)x[(size_t)perm_token[r + q] * H + c], acc[q]);
+      for (int q = 0; q < 8; ++q) acc[q] = fmaf(d, (float)v[q], acc[q]);
+    }
+#pragma unroll
+  for (int q = 0; q < 8; ++q) red[rl][cg * 8 + q] = acc[q];
+  __syncthreads();
+  const int col = blockIdx.x * 256 + threadIdx.x;
+  if (col < H) {
+    const int t = threadIdx.x;
+    part[((size_t)e * kDwrSplit + z) * H + col] =
+        ((red[0][t] + red[1][t]) + (red[2][t] + red[3][t])) + ((red[4][t] + red[5][t]) + (red[6][t] + red[7][t]));
   }
-  for (; r < hi; ++r) acc[0] = fmaf(dl[perm_slot[r]], (float)x[(size_t)perm_token[r] * H + c], acc[0]);
-  dwr[(size_t)e * H + c] = (bf16_t)(((acc[0] + acc[1]) + (acc[2] + acc[3])) + ((acc[4] + acc[5]) + (acc[6] + acc[7])));
+}
+
+__global__ __launch_bounds__(256) void dwr_sum_kernel(const float* __restrict__ part, int H, int n, bf16_t* __restrict__ dwr) {
+  const int i = blockIdx.x * 256 + threadIdx.x;                 // element of [E, H]
+  if (i >= n) return;
+  const int e = i / H, c = i - e * H;
+  float acc = 0.f;
+#pragma unroll
+  for (int z = 0; z < kDwrSplit; ++z) acc += part[((size_t)e * kDwrSplit + z) * H + c];
+  dwr[i] = (bf16_t)acc;
 }
 
 // zero n 4-byte words (a kernel rather than a memset node, so that the call can be captured into a graph)
@@ -451,16 +505,18 @@ void zero_bytes(void* p, size_t bytes, hipStream_t s) {          // bytes is a m
 }  // namespace
 
 bool backward_supported(int H, int I, int k, int dtype) {
-  return dtype == BIBO_DTYPE_BF16 && H >= 128 && H % 128 == 0 && I >= 128 && I % 128 == 0 && I <= 64 * kActPer &&
+  return dtype == BIBO_DTYPE_BF16 && H >= 128 && H % 128 == 0 && I >= 128 && I % 128 == 0 && I <= kActMaxI &&
          k <= kMaxK;
 }
+
+int backward_dwr_split() { return kDwrSplit; }
 
 // leading dimension of the transposed activation buffers: every expert's rows padded to a multiple of kPad
 size_t backward_padded_rows(int T, int E, int k) { return ((size_t)T * k + (size_t)E * (kPad - 1) + kPad - 1) / kPad * kPad; }
 
 // The launches after routing and permutation.  Buffers (bf16 unless noted): wd_t [E,I,H], wgu_t [E,H,2I], gu [S,2I],
 // dhp [S,I], dgu [S,2I], hidden [S,I], dxs [S,H], p_t [max(H,2I), ld], q_t [max(H,I), ld], dw_slot [S] f32,
-// dl [S] f32, dtheta_row [S] f32, pad_off [E+1] i32.
+// dl [S] f32, dtheta_row [S] f32, dwr_part [E, backward_dwr_split(), H] f32, pad_off [E+1] i32.
 hipError_t launch_backward(const void* x, const void* d_out, const void* w_router, const void* wgu, const void* wd,
                            const float* theta, const float* logits, const int32_t* idx, const float* w,
                            const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token, int T, int H, int E,
@@ -509,7 +565,9 @@ hipError_t launch_backward(const void* x, const void* d_out, const void* w_route
                      b.dl);
   hipLaunchKernelGGL(dx_combine_kernel, dim3((unsigned)(((long long)T * (H / 8) + 255) / 256)), dim3(256), 0, s, dxs, b.dl, idx,
                      wrp, T, H, k, static_cast<bf16_t*>(dx));
-  hipLaunchKernelGGL(dwr_kernel, dim3((H + 255) / 256, E), dim3(256), 0, s, xp, b.dl, offsets, perm_slot, perm_token, H,
+  hipLaunchKernelGGL(dwr_partial_kernel, dim3((H + 255) / 256, E, kDwrSplit), dim3(256), 0, s, xp, b.dl, offsets, perm_slot,
+                     perm_token, H, b.dwr_part);
+  hipLaunchKernelGGL(dwr_sum_kernel, dim3((E * H + 255) / 256), dim3(256), 0, s, b.dwr_part, H, E * H,
                      static_cast<bf16_t*>(d_w_router));
   // weight gradients: dW_down[e] = (w d)^T h, dW_gate_up[e] = [dg, du]^T x, contracted over the expert's rows
   const dim3 tgrid_h(ld / 64, H / 64), tgrid_i(ld / 64, I / 64), tgrid_2i(ld / 64, 2 * I / 64);

@@ -183,10 +183,12 @@ hipError_t launch_down_stream(const void* gu, const void* wd, const float* theta
 struct BackwardBuffers {
   void *wd_t, *wgu_t, *gu, *dhp, *dgu, *hidden, *dxs, *p_t, *q_t;   // bf16 device buffers, sizes in launch_backward's comment
   float *dw_slot, *dl, *dtheta_row;                                 // [T*k] each
+  float* dwr_part;                                                  // [E, backward_dwr_split(), H]
   int32_t* pad_off;                                                 // [E + 1]
 };
 bool backward_supported(int H, int I, int k, int dtype);
 size_t backward_padded_rows(int T, int E, int k);
+int backward_dwr_split();
 hipError_t launch_backward(const void* x, const void* d_out, const void* w_router, const void* wgu, const void* wd,
                            const float* theta, const float* logits, const int32_t* idx, const float* w,
                            const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token, int T, int H, int E,
