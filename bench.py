@@ -263,6 +263,33 @@ def side_workload(name, dev, algo, steps, warmup):
             "parity_rel_err_sample": rel}
 
 
+def backward_pass(lay, steps, warmup):
+    """The layer's backward (bibo_moe_backward) on the headline workload, next to its forward: us/step and algorithmic
+    TFLOP/s (twice the forward's contraction flops: one GEMM per operand gradient; what the call recomputes does not
+    count)."""
+    import torch
+    from bibo_amd import ops
+    g = torch.Generator(device=lay.dev).manual_seed(9)
+    d_out = torch.randn(lay.T, lay.H, device=lay.dev, generator=g).to(torch.bfloat16)
+    args = (lay.x, d_out, lay.wr, lay.bias, lay.wgu, lay.wd, lay.theta, lay.k)
+    for _ in range(max(2, warmup // 4)):
+        grads = ops.moe_backward(*args)
+    runs = []
+    n = max(5, steps // 10)
+    for _ in range(3):
+        torch.cuda.synchronize(lay.dev)
+        t0 = time.perf_counter()
+        for _ in range(n):
+            grads = ops.moe_backward(*args)
+        torch.cuda.synchronize(lay.dev)
+        runs.append((time.perf_counter() - t0) / n)
+    sec = sorted(runs)[1]
+    fl = 2.0 * flops_layer(lay.T, lay.H, lay.E, lay.k, lay.I)
+    return {"entry": "bibo_moe_backward: d_x, d_w_router, d_w_gate_up, d_w_down, d_theta from d_out", "us_per_step": sec * 1e6,
+            "steps_timed": n, "tflops": fl / sec / 1e12, "pct_bf16_mfma_peak": 100.0 * fl / sec / 1e12 / PEAK_BF16_TFLOPS,
+            "gradients_finite": all(bool(torch.isfinite(t.float()).all()) for t in grads[:5])}
+
+
 def full_model(dev, batch=8, seq=2048, steps=10, warmup=3):
     """Config 5: the 10-layer experimental forward (HIP MoE block in layers 1-8, dense SwiGLU in 0 and 9, hybrid
     global / window-128 attention, Block Attention Residuals, tied 32000-token head), bf16, random init, uniform
@@ -305,6 +332,10 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true")
     ap.add_argument("--no-model", action="store_true", help="skip the 10-layer forward (c5)")
+    ap.add_argument("--no-side", action="store_true", help="skip the c1 / c4 lines, the seam and the backward pass")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="only copy 256 MiB device to device a few times: the known-size kernel the FETCH_SIZE / WRITE_SIZE "
+                         "counters of a profile are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -316,6 +347,14 @@ def main():
         __graft_entry__.build()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.calibrate_copy:
+        src = torch.full((256 << 20,), 3, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize(dev)
+        print(json.dumps({"calibrate_copy_bytes": src.numel(), "copies": 5}))
+        return
 
     layer = Layer(args.workload, dev, args.algo)
     rel, e_active = layer.check()
@@ -353,9 +392,12 @@ def main():
                            "bound": "hbm", "achieved": nbytes / rsec / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                            "frac": nbytes / rsec / 1e9 / PEAK_HBM_GBS, "traffic": measured_traffic(args.workload, "stream")}
         out["stage_us"] = {n: v for n, v in out["stage_us"].items() if n in ("router", "permute")}
-    ffn_sec = layer.time_ffn_seam(args.steps, args.warmup)
-    out["ffn_seam"] = {"entry": "bibo_moe_ffn_forward: out = h + moe(rmsnorm(h))", "us_per_step": ffn_sec * 1e6,
-                       "extra_us_over_layer": (ffn_sec - sec) * 1e6}
+    if not args.no_side:
+        ffn_sec = layer.time_ffn_seam(args.steps, args.warmup)
+        out["ffn_seam"] = {"entry": "bibo_moe_ffn_forward: out = h + moe(rmsnorm(h))", "us_per_step": ffn_sec * 1e6,
+                           "extra_us_over_layer": (ffn_sec - sec) * 1e6}
+        if args.workload == "c2":
+            out["backward"] = backward_pass(layer, args.steps, args.warmup)
     if not args.no_decode and args.workload == "c2":
         d = Layer("c3", dev, args.algo)
         drel, dact = d.check()
@@ -373,8 +415,9 @@ def main():
                          "note": "whole layer through bibo_moe_forward (weight-streaming kernels); hbm_gbs rotates the "
                                  "expert weights over 4 separately allocated sets (805 MB, more than the 256 MB Infinity "
                                  "Cache) so every step streams them from HBM; cache_warm re-reads one 201 MB set"}
-        out["c1"] = side_workload("c1", dev, args.algo, args.steps, args.warmup)
-        out["c4"] = side_workload("c4", dev, args.algo, max(10, args.steps // 2), args.warmup)
+        if not args.no_side:
+            out["c1"] = side_workload("c1", dev, args.algo, args.steps, args.warmup)
+            out["c4"] = side_workload("c4", dev, args.algo, max(10, args.steps // 2), args.warmup)
         if not args.no_model:
             out["c5"] = full_model(dev)
     if not args.no_cpu_baseline:
