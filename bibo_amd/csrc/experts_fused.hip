@@ -272,10 +272,23 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
     w_s[tid] = w[slot];
   }
   __syncthreads();
+  // phase 3 streams w_down through registers; its first K blocks are requested here, between the two M tiles of
+  // the activation: the accumulators of the first tile are dead by then and make room, and the loads fly during
+  // the rest of the activation arithmetic
+  constexpr int KB = I / 64;                 // 128-byte K blocks
+  const size_t tile_stride = (size_t)16 * I;
+  const bf16_t* wp = wd + ((size_t)e * H + wave * (16 * CT) + (lane >> 2)) * I + (lane & 3) * 8;
+  constexpr int D = KB > 3 ? 3 : KB - 1;      // K blocks requested ahead of the one being multiplied
+  constexpr int NB = D + 1;
+  WBlock<CT> wb[NB];
   {
     // stage t holds activation columns [128t, 128t + 128) of all 128 rows, [128][128], granules swizzled
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
+      if (mt == MT - 1) {
+#pragma unroll
+        for (int d = 0; d < D; ++d) load_wblock<CT>(wb[d], wp, tile_stride, d);
+      }
       const int m = mbase + mt * 32 + n;
       const float rinv = rinv_s[m];
       const float nrl = -1.44269504f * rinv, rg = rinv * gain_s[m];            // per-row constants folded once
@@ -301,17 +314,9 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
   __syncthreads();                         // the activation tile is complete
 
   // ---- phase 3: down projection, routing weight, scatter to slot order (moe.py:92-93) ----
-  constexpr int KB = I / 64;                 // 128-byte K blocks
   const int r16 = lane & 15, g4 = lane >> 4;
-  const size_t tile_stride = (size_t)16 * I;
   const int nblk = H / F::BN2;
-  const bf16_t* wp = wd + ((size_t)e * H + wave * (16 * CT) + (lane >> 2)) * I + (lane & 3) * 8;
   const int sel = 4 * (4 * r16 + g4);
-  constexpr int D = KB > 3 ? 3 : KB - 1;      // K blocks requested ahead of the one being multiplied
-  constexpr int NB = D + 1;
-  WBlock<CT> wb[NB];
-#pragma unroll
-  for (int d = 0; d < D; ++d) load_wblock<CT>(wb[d], wp, tile_stride, d);
   for (int nb = 0; nb < nblk; ++nb) {
     const int n0 = nb * F::BN2;
     floatx4 acc2[CT][8];
