@@ -575,4 +575,20 @@ int bibo_moe_backward(const void* x, const void* d_out, const void* w_router, co
                                 T, H, E, k, I, norm_mode, sh->act, b, d_x, d_w_router, d_w_gate_up, d_w_down, d_theta, s));
 }
 
+int bibo_moe_exp_attn_res_fwd(const void* const* candidates, int n_candidates, const float* score_weight, float eps, int T, int H,
+                          int dtype, void* out, void* stream) {
+  const int rc = check_dims(T, H, 1, 1, 1, dtype);
+  if (rc != BIBO_OK) return rc;
+  if (!attn_res_supported(H, n_candidates, dtype)) return BIBO_ERR_UNSUPPORTED;
+  if (!candidates || !score_weight) return BIBO_ERR_NULL_POINTER;
+  if (T == 0) return BIBO_OK;
+  if (!out) return BIBO_ERR_NULL_POINTER;
+  for (int i = 0; i < n_candidates; ++i) {
+    if (!candidates[i]) return BIBO_ERR_NULL_POINTER;
+    if (!aligned16(candidates[i])) return BIBO_ERR_MISALIGNED;
+  }
+  if (!aligned16(out)) return BIBO_ERR_MISALIGNED;
+  return hip_rc(launch_attn_res(candidates, n_candidates, score_weight, eps, T, H, out, static_cast<hipStream_t>(stream)));
+}
+
 }  // extern "C"

@@ -179,6 +179,10 @@ hipError_t launch_gateup_stream(const void* x, const void* wgu, const int32_t* i
 hipError_t launch_down_stream(const void* gu, const void* wd, const float* theta, const float* w, const int32_t* idx,
                               int T, int H, int E, int k, int I, int act, void* hidden, float* yw, hipStream_t s);
 
+bool attn_res_supported(int H, int n_cand, int dtype);
+hipError_t launch_attn_res(const void* const* cands, int n_cand, const float* score_w, float eps, int T, int H, void* out,
+                           hipStream_t s);
+
 // ---- backward pass (backward.hip) ----
 struct BackwardBuffers {
   void *wd_t, *wgu_t, *gu, *dhp, *dgu, *hidden, *dxs, *p_t, *q_t;   // bf16 device buffers, sizes in launch_backward's comment

@@ -78,7 +78,99 @@ __global__ __launch_bounds__(256) void rmsnorm_bf16x8_kernel(const bf16_t* __res
   }
 }
 
+// Depth mix of Block Attention Residuals (apply_attention_residual, exp/modeling_bibo.py:119-232, softmax scores,
+// dense): candidates = the completed block representatives and the running prefix sum of a token; score of a
+// candidate = rsqrt(mean(c^2) + eps) * <c, score_w> with score_w = norm weight * pseudo-query (fp32); out = the
+// candidates averaged with the softmax of their scores, fp32, rounded once.  One wave per token, the candidates' rows
+// stay in registers (two 16-byte granules per lane: H <= 1024).
+constexpr int kAttnResMaxCand = 8;
+struct AttnResPtrs {
+  const bf16_t* c[kAttnResMaxCand];
+};
+
+__global__ __launch_bounds__(256) void attn_res_kernel(AttnResPtrs cand, int n_cand, const float* __restrict__ score_w,
+                                                       float eps, int T, int H, bf16_t* __restrict__ out) {
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (row >= T) return;
+  const int nchunk = H / 8;
+  float sw[2][8];
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int c = u * kWave + lane;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) sw[u][q] = c < nchunk ? score_w[c * 8 + q] : 0.f;
+  }
+  bf16x8 v[kAttnResMaxCand][2];
+  float score[kAttnResMaxCand];
+  float mx = -3.0e38f;
+#pragma unroll
+  for (int i = 0; i < kAttnResMaxCand; ++i)
+    if (i < n_cand) {
+      const bf16x8* r = reinterpret_cast<const bf16x8*>(cand.c[i] + (size_t)row * H);
+      float ss = 0.f, dot = 0.f;
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int c = u * kWave + lane;
+        if (c < nchunk) {
+          v[i][u] = r[c];
+#pragma unroll
+          for (int q = 0; q < 8; ++q) {
+            const float f = (float)v[i][u][q];
+            ss = fmaf(f, f, ss);
+            dot = fmaf(f, sw[u][q], dot);
+          }
+        }
+      }
+      ss = wave_sum(ss);
+      dot = wave_sum(dot);
+      score[i] = dot * rsqrtf(ss / (float)H + eps);
+      mx = fmaxf(mx, score[i]);
+    }
+  float den = 0.f;
+#pragma unroll
+  for (int i = 0; i < kAttnResMaxCand; ++i)
+    if (i < n_cand) {
+      score[i] = __expf(score[i] - mx);
+      den += score[i];
+    }
+  const float inv = 1.f / den;
+  bf16x8* orow = reinterpret_cast<bf16x8*>(out + (size_t)row * H);
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int c = u * kWave + lane;
+    if (c < nchunk) {
+      float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int i = 0; i < kAttnResMaxCand; ++i)
+        if (i < n_cand) {
+          const float pr = score[i] * inv;
+#pragma unroll
+          for (int q = 0; q < 8; ++q) acc[q] = fmaf(pr, (float)v[i][u][q], acc[q]);
+        }
+      bf16x8 o;
+#pragma unroll
+      for (int q = 0; q < 8; ++q) o[q] = (bf16_t)acc[q];
+      orow[c] = o;
+    }
+  }
+}
+
 }  // namespace
+
+bool attn_res_supported(int H, int n_cand, int dtype) {
+  return dtype == BIBO_DTYPE_BF16 && H % 8 == 0 && H <= 1024 && n_cand >= 1 && n_cand <= kAttnResMaxCand;
+}
+
+hipError_t launch_attn_res(const void* const* cands, int n_cand, const float* score_w, float eps, int T, int H, void* out,
+                           hipStream_t s) {
+  if (T == 0) return hipSuccess;
+  AttnResPtrs p;
+  for (int i = 0; i < kAttnResMaxCand; ++i) p.c[i] = static_cast<const bf16_t*>(i < n_cand ? cands[i] : cands[0]);
+  hipLaunchKernelGGL(attn_res_kernel, dim3((T + 3) / 4), dim3(256), 0, s, p, n_cand, score_w, eps, T, H,
+                     static_cast<bf16_t*>(out));
+  return hipGetLastError();
+}
 
 hipError_t launch_rmsnorm(const void* x, const float* weight, float eps, int T, int H, int dtype, void* out,
                           hipStream_t s) {

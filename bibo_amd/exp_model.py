@@ -20,6 +20,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .config import BiBoMoEConfig
+from . import ops
 from .moe import BiBoMoELayer
 
 __all__ = ["BiBoExpConfig", "BiBoExpForCausalLM"]
@@ -81,8 +82,28 @@ class RMSNorm(nn.Module):
         self.variance_epsilon = eps
 
     def forward(self, x):
+        if _hip_ok(x) and x.shape[-1] % 8 == 0:
+            # the library's row norm (bibo_moe_rmsnorm_fwd): the same arithmetic in one launch
+            w32 = _fp32_copy(self, "weight")
+            return ops.rmsnorm_fwd(x.reshape(-1, x.shape[-1]).contiguous(), w32, float(self.variance_epsilon)).view(x.shape)
         xf = x.float()
         return self.weight * (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.variance_epsilon)).to(x.dtype)
+
+
+def _hip_ok(x) -> bool:
+    """bf16 on the GPU with no autograd graph to build: the cases the library's caller-side kernels serve."""
+    return x.is_cuda and x.dtype == torch.bfloat16 and not (torch.is_grad_enabled() and x.requires_grad)
+
+
+def _fp32_copy(module, name):
+    """fp32 copy of a small parameter, refreshed when the parameter changes (storage address or version counter)."""
+    p = getattr(module, name)
+    tag = (p.data_ptr(), p._version, p.device)
+    hit = module.__dict__.get("_fp32_" + name)
+    if hit is None or hit[0] != tag:
+        hit = (tag, p.detach().float().contiguous())
+        module.__dict__["_fp32_" + name] = hit
+    return hit[1]
 
 
 def _rotate_half(x):
@@ -94,6 +115,9 @@ def attention_residual(prefix, blocks, proj_w, norm_w, eps):
     """apply_attention_residual (exp/modeling_bibo.py:119-232): fp32 scores `inv_rms * (v . (norm_w * proj_w))` per
     candidate, softmax over the candidates, fp32 weighted sum, result in prefix's dtype.  blocks: list of [T,H]."""
     sw = norm_w.float() * proj_w.reshape(-1).float()
+    if (_hip_ok(prefix) and prefix.shape[-1] % 8 == 0 and prefix.shape[-1] <= 1024 and len(blocks) < 8
+            and not (torch.is_grad_enabled() and (norm_w.requires_grad or proj_w.requires_grad))):
+        return ops.attn_res_fwd([b.contiguous() for b in blocks] + [prefix.contiguous()], sw.contiguous(), float(eps))
     cands = [b.float() for b in blocks] + [prefix.float()]
     scores = torch.stack([(c @ sw) * torch.rsqrt(c.pow(2).mean(-1) + eps) for c in cands], dim=-1)
     prob = scores.softmax(-1)

@@ -316,6 +316,23 @@ def moe_backward(x, d_out, w_router, bias, w_gate_up, w_down, theta, k, norm="su
     return d_x, d_wr, d_gu, d_dn, d_theta, d_w
 
 
+def attn_res_fwd(candidates, score_weight, eps):
+    """bibo_moe_exp_attn_res_fwd: softmax-weighted average of the candidate rows, scores rsqrt(mean c^2 + eps) <c, score_weight>
+    (apply_attention_residual, exp/modeling_bibo.py:119-232).  candidates: list of [T,H] bf16; score_weight fp32 [H]."""
+    T, H = candidates[0].shape
+    for c in candidates:
+        _chk(c, "candidate", torch.bfloat16, (T, H))
+    _chk(score_weight, "score_weight", torch.float32, (H,))
+    out = torch.empty_like(candidates[0])
+    arr = (ctypes.c_void_p * len(candidates))(*[c.data_ptr() for c in candidates])
+    dev = out.device
+    with torch.cuda.device(dev):
+        L.check(L.lib().bibo_moe_exp_attn_res_fwd(ctypes.cast(arr, ctypes.c_void_p), len(candidates), _ptr(score_weight),
+                                              ctypes.c_float(eps), T, H, _dtype_code(out), _ptr(out), _stream(dev)),
+                "bibo_moe_exp_attn_res_fwd")
+    return out
+
+
 def rmsnorm_fwd(x, norm_weight, eps):
     """out = norm_weight * round(x * rsqrt(mean(x^2) + eps)) in x.dtype (the block's input norm, norm.py:19-24)."""
     T, H = x.shape

@@ -281,6 +281,19 @@ int bibo_moe_backward(const void* x, const void* d_out, const void* w_router, co
                       void* d_w_router, void* d_w_gate_up, void* d_w_down, float* d_theta, float* d_w_out,
                       void* workspace, size_t workspace_bytes, void* stream);
 
+/*
+ * Depth mix of the experimental model's Block Attention Residuals: apply_attention_residual
+ * (exp/modeling_bibo.py:119-232; softmax scores, dense), the operation the reference hands to its optional external
+ * kernel `kernels.sm120.attn_res.attn_res(block_residual, prefix, score_weight, eps, ...)` (exp/modeling_bibo.py:44,
+ * 188-190).  candidates: host array of n_candidates device pointers to [T,H] rows (the completed block
+ * representatives, then the running prefix sum); score_weight fp32 [H] = norm weight * pseudo-query;
+ *   score_c = rsqrt(mean(c^2) + eps) * <c, score_weight>,  out = sum_c softmax(score)_c * c   (fp32, rounded once).
+ * bf16, H % 8 == 0, H <= 1024, 1 <= n_candidates <= 8 (BIBO_ERR_UNSUPPORTED otherwise).  Not part of the MoE block:
+ * a caller-side kernel of the 10-layer forward the block sits in.
+ */
+int bibo_moe_exp_attn_res_fwd(const void* const* candidates, int n_candidates, const float* score_weight, float eps, int T, int H,
+                          int dtype, void* out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -237,3 +237,30 @@ def test_model_with_hip_moe_layers_matches_the_oracle(dtype, tol):
     sd = {k: v.detach().cpu() for k, v in model.state_dict().items()}
     ref = XO.forward(ids, sd, cfg, dtype=torch.float32, routing=routing)
     assert torch.isfinite(logits).all() and rel_err(logits.cpu(), ref) <= tol
+
+
+@pytest.mark.gpu
+def test_hip_depth_mix_and_row_norm_match_the_stock_operations():
+    """The two caller-side kernels of the 10-layer forward against the tensor-operation versions they replace:
+    bibo_moe_exp_attn_res_fwd (depth mix, 1 to 5 candidates) and bibo_moe_rmsnorm_fwd on head-sized rows."""
+    from bibo_amd import exp_model as X
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(8)
+    T, H = 1000, 768
+    rows = [(torch.randn(T, H, generator=g) * (1 + i)).to(torch.bfloat16).to(dev) for i in range(5)]
+    proj = torch.randn(1, H, generator=g).to(dev) * 0.2
+    nw = (1 + 0.1 * torch.randn(H, generator=g)).to(dev)
+    for n in range(0, 5):
+        blocks, prefix = rows[:n], rows[4]
+        got = X.attention_residual(prefix, blocks, proj, nw, 1e-6)                       # HIP kernel
+        with torch.enable_grad():                                                        # the tensor-operation path
+            ref = X.attention_residual(prefix.clone().requires_grad_(True), blocks, proj, nw, 1e-6).detach()
+        assert float((got.float() - ref.float()).abs().max()) <= 2e-2 * float(ref.float().abs().max())
+    x = torch.randn(4, 50, 4, 192, generator=g).to(torch.bfloat16).to(dev)
+    norm = X.RMSNorm(192, 1e-6).to(dev).to(torch.bfloat16)
+    with torch.no_grad():
+        norm.weight.copy_((1 + 0.1 * torch.randn(192, generator=g)).to(torch.bfloat16))
+    got = norm(x)
+    with torch.enable_grad():
+        ref = norm(x.clone().requires_grad_(True)).detach()
+    assert got.shape == x.shape and float((got.float() - ref.float()).abs().max()) <= 1e-2 * float(ref.float().abs().max())
