@@ -318,8 +318,9 @@ def full_model(dev, batch=8, seq=2048, steps=10, warmup=3):
                         f"window 128 on [G,S,S], AttnRes block 3, E=64 k=6 I=384 in {n_moe} MoE layers, vocab 32000, bf16",
             "tokens_per_s": batch * seq / sec, "ms_per_forward": sec * 1e3, "ms_per_forward_runs": [r * 1e3 for r in runs],
             "logits_finite": finite, "params": sum(p.numel() for p in model.parameters()),
-            "note": "HIP MoE block per layer through bibo_moe_ffn_forward (norm + block + residual in one call); attention, "
-                    "depth mixes, dense layers and the head are stock PyTorch-ROCm operations"}
+            "note": "HIP MoE block per layer through bibo_moe_ffn_forward (norm + block + residual in one call), HIP depth "
+                    "mix (bibo_moe_exp_attn_res_fwd) and row norms (bibo_moe_rmsnorm_fwd); attention, dense layers and the "
+                    "head are stock PyTorch-ROCm operations"}
 
 
 def main():
