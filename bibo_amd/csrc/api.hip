@@ -575,6 +575,43 @@ int bibo_moe_backward(const void* x, const void* d_out, const void* w_router, co
                                 T, H, E, k, I, norm_mode, sh->act, b, d_x, d_w_router, d_w_gate_up, d_w_down, d_theta, s));
 }
 
+int bibo_moe_experts_backward(const void* x, const void* d_out, const int32_t* idx, const float* w, const void* w_gate_up,
+                              const void* w_down, const float* theta, const bibo_moe_shape* sh, void* d_x, float* d_w,
+                              void* d_w_gate_up, void* d_w_down, float* d_theta, void* workspace, size_t workspace_bytes,
+                              void* stream) {
+  int rc = backward_check(sh, BIBO_NORM_SUM);
+  if (rc != BIBO_OK) return rc;
+  const int T = sh->T, H = sh->H, E = sh->E, k = sh->k, I = sh->I;
+  if (!workspace) return BIBO_ERR_NULL_POINTER;
+  if (!aligned_ws(workspace)) return BIBO_ERR_MISALIGNED;
+  if (!d_w_gate_up || !d_w_down || !d_theta) return BIBO_ERR_NULL_POINTER;
+  if (T > 0 && (!x || !d_out || !idx || !w || !w_gate_up || !w_down || !d_x || !d_w)) return BIBO_ERR_NULL_POINTER;
+  if (T > 0 && !theta && sh->act != BIBO_ACT_SILU) return BIBO_ERR_NULL_POINTER;
+  if (!aligned16(x) || !aligned16(d_out) || !aligned16(w_gate_up) || !aligned16(w_down) || !aligned16(d_x) ||
+      !aligned16(d_w_gate_up) || !aligned16(d_w_down))
+    return BIBO_ERR_MISALIGNED;
+  const BackwardWorkspace ws = carve_backward(T, H, E, k, I);
+  if (workspace_bytes < ws.total) return BIBO_ERR_WORKSPACE_TOO_SMALL;
+  char* base = static_cast<char*>(workspace);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  int32_t* counts = reinterpret_cast<int32_t*>(base + ws.counts);
+  int32_t* offsets = reinterpret_cast<int32_t*>(base + ws.offsets);
+  int32_t* perm_slot = reinterpret_cast<int32_t*>(base + ws.perm_slot);
+  int32_t* perm_token = reinterpret_cast<int32_t*>(base + ws.perm_token);
+  if ((rc = hip_rc(launch_permute(idx, T, E, k, counts, offsets, perm_slot, perm_token, base + ws.hist, s))) != BIBO_OK)
+    return rc;
+  BackwardBuffers b;
+  b.wd_t = base + ws.wd_t; b.wgu_t = base + ws.wgu_t; b.gu = base + ws.gu; b.dhp = base + ws.dhp; b.dgu = base + ws.dgu;
+  b.hidden = base + ws.hidden; b.dxs = base + ws.dxs; b.p_t = base + ws.p_t; b.q_t = base + ws.q_t;
+  b.dw_slot = d_w;
+  b.dl = reinterpret_cast<float*>(base + ws.dl);
+  b.dtheta_row = reinterpret_cast<float*>(base + ws.dtheta_row);
+  b.dwr_part = reinterpret_cast<float*>(base + ws.dwr_part);
+  b.pad_off = reinterpret_cast<int32_t*>(base + ws.pad_off);
+  return hip_rc(launch_backward(x, d_out, nullptr, w_gate_up, w_down, theta, nullptr, idx, w, offsets, perm_slot, perm_token,
+                                T, H, E, k, I, BIBO_NORM_SUM, sh->act, b, d_x, nullptr, d_w_gate_up, d_w_down, d_theta, s));
+}
+
 int bibo_moe_exp_attn_res_fwd(const void* const* candidates, int n_candidates, const float* score_weight, float eps, int T, int H,
                           int dtype, void* out, void* stream) {
   const int rc = check_dims(T, H, 1, 1, 1, dtype);

@@ -421,7 +421,8 @@ __global__ void router_bwd_kernel(const float* __restrict__ logits, const int32_
   }
 }
 
-// dx[t, c] = sum_j dxs[t k + j, c] + sum_j dl[t, j] W_router[idx[t, j], c]; one thread per 8 columns.
+// dx[t, c] = sum_j dxs[t k + j, c] + sum_j dl[t, j] W_router[idx[t, j], c]; one thread per 8 columns.  dl == NULL: the
+// slot rows alone (the experts without their router).
 __global__ __launch_bounds__(256) void dx_combine_kernel(const bf16_t* __restrict__ dxs, const float* __restrict__ dl,
                                                          const int32_t* __restrict__ idx,
                                                          const bf16_t* __restrict__ w_router, int T, int H, int k,
@@ -433,10 +434,15 @@ __global__ __launch_bounds__(256) void dx_combine_kernel(const bf16_t* __restric
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   for (int j = 0; j < k; ++j) {
     const bf16x8 v = *reinterpret_cast<const bf16x8*>(dxs + ((size_t)t * k + j) * H + c);
-    const bf16x8 r = *reinterpret_cast<const bf16x8*>(w_router + (size_t)idx[t * k + j] * H + c);
-    const float d = dl[t * k + j];
+    if (dl != nullptr) {
+      const bf16x8 r = *reinterpret_cast<const bf16x8*>(w_router + (size_t)idx[t * k + j] * H + c);
+      const float d = dl[t * k + j];
 #pragma unroll
-    for (int q = 0; q < 8; ++q) acc[q] += (float)v[q] + d * (float)r[q];
+      for (int q = 0; q < 8; ++q) acc[q] += (float)v[q] + d * (float)r[q];
+    } else {
+#pragma unroll
+      for (int q = 0; q < 8; ++q) acc[q] += (float)v[q];
+    }
   }
   bf16x8 o;
 #pragma unroll
@@ -539,7 +545,7 @@ hipError_t launch_backward(const void* x, const void* d_out, const void* w_route
   hipError_t err = hipSuccess;
   if (S == 0) {
     zero_bytes(d_theta, (size_t)E * sizeof(float), s);
-    zero_bytes(d_w_router, (size_t)E * H * sizeof(bf16_t), s);
+    if (d_w_router != nullptr) zero_bytes(d_w_router, (size_t)E * H * sizeof(bf16_t), s);
     zero_bytes(d_wgu, (size_t)E * 2 * I * H * sizeof(bf16_t), s);
     zero_bytes(d_wd, (size_t)E * H * I * sizeof(bf16_t), s);
     return hipGetLastError();
@@ -561,14 +567,18 @@ hipError_t launch_backward(const void* x, const void* d_out, const void* w_route
   // dx of every slot, in slot order: [dg, du] W_gate_up
   err = launch_ggemm<false, true>(dgu, nullptr, wgu_t, offsets, perm_slot, S, 2 * I, H, E, dxs, s);
   if (err != hipSuccess) return err;
-  hipLaunchKernelGGL(router_bwd_kernel, dim3((T + 255) / 256), dim3(256), 0, s, logits, idx, w, b.dw_slot, T, E, k, norm_mode,
-                     b.dl);
-  hipLaunchKernelGGL(dx_combine_kernel, dim3((unsigned)(((long long)T * (H / 8) + 255) / 256)), dim3(256), 0, s, dxs, b.dl, idx,
-                     wrp, T, H, k, static_cast<bf16_t*>(dx));
-  hipLaunchKernelGGL(dwr_partial_kernel, dim3((H + 255) / 256, E, kDwrSplit), dim3(256), 0, s, xp, b.dl, offsets, perm_slot,
-                     perm_token, H, b.dwr_part);
-  hipLaunchKernelGGL(dwr_sum_kernel, dim3((E * H + 255) / 256), dim3(256), 0, s, b.dwr_part, H, E * H,
-                     static_cast<bf16_t*>(d_w_router));
+  const bool with_router = w_router != nullptr;      // else: the experts alone, the caller owns the routing
+  if (with_router)
+    hipLaunchKernelGGL(router_bwd_kernel, dim3((T + 255) / 256), dim3(256), 0, s, logits, idx, w, b.dw_slot, T, E, k, norm_mode,
+                       b.dl);
+  hipLaunchKernelGGL(dx_combine_kernel, dim3((unsigned)(((long long)T * (H / 8) + 255) / 256)), dim3(256), 0, s, dxs,
+                     with_router ? b.dl : nullptr, idx, wrp, T, H, k, static_cast<bf16_t*>(dx));
+  if (with_router) {
+    hipLaunchKernelGGL(dwr_partial_kernel, dim3((H + 255) / 256, E, kDwrSplit), dim3(256), 0, s, xp, b.dl, offsets, perm_slot,
+                       perm_token, H, b.dwr_part);
+    hipLaunchKernelGGL(dwr_sum_kernel, dim3((E * H + 255) / 256), dim3(256), 0, s, b.dwr_part, H, E * H,
+                       static_cast<bf16_t*>(d_w_router));
+  }
   // weight gradients: dW_down[e] = (w d)^T h, dW_gate_up[e] = [dg, du]^T x, contracted over the expert's rows
   const dim3 tgrid_h(ld / 64, H / 64), tgrid_i(ld / 64, I / 64), tgrid_2i(ld / 64, 2 * I / 64);
   hipLaunchKernelGGL(transpose_rows_kernel, tgrid_h, dim3(256), 0, s, dop, perm_token, w, perm_slot, offsets, b.pad_off, E, H,

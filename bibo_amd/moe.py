@@ -3,8 +3,9 @@
 Class names, constructor argument, attribute names, parameter shapes and state_dict keys follow
 src/modeling/ffn/router.py and src/modeling/ffn/moe.py of the reference, so a reference checkpoint
 loads with strict=True and code that pokes at `layer.gate.bias` or `layer.experts.radial_theta`
-keeps working.  `BiBoMoELayer.forward` is differentiable (its backward is the library's bibo_moe_backward) for bf16
-compute without hooks; `BiBoMoERouter` and `BiBoFusedExperts` called on their own are forward only."""
+keeps working.  The modules are differentiable for bf16 compute: `BiBoMoELayer.forward` is one autograd node
+(backward = bibo_moe_backward); with hooks present, or called on their own, `BiBoFusedExperts` is one node (backward =
+bibo_moe_experts_backward) and `BiBoMoERouter` returns the kernel's selection with differentiable weights."""
 from __future__ import annotations
 
 import torch
@@ -23,14 +24,6 @@ except AttributeError:                                    # older torch
 
 def _wants_grad(*tensors) -> bool:
     return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors)
-
-
-def _forward_only_guard(*tensors):
-    if _wants_grad(*tensors):
-        raise RuntimeError(
-            "this bibo_amd entry point implements the forward pass only; call it under torch.no_grad() or "
-            "torch.inference_mode() (an input or parameter requires grad and autograd is enabled, so gradients would "
-            "silently be lost).  BiBoMoELayer.forward without hooks is the differentiable path")
 
 
 class _MoELayerFn(torch.autograd.Function):
@@ -61,6 +54,37 @@ class _MoELayerFn(torch.autograd.Function):
         d = d_out.to(torch.bfloat16).contiguous()
         grads = ops.moe_backward(xb, d, wr, b, gu, dn, th, k, norm=norm, act=act)[:5]
         return tuple(g.to(dt) for g, dt in zip(grads, ctx.in_dtypes)) + (None,) * 6
+
+
+class _ExpertsFn(torch.autograd.Function):
+    """BiBoFusedExperts.forward as one autograd node for a caller-owned routing: forward = bibo_moe_experts_fwd, backward
+    = bibo_moe_experts_backward.  The gradient of the combine weights (moe.py:93) flows back to whoever made them."""
+
+    @staticmethod
+    def forward(ctx, x, top_w, w_gate_up, w_down, theta, idx, act, algo, want_counts):
+        cd = torch.bfloat16
+        cast = lambda t, d: (t if t.dtype == d else t.to(d)).contiguous()
+        xb, gu, dn = cast(x.detach(), cd), cast(w_gate_up.detach(), cd), cast(w_down.detach(), cd)
+        th, w = cast(theta.detach(), torch.float32), cast(top_w.detach(), torch.float32)
+        out, counts = ops.experts_fwd(xb, idx, w, gu, dn, th, algo=algo, want_counts=want_counts, act=act)
+        ctx.save_for_backward(xb, w, gu, dn, th, idx)
+        ctx.act = act
+        ctx.in_dtypes = (x.dtype, top_w.dtype, w_gate_up.dtype, w_down.dtype, theta.dtype)
+        if counts is None:
+            counts = torch.empty(0, dtype=torch.int32, device=x.device)
+        ctx.mark_non_differentiable(counts)
+        return out, counts
+
+    @staticmethod
+    def backward(ctx, d_out, _d_counts):
+        xb, w, gu, dn, th, idx = ctx.saved_tensors
+        grads = ops.experts_backward(xb, d_out.to(torch.bfloat16).contiguous(), idx, w, gu, dn, th, act=ctx.act)
+        return tuple(g.to(dt) for g, dt in zip(grads, ctx.in_dtypes)) + (None,) * 4
+
+
+def _backward_covers(experts) -> bool:
+    return (experts.num_pos + experts.num_neg == 0 and experts.hidden_size % 128 == 0
+            and experts.intermediate_size % 128 == 0 and experts.intermediate_size <= 512)
 
 
 class _CastCache:
@@ -142,14 +166,23 @@ class BiBoMoERouter(nn.Module):
 
     @_no_compile
     def forward(self, hidden_states: torch.Tensor):
-        _forward_only_guard(hidden_states, self.gate_proj.weight)
         bsz, seq, _ = hidden_states.shape
         x, w, b = self._operands(hidden_states)
         probe = self._probe_gap and self.top_k < self.num_routed_experts
         idx, wgt, _, gap = ops.router_fwd(x, w, b, self.top_k, self.norm_topk_prob, want_gap=probe)
         if probe:
             self.boundary_gap = gap.mean()                                   # router.py:33-36
-        return idx.view(bsz, seq, -1).long(), wgt.view(bsz, seq, -1)
+        idx = idx.view(bsz, seq, -1).long()
+        if _wants_grad(hidden_states, self.gate_proj.weight):
+            # the kernel's selection, the weights again as differentiable tensor operations (router.py:25-26,31,41-47)
+            scores = torch.sigmoid(self.gate_proj(hidden_states).float())
+            raw = scores.gather(-1, idx)
+            if self.top_k > 1 and self.norm_topk_prob == "softmax":
+                return idx, torch.softmax(raw, dim=-1)
+            if self.top_k > 1 and self.norm_topk_prob:
+                return idx, raw / (raw.sum(dim=-1, keepdim=True) + 1e-20)
+            return idx, raw
+        return idx, wgt.view(bsz, seq, -1)
 
 
 class BiBoFusedExperts(nn.Module):
@@ -213,7 +246,18 @@ class BiBoFusedExperts(nn.Module):
     @_no_compile
     def forward(self, hidden_states: torch.Tensor, top_k_indices: torch.Tensor, top_k_weights: torch.Tensor,
                 _want_counts: bool = False):
-        _forward_only_guard(hidden_states, top_k_weights, self.gate_up_proj)
+        if _wants_grad(hidden_states, top_k_weights, self.gate_up_proj, self.down_proj, self.radial_theta):
+            if _compute_dtype(hidden_states) != torch.bfloat16:
+                raise RuntimeError("the backward pass runs in bf16: use bf16 activations or bf16 autocast, or call the "
+                                   "experts under torch.no_grad()")
+            if not _backward_covers(self):
+                raise NotImplementedError("the backward pass covers GLU experts only (no +/-Identity experts), hidden and "
+                                          "expert sizes that are multiples of 128 and expert size <= 512")
+            out, counts = _ExpertsFn.apply(hidden_states, top_k_weights, self.gate_up_proj, self.down_proj, self.radial_theta,
+                                           top_k_indices.detach().to(torch.int32).contiguous(), self.act, self.algo,
+                                           _want_counts)
+            out = out if out.dtype == hidden_states.dtype else out.to(hidden_states.dtype)
+            return (out, counts) if _want_counts else out
         cd = _compute_dtype(hidden_states)
         x = hidden_states.detach()
         x = (x.to(cd) if x.dtype != cd else x).contiguous()
@@ -379,7 +423,7 @@ class BiBoMoELayer(nn.Module):
         if _compute_dtype(x) != torch.bfloat16:
             raise RuntimeError("the backward pass runs in bf16: use bf16 activations or bf16 autocast, or call the layer "
                                "under torch.no_grad()")
-        if e.num_pos + e.num_neg > 0 or self.hidden_size % 128 or e.intermediate_size % 128 or e.intermediate_size > 512:
+        if not _backward_covers(e):
             raise NotImplementedError("the backward pass covers GLU experts only (no +/-Identity experts), hidden and "
                                       "expert sizes that are multiples of 128 and expert size <= 512")
         out, counts = _MoELayerFn.apply(x, self.gate.gate_proj.weight, e.gate_up_proj, e.down_proj, e.radial_theta,

@@ -316,6 +316,33 @@ def moe_backward(x, d_out, w_router, bias, w_gate_up, w_down, theta, k, norm="su
     return d_x, d_wr, d_gu, d_dn, d_theta, d_w
 
 
+def experts_backward(x, d_out, idx, w, w_gate_up, w_down, theta, act="radial"):
+    """bibo_moe_experts_backward: gradients of experts_fwd for a caller-owned routing (idx int32 [T,k], w fp32 [T,k]).
+    -> d_x [T,H], d_w fp32 [T,k], d_w_gate_up, d_w_down (x.dtype), d_theta fp32 [E]."""
+    T, H = x.shape
+    E, two_i, _ = w_gate_up.shape
+    I = two_i // 2
+    k = idx.shape[1]
+    dc = _dtype_code(x)
+    _chk(x, "x"); _chk(d_out, "d_out", x.dtype, (T, H)); _chk(idx, "idx", torch.int32, (T, k)); _chk(w, "w", torch.float32, (T, k))
+    _chk(w_gate_up, "w_gate_up", x.dtype, (E, 2 * I, H)); _chk(w_down, "w_down", x.dtype, (E, H, I))
+    _chk(theta, "theta", torch.float32, (E,))
+    dev = x.device
+    d_x, d_gu, d_dn = torch.empty_like(x), torch.empty_like(w_gate_up), torch.empty_like(w_down)
+    d_w = torch.empty(T, k, dtype=torch.float32, device=dev)
+    d_theta = torch.empty(E, dtype=torch.float32, device=dev)
+    sh = L.Shape(T, H, E, k, I, dc, 0, 0, act_code(act), 0)
+    nbytes = ctypes.c_size_t(0)
+    L.check(L.lib().bibo_moe_backward_workspace_bytes(ctypes.byref(sh), ctypes.byref(nbytes)), "bibo_moe_backward_workspace_bytes")
+    ws = workspace(dev, nbytes.value)
+    with torch.cuda.device(dev):
+        L.check(L.lib().bibo_moe_experts_backward(_ptr(x), _ptr(d_out), _ptr(idx), _ptr(w), _ptr(w_gate_up), _ptr(w_down),
+                                                  _ptr(theta), ctypes.byref(sh), _ptr(d_x), _ptr(d_w), _ptr(d_gu), _ptr(d_dn),
+                                                  _ptr(d_theta), _ptr(ws), ws.numel(), _stream(dev)),
+                "bibo_moe_experts_backward")
+    return d_x, d_w, d_gu, d_dn, d_theta
+
+
 def attn_res_fwd(candidates, score_weight, eps):
     """bibo_moe_exp_attn_res_fwd: softmax-weighted average of the candidate rows, scores rsqrt(mean c^2 + eps) <c, score_weight>
     (apply_attention_residual, exp/modeling_bibo.py:119-232).  candidates: list of [T,H] bf16; score_weight fp32 [H]."""

@@ -282,6 +282,17 @@ int bibo_moe_backward(const void* x, const void* d_out, const void* w_router, co
                       void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * Backward pass of the experts alone (what autograd derives for BiBoFusedExperts.forward, src/modeling/ffn/moe.py:46-101)
+ * for a caller that owns the routing: idx int32 [T,k] (every entry a valid expert id) and w fp32 [T,k] as handed to
+ * bibo_moe_experts_fwd.  d_w fp32 [T,k] is the gradient with respect to w (moe.py:93), through which the caller's own
+ * router is reached; the other results and the limits are those of bibo_moe_backward, whose workspace size it shares.
+ */
+int bibo_moe_experts_backward(const void* x, const void* d_out, const int32_t* idx, const float* w, const void* w_gate_up,
+                              const void* w_down, const float* theta, const bibo_moe_shape* shape, void* d_x, float* d_w,
+                              void* d_w_gate_up, void* d_w_down, float* d_theta, void* workspace, size_t workspace_bytes,
+                              void* stream);
+
+/*
  * Depth mix of the experimental model's Block Attention Residuals: apply_attention_residual
  * (exp/modeling_bibo.py:119-232; softmax scores, dense), the operation the reference hands to its optional external
  * kernel `kernels.sm120.attn_res.attn_res(block_residual, prefix, score_weight, eps, ...)` (exp/modeling_bibo.py:44,

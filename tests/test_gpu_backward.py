@@ -175,3 +175,44 @@ def test_what_the_backward_does_not_cover_is_refused():
     with torch.autocast("cuda", dtype=torch.bfloat16):
         fp32(torch.randn(1, 8, 256, device=DEV)).sum().backward()  # fp32 master weights under bf16 autocast train
     assert fp32.experts.gate_up_proj.grad is not None and fp32.experts.gate_up_proj.grad.dtype == torch.float32
+
+
+def test_experts_backward_with_caller_owned_routing():
+    """bibo_moe_experts_backward: the experts alone, routing handed in (an expert may repeat inside a token); d_w is the
+    gradient of the combine weights."""
+    T, H, E, k, I = 200, 256, 8, 3, 128
+    p = O.make_inputs(T=T, H=H, E=E, k=k, I=I, theta="normal", seed=9)
+    g = torch.Generator().manual_seed(4)
+    idx = torch.randint(0, E, (T, k), generator=g, dtype=torch.int32)
+    w = torch.rand(T, k, generator=g) + 0.1
+    d_out = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    dev = lambda t: t.to(DEV)
+    got = ops.experts_backward(dev(p["x"]), dev(d_out), dev(idx), dev(w), dev(p["w_gate_up"]), dev(p["w_down"]), dev(p["theta"]))
+    torch.cuda.synchronize()
+    leaf = lambda t: t.double().clone().requires_grad_(True)
+    x, wl, gu, dn, th = leaf(p["x"]), leaf(w), leaf(p["w_gate_up"]), leaf(p["w_down"]), leaf(p["theta"])
+    (O.experts_forward(x, idx, wl, gu, dn, th, dtype=torch.float64) * d_out.double()).sum().backward()
+    for a, r, name in zip(got, (x.grad, wl.grad, gu.grad, dn.grad, th.grad), ("x", "w", "w_gate_up", "w_down", "theta")):
+        assert _rel(a, r) <= TOL, (name, _rel(a, r))
+
+
+def test_hooks_path_trains_module_by_module():
+    """With a hook present the layer calls router and experts as modules; both carry autograd graphs, and the
+    gradients agree with the single-node path."""
+    layer = _layer(H=256, I=128, E=16, k=4)
+    with torch.no_grad():
+        layer.experts.radial_theta.copy_(torch.linspace(-1, 1, 16))
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn(2, 40, 256, generator=g).to(torch.bfloat16).to(DEV)
+    d = torch.randn(2, 40, 256, generator=g).to(torch.bfloat16).to(DEV)
+    layer(x).backward(d)
+    ref = {n: p.grad.clone() for n, p in layer.named_parameters() if p.grad is not None}
+    layer.zero_grad()
+    seen = []
+    h = layer.gate.register_forward_hook(lambda m, i, o: seen.append(o[0].shape))
+    layer(x).backward(d)
+    h.remove()
+    assert seen == [torch.Size([2, 40, 4])]
+    for n, p in layer.named_parameters():
+        if n in ref:
+            assert _rel(p.grad, ref[n].cpu()) <= 3e-2, n

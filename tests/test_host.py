@@ -240,13 +240,13 @@ def test_specials_and_shared_expert_follow_the_reference_layout():
 
 
 def test_forward_refuses_to_drop_gradients():
-    """What has no backward says so instead of returning a result without a graph: fp32 compute in the layer, and
-    the router / experts modules called on their own."""
+    """What has no backward says so instead of returning a result without a graph: fp32 compute in the layer and in
+    the experts module called on its own."""
     layer = bibo_amd.BiBoMoELayer(make_config())
     with pytest.raises(RuntimeError, match="backward pass runs in bf16"):
         layer(torch.zeros(1, 4, 64))
-    with pytest.raises(RuntimeError, match="forward pass only"):
-        layer.gate(torch.zeros(1, 4, 64))
+    with pytest.raises(RuntimeError, match="backward pass runs in bf16"):
+        layer.experts(torch.zeros(4, 64), torch.zeros(4, 2, dtype=torch.long), torch.ones(4, 2))
 
 
 # ------------------------------------------------------------------ balancing closed forms
