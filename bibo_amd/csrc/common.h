@@ -116,6 +116,17 @@ __device__ __forceinline__ void match64(int e, bool valid, int lane, unsigned lo
   }
 }
 
+// Workgroup barrier that lets the N most recent LDS-DMA loads of every thread stay in flight: s_waitcnt vmcnt(N)
+// lgkmcnt(0) (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4 left at "no wait", lgkmcnt 11:8), then s_barrier.
+// __syncthreads() cannot be used for this: its release fence waits for every outstanding LDS-DMA transfer.  The
+// older loads have landed in every wave once all waves have passed, and every wave's LDS reads of the stage that is
+// refilled next have returned.
+template <int N>
+__device__ __forceinline__ void sync_keep_loads() {
+  __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | (0x7 << 4));
+  __builtin_amdgcn_s_barrier();
+}
+
 // Map a workgroup id to a tile so that the workgroups of one XCD (ids congruent mod 8 are dispatched
 // to the same XCD) walk a contiguous range of tiles: tiles of one expert then share that XCD's L2.
 __device__ __forceinline__ int xcd_tile(int bid, int total) {

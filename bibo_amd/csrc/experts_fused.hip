@@ -58,17 +58,6 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, un
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);   // raw buffer, 32-bit data format
 }
 
-// Workgroup barrier that lets the N most recent LDS-DMA loads of every thread stay in flight: s_waitcnt vmcnt(N)
-// lgkmcnt(0) (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4 left at "no wait", lgkmcnt 11:8), then s_barrier.
-// __syncthreads() cannot be used for this: its release fence waits for every outstanding LDS-DMA transfer.  The
-// older loads have landed in every wave once all waves have passed, and every wave's LDS reads of the stage that is
-// refilled next have returned.
-template <int N>
-__device__ __forceinline__ void sync_keep_loads() {
-  __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | (0x7 << 4));
-  __builtin_amdgcn_s_barrier();
-}
-
 // What one thread needs to request a weight stage and the x rows of a K step.
 template <typename F>
 struct SubLoader {

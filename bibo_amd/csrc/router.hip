@@ -137,46 +137,69 @@ __global__ __launch_bounds__(256) void router_generic_kernel(const TIn* __restri
   }
 }
 
-// One exchange of a (value, expert) pair with the lane a DPP control selects inside the 16-lane row; the
-// larger value wins, equal values go to the lower expert.
+// Integer key of a score whose unsigned order is the order of the floats (-0 counts as +0): the row-wide maximum
+// is then one v_max_u32 per butterfly step instead of a compare-and-select on (value, expert) pairs under exec
+// masks, which cost this selection 3.5 us per workgroup.
+__device__ __forceinline__ unsigned order_key(float v) {
+  const unsigned u = __float_as_uint(v + 0.f);
+  return u ^ ((unsigned)((int)u >> 31) | 0x80000000u);
+}
+__device__ __forceinline__ float key_value(unsigned key) {
+  return __uint_as_float((key & 0x80000000u) ? key ^ 0x80000000u : ~key);
+}
+
 template <int kCtrl>
-__device__ __forceinline__ void dpp_max_step(float& bv, int& be) {
-  const float ov = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, bv), kCtrl, 0xf, 0xf, false));
-  const int oe = __builtin_amdgcn_update_dpp(0, be, kCtrl, 0xf, 0xf, false);
-  if (ov > bv || (ov == bv && oe < be)) { bv = ov; be = oe; }
+__device__ __forceinline__ unsigned dpp_u32(unsigned v) {
+  return (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, kCtrl, 0xf, 0xf, false);
+}
+// 16-lane butterfly on DPP row operations (a DPP row is exactly one token's 16 lanes): swap within pairs, swap
+// pairs within quads, mirror within 8 lanes, mirror within 16 lanes.  Every lane ends with the row's result.
+__device__ __forceinline__ unsigned row_max_u32(unsigned v) {
+  v = max(v, dpp_u32<0xB1>(v));
+  v = max(v, dpp_u32<0x4E>(v));
+  v = max(v, dpp_u32<0x141>(v));
+  return max(v, dpp_u32<0x140>(v));
+}
+__device__ __forceinline__ unsigned row_min_u32(unsigned v) {
+  v = min(v, dpp_u32<0xB1>(v));
+  v = min(v, dpp_u32<0x4E>(v));
+  v = min(v, dpp_u32<0x141>(v));
+  return min(v, dpp_u32<0x140>(v));
 }
 
 // Cooperative selection: 16 lanes per token, lane `seg` owns experts 4*seg .. 4*seg+3.  k rounds of
-// "best remaining candidate": local scan in ascending expert order, then a 16-lane butterfly on
-// (value, expert) where the larger value wins and equal values go to the lower expert.  All 16 lanes
-// end every round with the same winner.  Returns the bit mask of the chosen experts.
+// "best remaining candidate": the row's largest key, then the lowest expert index among the lanes that hold it,
+// which is the tie rule (equal floats have equal keys).  All 16 lanes end every round with the same winner.
+// Returns the bit mask of the chosen experts.
 __device__ __forceinline__ unsigned long long select_mask16(const float (&v)[4], int seg, int rounds, float* kth,
                                                             float* kth1) {
+  unsigned key[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) key[q] = order_key(v[q]);
   unsigned taken = 0;
   unsigned long long mask = 0;
   for (int r = 0; r < rounds; ++r) {
-    float bv = -INFINITY;
-    int be = kMaxE;
+    unsigned bk = 0, be = kMaxE;                     // a taken expert counts as key 0, below every score's key
 #pragma unroll
-    for (int q = 0; q < 4; ++q)
-      if (!((taken >> q) & 1) && (v[q] > bv || be == kMaxE)) { bv = v[q]; be = seg * 4 + q; }
-    if (taken == 0xf) { bv = -INFINITY; be = kMaxE; }
-    // 16-lane butterfly on DPP row operations (a DPP row is exactly one token's 16 lanes): swap within
-    // pairs, swap pairs within quads, mirror within 8 lanes, mirror within 16 lanes.
-    dpp_max_step<0xB1>(bv, be);
-    dpp_max_step<0x4E>(bv, be);
-    dpp_max_step<0x141>(bv, be);
-    dpp_max_step<0x140>(bv, be);
+    for (int q = 0; q < 4; ++q) {
+      const unsigned kq = ((taken >> q) & 1) ? 0u : key[q];
+      if (kq > bk) { bk = kq; be = seg * 4 + q; }    // strict: the lower expert of the lane keeps an equal key
+    }
+    const unsigned mk = row_max_u32(bk);
+    be = row_min_u32(bk == mk ? be : (unsigned)kMaxE);
     be &= kMaxE - 1;
-    if ((be >> 2) == seg) taken |= 1u << (be & 3);
+    if ((int)(be >> 2) == seg) taken |= 1u << (be & 3);
     mask |= 1ull << be;
-    if (kth != nullptr) { if (r == rounds - 2) *kth = bv; if (r == rounds - 1) *kth1 = bv; }
+    if (kth != nullptr) { if (r == rounds - 2) *kth = key_value(mk); if (r == rounds - 1) *kth1 = key_value(mk); }
   }
   return mask;
 }
 
 // Selection for the tokens of one workgroup whose scores sit in LDS rows `sc` (stride kRowPad):
-// thread = (token tid>>4, segment tid&15); needs blockDim.x >= 16 * ntok_max.
+// thread = (token tid>>4, segment tid&15); needs blockDim.x >= 16 * ntok_max.  Lane j < k of a token's 16 then
+// owns output j (the j-th chosen expert in ascending order): it gathers the unbiased score, the row adds the scores
+// up one after the other in that order (a serial scan over lanes, so the sum has the bits of the sequential loop),
+// and every lane normalises and stores its own weight.
 // Returns the bit mask of the experts chosen for this thread's token (0 for a token past the end).
 __device__ __forceinline__ unsigned long long select_tokens16(const float* __restrict__ sc,
                                                               const float* __restrict__ bias_s, int E, int k,
@@ -196,41 +219,37 @@ __device__ __forceinline__ unsigned long long select_tokens16(const float* __res
   const unsigned long long mask = select_mask16(v, seg, k, nullptr, nullptr);
   float g_hi = 0.f, g_lo = 0.f;
   if (gap != nullptr && k < E) select_mask16(u, seg, k + 1, &g_hi, &g_lo);   // router.py:33-36, unbiased scores
-  if (live && seg == 0) {
-    const int t = t0 + tl;
-    float raw[kMaxK];
-    float sum = 0.f, mx = -INFINITY;
-    unsigned long long m = mask;
+  const bool mine = seg < k;                                              // this lane owns output `seg`
+  unsigned long long m = mask;
 #pragma unroll
-    for (int j = 0; j < kMaxK; ++j) {
-      raw[j] = 0.f;
-      if (j < k) {
-        const int e = __ffsll((long long)m) - 1;                          // ascending expert order
-        m &= m - 1;
-        idx[(size_t)t * k + j] = e;
-        raw[j] = row[e];                                                  // UNBIASED score, router.py:41
-        sum += raw[j];
-        mx = fmaxf(mx, raw[j]);
-      }
+  for (int j = 0; j < kMaxK - 1; ++j)
+    if (j < seg) m &= m - 1;                                              // drop the `seg` lowest chosen experts
+  const int e = mine ? __ffsll((long long)m) - 1 : 0;                     // ascending expert order
+  const float raw = mine ? row[e] : 0.f;                                  // UNBIASED score, router.py:41
+  // running sum in ascending j, one lane after the other: lane j ends with ((raw_0 + raw_1) + ...) + raw_j
+  auto scan = [&](float x) {
+    float s = x;
+#pragma unroll
+    for (int j = 1; j < kMaxK; ++j) {
+      const float prev = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, s), 0x111, 0xf, 0xf, false));
+      if (seg == j && j < k) s = prev + x;                                // row_shr:1, lane j reads lane j-1
     }
-    float* wo = w + (size_t)t * k;
-    if (k > 1 && norm_mode == BIBO_NORM_SOFTMAX) {                        // router.py:42-43
-      float ex[kMaxK];
-      float es = 0.f;
-#pragma unroll
-      for (int j = 0; j < kMaxK; ++j) { ex[j] = (j < k) ? expf(raw[j] - mx) : 0.f; es += ex[j]; }
-#pragma unroll
-      for (int j = 0; j < kMaxK; ++j) if (j < k) wo[j] = ex[j] / es;
-    } else if (k > 1 && norm_mode == BIBO_NORM_SUM) {                     // router.py:44-45
-      const float den = sum + kSumNormEps;
-#pragma unroll
-      for (int j = 0; j < kMaxK; ++j) if (j < k) wo[j] = raw[j] / den;
-    } else {                                                              // router.py:46-47
-#pragma unroll
-      for (int j = 0; j < kMaxK; ++j) if (j < k) wo[j] = raw[j];
-    }
-    if (gap != nullptr) gap[t] = (k < E) ? (g_hi - g_lo) : 0.f;
+    return __shfl(s, (tid & 48) + k - 1, kWave);                          // the whole sum, from lane k-1 of the row
+  };
+  float wv = raw;                                                         // router.py:46-47
+  if (k > 1 && norm_mode == BIBO_NORM_SOFTMAX) {                          // router.py:42-43
+    const float mx = key_value(row_max_u32(mine ? order_key(raw) : 0u));
+    const float ex = mine ? expf(raw - mx) : 0.f;
+    wv = ex / scan(ex);
+  } else if (k > 1 && norm_mode == BIBO_NORM_SUM) {                       // router.py:44-45
+    wv = raw / (scan(raw) + kSumNormEps);
   }
+  if (live && mine) {
+    const size_t o = (size_t)(t0 + tl) * k + seg;
+    idx[o] = e;
+    w[o] = wv;
+  }
+  if (live && seg == 0 && gap != nullptr) gap[t0 + tl] = (k < E) ? (g_hi - g_lo) : 0.f;
   return live ? mask : 0ull;
 }
 
