@@ -161,6 +161,49 @@ __global__ __launch_bounds__(256) void combine_bf16x8_kernel(const bf16_t* __res
   }
 }
 
+// fp32 slot rows -> bf16 output, 4 columns per thread: the decode-size combine, whose duration is one round trip of
+// its loads, issues a quarter of the threads and all k loads of a thread at once.  Same sum as combine_kernel.
+__global__ __launch_bounds__(256) void combine_f32x4_kernel(const float* __restrict__ yw, CombineArgs a, int T, int H4,
+                                                            int k, bf16_t* __restrict__ out) {
+  const size_t n = (size_t)T * H4;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
+    const size_t t = i / H4, c = i - t * H4;
+    floatx4 v[kMaxK];
+    int sign[kMaxK];
+    bool special[kMaxK];
+    const floatx4* src = reinterpret_cast<const floatx4*>(yw) + (t * k) * H4 + c;
+#pragma unroll
+    for (int j = 0; j < kMaxK; ++j)
+      if (j < k) {
+        special[j] = special_slot<bf16_t>(a, t * k + j, &sign[j]);
+        if (!special[j]) v[j] = src[(size_t)j * H4];
+      }
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < kMaxK; ++j)
+      if (j < k) {
+        if (special[j]) {
+          if (sign[j] != 0) {
+            const float sw = (float)sign[j] * a.w[t * k + j];
+            const bf16x4 xv = reinterpret_cast<const bf16x4*>(a.x)[i];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) acc[q] += sw * (float)xv[q];
+          }
+        } else {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) acc[q] += v[j][q];
+        }
+      }
+    if (a.residual != nullptr) {
+      const bf16x4 r = reinterpret_cast<const bf16x4*>(a.residual)[i];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) acc[q] = (a.round_block ? (float)(bf16_t)acc[q] : acc[q]) + (float)r[q];
+    }
+    bf16x4 o = {(bf16_t)acc[0], (bf16_t)acc[1], (bf16_t)acc[2], (bf16_t)acc[3]};
+    reinterpret_cast<bf16x4*>(out)[i] = o;
+  }
+}
+
 }  // namespace
 
 hipError_t launch_gateup_generic(const void* x, const void* wgu, const float* theta, const int32_t* offsets,
@@ -212,8 +255,15 @@ hipError_t launch_combine(const void* yw, int yw_is_bf16, const CombineArgs& a, 
       hipLaunchKernelGGL((combine_kernel<bf16_t, bf16_t>), dim3(grid), dim3(256), 0, s,
                          static_cast<const bf16_t*>(yw), a, T, H, k, static_cast<bf16_t*>(out));
   } else if (dtype == BIBO_DTYPE_BF16) {
-    hipLaunchKernelGGL((combine_kernel<float, bf16_t>), dim3(grid), dim3(256), 0, s, static_cast<const float*>(yw), a, T,
-                       H, k, static_cast<bf16_t*>(out));
+    if ((H % 4) == 0 && ((reinterpret_cast<uintptr_t>(yw) | reinterpret_cast<uintptr_t>(out) |
+                          reinterpret_cast<uintptr_t>(a.residual) | reinterpret_cast<uintptr_t>(a.x)) & 15) == 0) {
+      const size_t n4 = n / 4;
+      const int g4 = (int)((n4 + 255) / 256 < 65536 ? (n4 + 255) / 256 : 65536);
+      hipLaunchKernelGGL(combine_f32x4_kernel, dim3(g4), dim3(256), 0, s, static_cast<const float*>(yw), a, T, H / 4, k,
+                         static_cast<bf16_t*>(out));
+    } else
+      hipLaunchKernelGGL((combine_kernel<float, bf16_t>), dim3(grid), dim3(256), 0, s, static_cast<const float*>(yw), a, T,
+                         H, k, static_cast<bf16_t*>(out));
   } else {
     hipLaunchKernelGGL((combine_kernel<float, float>), dim3(grid), dim3(256), 0, s, static_cast<const float*>(yw), a, T,
                        H, k, static_cast<float*>(out));
