@@ -77,7 +77,7 @@ __global__ __launch_bounds__(256) void scatter_kernel(const int32_t* __restrict_
   wave_cnt[wave][lane] = mycnt;
 
   int tot = 0, bef = 0;
-  constexpr int kBatch = 16;                       // histograms requested together: one memory latency per batch
+  constexpr int kBatch = 64;                       // histograms requested together: one memory latency per batch
   for (int bb0 = wave; bb0 < nhist; bb0 += 4 * kBatch) {
     int v[kBatch];
 #pragma unroll
