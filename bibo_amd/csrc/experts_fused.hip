@@ -23,6 +23,12 @@
 // activations already fill most of the LDS.
 // Each block of columns is scaled by the routing weight, staged through LDS 32 rows at a time (in the two x
 // buffers, which are idle by then) and scattered to slot order as 256-byte row segments.
+// A tile may hold fewer than 128 rows (an expert's last tile, or all of its rows).  32-row blocks without rows are
+// not multiplied: the kernel body exists once per number of blocks (1 to 4), with the MFMAs, activations, down
+// projection row tiles and output rounds of the missing blocks left out; every wave still issues its share of
+// the weight requests.  A tile's duration hardly depends on its rows all the same (it is the stream of its
+// expert's weights through one CU: 3-block tiles take as long as 4-block tiles), which is why cutting the tiles
+// so that they fill whole rounds of the chip (512 tiles of 96 rows for the 410 of the prefill shape) gained nothing.
 // Reference: BiBoFusedExperts.forward, src/modeling/ffn/moe.py:81-93.
 #include <type_traits>
 
@@ -147,9 +153,18 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
   e = __builtin_amdgcn_readfirstlane(e);                // the same for every lane: keep them in scalar registers
   row0 = __builtin_amdgcn_readfirstlane(row0);
   rows = __builtin_amdgcn_readfirstlane(rows);
+  const int nblocks = (rows + 31) >> 5;                 // 32-row blocks that hold rows: 1 .. 4
 
+  // The rest of the kernel exists once per number of blocks, chosen here, where nothing is alive yet: the copies
+  // share no values, so each gets the registers the kernel would get if it were the only one.
+  auto body = [&](auto nblocks_c) {
+  constexpr int kBlocks = decltype(nblocks_c)::value;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int wn = wave & 3, wm = wave >> 2;
+  // M wave wm owns blocks 2 wm and 2 wm + 1; blocks without rows are not multiplied.  The two waves of a SIMD
+  // belong to different M waves, so what a SIMD's MFMA pipe has to do goes with the tile's blocks either way.
+  static_assert(MT == 2, "two blocks per M wave");
+  const int my_blocks = __builtin_amdgcn_readfirstlane(wm == 0 ? (kBlocks < 2 ? kBlocks : 2) : (kBlocks > 2 ? kBlocks - 2 : 0));
   const int n = lane & 31;
   const int mbase = wm * MT * 32;
   auto stage = [&](auto ic) -> bf16_t* {
@@ -210,7 +225,8 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
     // fragment side: lane (n, h) reads logical granule 2*ss + h of rows congruent to n mod 32
     const int pos0 = ((lane >> 5) ^ ((n >> 1) & 7)) * 8;
     auto frag_row = [&](int j) { return (wn * 2 + j) * 32; };
-    auto substep = [&](auto tc, auto pc, int s) {
+    auto substep = [&](auto mc, auto tc, auto pc, int s) {
+      constexpr int nmt = decltype(mc)::value;           // M tiles of this wave that hold rows
       constexpr int t = decltype(tc)::value, par = decltype(pc)::value;
       constexpr int cur = NT == 1 ? par : t;
       // loads still allowed in flight: those of the sub-steps after the one whose stage is read now
@@ -221,17 +237,28 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
       const bf16_t* b0 = stage(std::integral_constant<int, cur>{}) + n * BK;
       request(tc, pc, s);
       const SubIssuer<F, t == 0> issuer{ld};
-      stripe_step<MT, 2, BK, true, 2 * NT, t, NT>(acc, a0, 32 * BK, b0, pos0, frag_row, issuer, true, 0, nullptr);
+      if constexpr (nmt > 0)
+        stripe_step<nmt, 2, BK, true, 2 * NT, t, NT>(acc, a0, 32 * BK, b0, pos0, frag_row, issuer, true, 0, nullptr);
+      else
+        issue_some<0, SubIssuer<F, t == 0>::kInstr>(issuer, 0, nullptr);   // its share of the requests all the same
     };
     using std::integral_constant;
-    for (int s = 0; s < nsteps; s += 2) {                                         // H / BK is even
-      substep(integral_constant<int, 0>{}, integral_constant<int, 0>{}, s);
-      if constexpr (NT > 1) substep(integral_constant<int, 1>{}, integral_constant<int, 0>{}, s);
-      if constexpr (NT > 2) substep(integral_constant<int, 2>{}, integral_constant<int, 0>{}, s);
-      substep(integral_constant<int, 0>{}, integral_constant<int, 1>{}, s + 1);
-      if constexpr (NT > 1) substep(integral_constant<int, 1>{}, integral_constant<int, 1>{}, s + 1);
-      if constexpr (NT > 2) substep(integral_constant<int, 2>{}, integral_constant<int, 1>{}, s + 1);
-    }
+    // one copy of the K loop per number of M tiles with rows, chosen once: a choice inside the loop would meet at
+    // every sub-step with all 192 accumulator registers alive
+    auto kloop = [&](auto mc) {
+      for (int s = 0; s < nsteps; s += 2) {                                       // H / BK is even
+        substep(mc, integral_constant<int, 0>{}, integral_constant<int, 0>{}, s);
+        if constexpr (NT > 1) substep(mc, integral_constant<int, 1>{}, integral_constant<int, 0>{}, s);
+        if constexpr (NT > 2) substep(mc, integral_constant<int, 2>{}, integral_constant<int, 0>{}, s);
+        substep(mc, integral_constant<int, 0>{}, integral_constant<int, 1>{}, s + 1);
+        if constexpr (NT > 1) substep(mc, integral_constant<int, 1>{}, integral_constant<int, 1>{}, s + 1);
+        if constexpr (NT > 2) substep(mc, integral_constant<int, 2>{}, integral_constant<int, 1>{}, s + 1);
+      }
+    };
+    static_assert(MT == 2, "the three copies below are 2, 1 and 0 M tiles");
+    if (my_blocks == 2) kloop(integral_constant<int, 2>{});
+    else if (my_blocks == 1) kloop(integral_constant<int, 1>{});
+    else kloop(integral_constant<int, 0>{});
   }
   wait_loads_and_sync();                   // every transfer has landed and every wave is done with the stages
 
@@ -278,6 +305,7 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
 #pragma unroll
         for (int d = 0; d < D; ++d) load_wblock<CT>(wb[d], wp, tile_stride, d);
       }
+      if (mt >= my_blocks) continue;          // a block without rows: nobody reads its activations
       const int m = mbase + mt * 32 + n;
       const float rinv = rinv_s[m];
       const float nrl = -1.44269504f * rinv, rg = rinv * gain_s[m];            // per-row constants folded once
@@ -306,13 +334,15 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
   const int r16 = lane & 15, g4 = lane >> 4;
   const int nblk = H / F::BN2;
   const int sel = 4 * (4 * r16 + g4);
-  for (int nb = 0; nb < nblk; ++nb) {
+  // One block of F::BN2 output columns for the first NRT 16-row tiles of the tile (NRT = 2 per block that holds rows).
+  auto down_block = [&](auto nrt_c, int nb) {
+    constexpr int NRT = decltype(nrt_c)::value;
     const int n0 = nb * F::BN2;
-    floatx4 acc2[CT][8];
+    floatx4 acc2[CT][NRT];
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct)
 #pragma unroll
-      for (int rt = 0; rt < 8; ++rt) acc2[ct][rt] = floatx4{0.f, 0.f, 0.f, 0.f};
+      for (int rt = 0; rt < NRT; ++rt) acc2[ct][rt] = floatx4{0.f, 0.f, 0.f, 0.f};
     // Activation fragments are read a row tile ahead of the MFMAs that consume them (across K block
     // boundaries too).
     auto frag = [&](int kb, int rt, int s) {
@@ -321,7 +351,7 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
       const bf16_t* slice = (kb >> 1) == 0 ? S0 : ((kb >> 1) == 1 ? S1 : S2);
       return *reinterpret_cast<const bf16x8*>(slice + (rt * 16 + r16) * 128 + gq);
     };
-    // The multiply walks half K blocks (32 elements, one MFMA deep): while half hs is multiplied with all eight
+    // The multiply walks half K blocks (32 elements, one MFMA deep): while half hs is multiplied with all NRT
     // row tiles, the weights of half hs + 1 change lanes and the activation fragment of the next row tile is read.
     bf16x8 wc[2][CT], xa[2];
 #pragma unroll
@@ -335,10 +365,14 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
       for (int s = 0; s < 2; ++s) {
         const int hs = 2 * kb + s;
 #pragma unroll
-        for (int rt = 0; rt < 8; ++rt) {
-          const int g = hs * 8 + rt;           // running (half K block, row tile) index
-          if (g + 1 < KB * 16) xa[(g + 1) & 1] = frag((g + 1) >> 4, (g + 1) & 7, ((g + 1) >> 3) & 1);
-          if (rt < CT && hs + 1 < 2 * KB) wc[(hs + 1) & 1][rt] = to_operand_lanes(wb[((hs + 1) >> 1) % NB].w[rt][(hs + 1) & 1], sel);
+        for (int rt = 0; rt < NRT; ++rt) {
+          const int g = hs * NRT + rt;         // running (half K block, row tile) index
+          if (g + 1 < KB * 2 * NRT) xa[(g + 1) & 1] = frag(((g + 1) / NRT) >> 1, (g + 1) % NRT, ((g + 1) / NRT) & 1);
+          // the CT lane exchanges of the next half are spread over the row tiles (the last tile takes what is left)
+#pragma unroll
+          for (int cx = 0; cx < CT; ++cx)
+            if ((cx == rt || (rt == NRT - 1 && cx > rt)) && hs + 1 < 2 * KB)
+              wc[(hs + 1) & 1][cx] = to_operand_lanes(wb[((hs + 1) >> 1) % NB].w[cx][(hs + 1) & 1], sel);
 #pragma unroll
           for (int ct = 0; ct < CT; ++ct)
             acc2[ct][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[hs & 1][ct], xa[g & 1], acc2[ct][rt], 0, 0, 0);
@@ -391,7 +425,7 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
         }
       }
     };
-    constexpr int NR = BM / F::kOutRows;
+    constexpr int NR = NRT * 16 / F::kOutRows;
     stage_rows(0);
 #pragma unroll
     for (int hf = 0; hf < NR; ++hf) {
@@ -399,8 +433,15 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
       if (hf + 1 < NR) stage_rows(hf + 1);
       copy_out(hf);
     }
-  }
+  };
+  for (int nb = 0; nb < nblk; ++nb) down_block(std::integral_constant<int, 2 * kBlocks>{}, nb);
+  };   // body
+  if (nblocks == 4) body(std::integral_constant<int, 4>{});
+  else if (nblocks == 3) body(std::integral_constant<int, 3>{});
+  else if (nblocks == 2) body(std::integral_constant<int, 2>{});
+  else body(std::integral_constant<int, 1>{});
 }
+
 
 template <int NT, int CT>
 void launch_fused_t(const bf16_t* x, const bf16_t* wgu, const bf16_t* wd, const float* theta, const float* w,

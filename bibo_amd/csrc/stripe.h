@@ -139,8 +139,8 @@ __device__ __forceinline__ void issue_some(const Loader& ld, int k_next, bf16_t*
 // (if there is one): spreading the loads through the MFMAs keeps the waves from queueing up at the
 // texture-address unit before they start multiplying.  `a1` points at this lane's A fragment of the
 // second sub-step for M tile 0; tile mt is `astride` elements further.
-template <int Q, int MT, int NTW, int BK, bool TR, int NACC, int J0, int JS, typename Loader, typename FragRow>
-__device__ __forceinline__ void stripe_pair(floatx16 (&acc)[MT][NACC], bf16x8 (&a)[2][MT], bf16x8 (&b)[3],
+template <int Q, int MT, int NTW, int BK, bool TR, int NACC, int J0, int JS, typename Loader, typename FragRow, int AMT>
+__device__ __forceinline__ void stripe_pair(floatx16 (&acc)[AMT][NACC], bf16x8 (&a)[2][MT], bf16x8 (&b)[3],
                                             const bf16_t* a0, int astride, const bf16_t* bstage, int pos0,
                                             FragRow frag_row, const Loader& ld, bool prefetch, int k_next,
                                             bf16_t* next_stage) {
@@ -170,8 +170,8 @@ __device__ __forceinline__ void stripe_pair(floatx16 (&acc)[MT][NACC], bf16x8 (&
   __builtin_amdgcn_sched_group_barrier(0x008, MT, 0);
 }
 
-template <int MT, int NTW, int BK, bool TR, int NACC, int J0, int JS, typename Loader, typename FragRow, int... Qs>
-__device__ __forceinline__ void stripe_pairs(floatx16 (&acc)[MT][NACC], bf16x8 (&a)[2][MT], bf16x8 (&b)[3],
+template <int MT, int NTW, int BK, bool TR, int NACC, int J0, int JS, typename Loader, typename FragRow, int AMT, int... Qs>
+__device__ __forceinline__ void stripe_pairs(floatx16 (&acc)[AMT][NACC], bf16x8 (&a)[2][MT], bf16x8 (&b)[3],
                                              const bf16_t* a0, int astride, const bf16_t* bstage, int pos0,
                                              FragRow frag_row, const Loader& ld, bool prefetch, int k_next,
                                              bf16_t* next_stage, std::integer_sequence<int, Qs...>) {
@@ -185,8 +185,9 @@ __device__ __forceinline__ void stripe_pairs(floatx16 (&acc)[MT][NACC], bf16x8 (
 // fragment of sub-step 0 for M tile 0 (position pos0 of its row; sub-step s sits at pos0 ^ 16s, M tile
 // mt `astride` elements further); bstage: this lane's row of the B stage (N tile 0).  The NTW tiles multiplied
 // here are columns J0, J0+JS, .. of an accumulator array NACC tiles wide.
-template <int MT, int NTW, int BK, bool TR, int NACC = NTW, int J0 = 0, int JS = 1, typename Loader, typename FragRow>
-__device__ __forceinline__ void stripe_step(floatx16 (&acc)[MT][NACC], const bf16_t* a0, int astride, const bf16_t* bstage,
+// The accumulator array may have more M tiles (AMT) than the MT that are multiplied: the first MT are.
+template <int MT, int NTW, int BK, bool TR, int NACC = NTW, int J0 = 0, int JS = 1, typename Loader, typename FragRow, int AMT>
+__device__ __forceinline__ void stripe_step(floatx16 (&acc)[AMT][NACC], const bf16_t* a0, int astride, const bf16_t* bstage,
                                             int pos0, FragRow frag_row, const Loader& ld, bool prefetch, int k_next,
                                             bf16_t* next_stage) {
   constexpr int SS = BK / 16;
