@@ -287,8 +287,8 @@ int backward_check(const bibo_moe_shape* sh, int norm_mode) {
   const int rc = check_dims(sh->T, sh->H, sh->E, sh->k, sh->I, sh->dtype, sh->n_pos, sh->n_neg);
   if (rc != BIBO_OK) return rc;
   if (norm_mode < BIBO_NORM_NONE || norm_mode > BIBO_NORM_SOFTMAX || !act_ok(sh->act)) return BIBO_ERR_UNSUPPORTED;
-  // bf16, GLU experts only, dimensions the MFMA tiles divide
-  if (sh->n_pos + sh->n_neg > 0 || !backward_supported(sh->H, sh->I, sh->k, sh->dtype)) return BIBO_ERR_UNSUPPORTED;
+  // bf16, dimensions the MFMA tiles divide
+  if (!backward_supported(sh->H, sh->I, sh->k, sh->dtype)) return BIBO_ERR_UNSUPPORTED;
   return BIBO_OK;
 }
 
@@ -572,7 +572,8 @@ int bibo_moe_backward(const void* x, const void* d_out, const void* w_router, co
   b.dwr_part = reinterpret_cast<float*>(base + ws.dwr_part);
   b.pad_off = reinterpret_cast<int32_t*>(base + ws.pad_off);
   return hip_rc(launch_backward(x, d_out, w_router, w_gate_up, w_down, theta, logits, idx, w, offsets, perm_slot, perm_token,
-                                T, H, E, k, I, norm_mode, sh->act, b, d_x, d_w_router, d_w_gate_up, d_w_down, d_theta, s));
+                                T, H, E - sh->n_pos - sh->n_neg, sh->n_pos, sh->n_neg, k, I, norm_mode, sh->act, b, d_x,
+                                d_w_router, d_w_gate_up, d_w_down, d_theta, s));
 }
 
 int bibo_moe_experts_backward(const void* x, const void* d_out, const int32_t* idx, const float* w, const void* w_gate_up,
@@ -609,7 +610,8 @@ int bibo_moe_experts_backward(const void* x, const void* d_out, const int32_t* i
   b.dwr_part = reinterpret_cast<float*>(base + ws.dwr_part);
   b.pad_off = reinterpret_cast<int32_t*>(base + ws.pad_off);
   return hip_rc(launch_backward(x, d_out, nullptr, w_gate_up, w_down, theta, nullptr, idx, w, offsets, perm_slot, perm_token,
-                                T, H, E, k, I, BIBO_NORM_SUM, sh->act, b, d_x, nullptr, d_w_gate_up, d_w_down, d_theta, s));
+                                T, H, E - sh->n_pos - sh->n_neg, sh->n_pos, sh->n_neg, k, I, BIBO_NORM_SUM, sh->act, b, d_x,
+                                nullptr, d_w_gate_up, d_w_down, d_theta, s));
 }
 
 int bibo_moe_exp_attn_res_fwd(const void* const* candidates, int n_candidates, const float* score_weight, float eps, int T, int H,

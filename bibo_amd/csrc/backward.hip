@@ -312,7 +312,7 @@ __global__ __launch_bounds__(256) void act_bwd_kernel(const bf16_t* __restrict__
                                                       float* __restrict__ dw_slot, float* __restrict__ dtheta_row) {
   const int lane = threadIdx.x & 63;
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (row >= S) return;
+  if (row >= S || row >= offsets[E]) return;                   // E = GLU experts: rows behind theirs have no activation
   int e = 0;
   {                                                            // expert of the row: offsets[e] <= row < offsets[e + 1]
     int lo = 0, hi = E;
@@ -384,6 +384,39 @@ __global__ __launch_bounds__(256) void act_bwd_kernel(const bf16_t* __restrict__
     const float dp = act == BIBO_ACT_RADIAL_TANH ? 1.f - p * p : p * (1.f - p);
     dtheta_row[row] = radial ? dp * __logf(r) * gain * sum_qa : 0.f;
   }
+}
+
+// +/-Identity experts (moe.py:95-99): a slot routed to one contributes sign w x[t] to the output, so
+//   dw[slot] = sign <d_out[t], x[t]>,  dx_slot[slot] = sign w[slot] d_out[t]
+// (the per-slot dx rows are summed over a token's slots by dx_combine_kernel like those of the GLU experts).
+// One wave per permuted row behind the GLU experts' rows: rows offsets[Eg] .. offsets[Eg + n_pos + n_neg).
+__global__ __launch_bounds__(256) void special_bwd_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ d_out,
+                                                          const float* __restrict__ w, const int32_t* __restrict__ offsets,
+                                                          const int32_t* __restrict__ perm_slot,
+                                                          const int32_t* __restrict__ perm_token, int Eg, int n_pos,
+                                                          int n_neg, int H, float* __restrict__ dw_slot,
+                                                          bf16_t* __restrict__ dxs) {
+  const int lane = threadIdx.x & 63;
+  const int row = offsets[Eg] + blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= offsets[Eg + n_pos + n_neg]) return;
+  const float sign = row < offsets[Eg + n_pos] ? 1.f : -1.f;
+  const int slot = perm_slot[row];
+  const size_t t = (size_t)perm_token[row];
+  const float sw = sign * w[slot];
+  float dot = 0.f;
+  for (int c = lane * 8; c < H; c += 64 * 8) {
+    const bf16x8 xv = *reinterpret_cast<const bf16x8*>(x + t * H + c);
+    const bf16x8 dv = *reinterpret_cast<const bf16x8*>(d_out + t * H + c);
+    bf16x8 o;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      dot = fmaf((float)dv[q], (float)xv[q], dot);
+      o[q] = (bf16_t)(sw * (float)dv[q]);
+    }
+    *reinterpret_cast<bf16x8*>(dxs + (size_t)slot * H + c) = o;
+  }
+  dot = wave_sum(dot);
+  if (lane == 0) dw_slot[slot] = sign * dot;
 }
 
 // dtheta[e] = sum of its rows' contributions, in a fixed order (no atomics: the same bits on every call).
@@ -526,8 +559,10 @@ size_t backward_padded_rows(int T, int E, int k) { return ((size_t)T * k + (size
 hipError_t launch_backward(const void* x, const void* d_out, const void* w_router, const void* wgu, const void* wd,
                            const float* theta, const float* logits, const int32_t* idx, const float* w,
                            const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token, int T, int H, int E,
-                           int k, int I, int norm_mode, int act, const BackwardBuffers& b, void* dx, void* d_w_router,
-                           void* d_wgu, void* d_wd, float* d_theta, hipStream_t s) {
+                           int n_pos, int n_neg, int k, int I, int norm_mode, int act, const BackwardBuffers& b, void* dx,
+                           void* d_w_router, void* d_wgu, void* d_wd, float* d_theta, hipStream_t s) {
+  // E = GLU experts (with weights); the router and the permutation know Et experts, the +/-Identity ones last
+  const int Et = E + n_pos + n_neg;
   const int S = T * k;
   const bf16_t* xp = static_cast<const bf16_t*>(x);
   const bf16_t* dop = static_cast<const bf16_t*>(d_out);
@@ -541,11 +576,11 @@ hipError_t launch_backward(const void* x, const void* d_out, const void* w_route
   bf16_t* dxs = static_cast<bf16_t*>(b.dxs);
   bf16_t* p_t = static_cast<bf16_t*>(b.p_t);
   bf16_t* q_t = static_cast<bf16_t*>(b.q_t);
-  const int ld = (int)backward_padded_rows(T, E, k);
+  const int ld = (int)backward_padded_rows(T, Et, k);
   hipError_t err = hipSuccess;
   if (S == 0) {
     zero_bytes(d_theta, (size_t)E * sizeof(float), s);
-    if (d_w_router != nullptr) zero_bytes(d_w_router, (size_t)E * H * sizeof(bf16_t), s);
+    if (d_w_router != nullptr) zero_bytes(d_w_router, (size_t)Et * H * sizeof(bf16_t), s);
     zero_bytes(d_wgu, (size_t)E * 2 * I * H * sizeof(bf16_t), s);
     zero_bytes(d_wd, (size_t)E * H * I * sizeof(bf16_t), s);
     return hipGetLastError();
@@ -567,16 +602,19 @@ hipError_t launch_backward(const void* x, const void* d_out, const void* w_route
   // dx of every slot, in slot order: [dg, du] W_gate_up
   err = launch_ggemm<false, true>(dgu, nullptr, wgu_t, offsets, perm_slot, S, 2 * I, H, E, dxs, s);
   if (err != hipSuccess) return err;
+  if (n_pos + n_neg > 0)   // (as many waves as there could be rows: how many there are is only known on the device)
+    hipLaunchKernelGGL(special_bwd_kernel, dim3((S + 3) / 4), dim3(256), 0, s, xp, dop, w, offsets, perm_slot, perm_token, E,
+                       n_pos, n_neg, H, b.dw_slot, dxs);
   const bool with_router = w_router != nullptr;      // else: the experts alone, the caller owns the routing
   if (with_router)
-    hipLaunchKernelGGL(router_bwd_kernel, dim3((T + 255) / 256), dim3(256), 0, s, logits, idx, w, b.dw_slot, T, E, k, norm_mode,
+    hipLaunchKernelGGL(router_bwd_kernel, dim3((T + 255) / 256), dim3(256), 0, s, logits, idx, w, b.dw_slot, T, Et, k, norm_mode,
                        b.dl);
   hipLaunchKernelGGL(dx_combine_kernel, dim3((unsigned)(((long long)T * (H / 8) + 255) / 256)), dim3(256), 0, s, dxs,
                      with_router ? b.dl : nullptr, idx, wrp, T, H, k, static_cast<bf16_t*>(dx));
   if (with_router) {
-    hipLaunchKernelGGL(dwr_partial_kernel, dim3((H + 255) / 256, E, kDwrSplit), dim3(256), 0, s, xp, b.dl, offsets, perm_slot,
+    hipLaunchKernelGGL(dwr_partial_kernel, dim3((H + 255) / 256, Et, kDwrSplit), dim3(256), 0, s, xp, b.dl, offsets, perm_slot,
                        perm_token, H, b.dwr_part);
-    hipLaunchKernelGGL(dwr_sum_kernel, dim3((E * H + 255) / 256), dim3(256), 0, s, b.dwr_part, H, E * H,
+    hipLaunchKernelGGL(dwr_sum_kernel, dim3((Et * H + 255) / 256), dim3(256), 0, s, b.dwr_part, H, Et * H,
                        static_cast<bf16_t*>(d_w_router));
   }
   // weight gradients: dW_down[e] = (w d)^T h, dW_gate_up[e] = [dg, du]^T x, contracted over the expert's rows

@@ -207,7 +207,7 @@ int backward_dwr_split();
 hipError_t launch_backward(const void* x, const void* d_out, const void* w_router, const void* wgu, const void* wd,
                            const float* theta, const float* logits, const int32_t* idx, const float* w,
                            const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token, int T, int H, int E,
-                           int k, int I, int norm_mode, int act, const BackwardBuffers& b, void* dx, void* d_w_router,
-                           void* d_wgu, void* d_wd, float* d_theta, hipStream_t s);
+                           int n_pos, int n_neg, int k, int I, int norm_mode, int act, const BackwardBuffers& b, void* dx,
+                           void* d_w_router, void* d_wgu, void* d_wd, float* d_theta, hipStream_t s);
 
 }  // namespace bibo

@@ -33,14 +33,15 @@ class _MoELayerFn(torch.autograd.Function):
     gets none (router.py:38).  The per-expert row counts come out as a second, non-differentiable result."""
 
     @staticmethod
-    def forward(ctx, x, w_router, w_gate_up, w_down, theta, bias, k, norm, act, algo, want_counts):
+    def forward(ctx, x, w_router, w_gate_up, w_down, theta, bias, k, norm, act, algo, want_counts, n_pos=0, n_neg=0):
         cd = torch.bfloat16
         cast = lambda t, d: (t if t.dtype == d else t.to(d)).contiguous()
         xb, wr, gu, dn = cast(x.detach(), cd), cast(w_router.detach(), cd), cast(w_gate_up.detach(), cd), cast(w_down.detach(), cd)
         th, b = cast(theta.detach(), torch.float32), cast(bias.detach(), torch.float32)
-        out, _, _, counts, _ = ops.moe_forward(xb, wr, b, gu, dn, th, k, norm=norm, algo=algo, want_counts=want_counts, act=act)
+        out, _, _, counts, _ = ops.moe_forward(xb, wr, b, gu, dn, th, k, norm=norm, algo=algo, want_counts=want_counts, act=act,
+                                               n_pos=n_pos, n_neg=n_neg)
         ctx.save_for_backward(xb, wr, gu, dn, th, b)
-        ctx.conf = (k, norm, act)
+        ctx.conf = (k, norm, act, n_pos, n_neg)
         ctx.in_dtypes = (x.dtype, w_router.dtype, w_gate_up.dtype, w_down.dtype, theta.dtype)
         if counts is None:
             counts = torch.empty(0, dtype=torch.int32, device=x.device)
@@ -50,10 +51,10 @@ class _MoELayerFn(torch.autograd.Function):
     @staticmethod
     def backward(ctx, d_out, _d_counts):
         xb, wr, gu, dn, th, b = ctx.saved_tensors
-        k, norm, act = ctx.conf
+        k, norm, act, n_pos, n_neg = ctx.conf
         d = d_out.to(torch.bfloat16).contiguous()
-        grads = ops.moe_backward(xb, d, wr, b, gu, dn, th, k, norm=norm, act=act)[:5]
-        return tuple(g.to(dt) for g, dt in zip(grads, ctx.in_dtypes)) + (None,) * 6
+        grads = ops.moe_backward(xb, d, wr, b, gu, dn, th, k, norm=norm, act=act, n_pos=n_pos, n_neg=n_neg)[:5]
+        return tuple(g.to(dt) for g, dt in zip(grads, ctx.in_dtypes)) + (None,) * 8
 
 
 class _ExpertsFn(torch.autograd.Function):
@@ -61,14 +62,15 @@ class _ExpertsFn(torch.autograd.Function):
     = bibo_moe_experts_backward.  The gradient of the combine weights (moe.py:93) flows back to whoever made them."""
 
     @staticmethod
-    def forward(ctx, x, top_w, w_gate_up, w_down, theta, idx, act, algo, want_counts):
+    def forward(ctx, x, top_w, w_gate_up, w_down, theta, idx, act, algo, want_counts, n_pos=0, n_neg=0):
         cd = torch.bfloat16
         cast = lambda t, d: (t if t.dtype == d else t.to(d)).contiguous()
         xb, gu, dn = cast(x.detach(), cd), cast(w_gate_up.detach(), cd), cast(w_down.detach(), cd)
         th, w = cast(theta.detach(), torch.float32), cast(top_w.detach(), torch.float32)
-        out, counts = ops.experts_fwd(xb, idx, w, gu, dn, th, algo=algo, want_counts=want_counts, act=act)
+        out, counts = ops.experts_fwd(xb, idx, w, gu, dn, th, algo=algo, want_counts=want_counts, act=act, n_pos=n_pos,
+                                      n_neg=n_neg)
         ctx.save_for_backward(xb, w, gu, dn, th, idx)
-        ctx.act = act
+        ctx.act, ctx.specials = act, (n_pos, n_neg)
         ctx.in_dtypes = (x.dtype, top_w.dtype, w_gate_up.dtype, w_down.dtype, theta.dtype)
         if counts is None:
             counts = torch.empty(0, dtype=torch.int32, device=x.device)
@@ -78,13 +80,14 @@ class _ExpertsFn(torch.autograd.Function):
     @staticmethod
     def backward(ctx, d_out, _d_counts):
         xb, w, gu, dn, th, idx = ctx.saved_tensors
-        grads = ops.experts_backward(xb, d_out.to(torch.bfloat16).contiguous(), idx, w, gu, dn, th, act=ctx.act)
-        return tuple(g.to(dt) for g, dt in zip(grads, ctx.in_dtypes)) + (None,) * 4
+        grads = ops.experts_backward(xb, d_out.to(torch.bfloat16).contiguous(), idx, w, gu, dn, th, act=ctx.act,
+                                     n_pos=ctx.specials[0], n_neg=ctx.specials[1])
+        return tuple(g.to(dt) for g, dt in zip(grads, ctx.in_dtypes)) + (None,) * 6
 
 
 def _backward_covers(experts) -> bool:
-    return (experts.num_pos + experts.num_neg == 0 and experts.hidden_size % 128 == 0
-            and experts.intermediate_size % 128 == 0 and experts.intermediate_size <= 512)
+    return (experts.hidden_size % 128 == 0 and experts.intermediate_size % 128 == 0
+            and experts.intermediate_size <= 512)
 
 
 class _CastCache:
@@ -251,11 +254,11 @@ class BiBoFusedExperts(nn.Module):
                 raise RuntimeError("the backward pass runs in bf16: use bf16 activations or bf16 autocast, or call the "
                                    "experts under torch.no_grad()")
             if not _backward_covers(self):
-                raise NotImplementedError("the backward pass covers GLU experts only (no +/-Identity experts), hidden and "
-                                          "expert sizes that are multiples of 128 and expert size <= 512")
+                raise NotImplementedError("the backward pass covers hidden and expert sizes that are multiples of 128 and "
+                                          "expert size <= 512")
             out, counts = _ExpertsFn.apply(hidden_states, top_k_weights, self.gate_up_proj, self.down_proj, self.radial_theta,
                                            top_k_indices.detach().to(torch.int32).contiguous(), self.act, self.algo,
-                                           _want_counts)
+                                           _want_counts, self.num_pos, self.num_neg)
             out = out if out.dtype == hidden_states.dtype else out.to(hidden_states.dtype)
             return (out, counts) if _want_counts else out
         cd = _compute_dtype(hidden_states)
@@ -424,11 +427,11 @@ class BiBoMoELayer(nn.Module):
             raise RuntimeError("the backward pass runs in bf16: use bf16 activations or bf16 autocast, or call the layer "
                                "under torch.no_grad()")
         if not _backward_covers(e):
-            raise NotImplementedError("the backward pass covers GLU experts only (no +/-Identity experts), hidden and "
-                                      "expert sizes that are multiples of 128 and expert size <= 512")
+            raise NotImplementedError("the backward pass covers hidden and expert sizes that are multiples of 128 and "
+                                      "expert size <= 512")
         out, counts = _MoELayerFn.apply(x, self.gate.gate_proj.weight, e.gate_up_proj, e.down_proj, e.radial_theta,
                                         self.gate.bias, self.num_experts_per_tok, self.gate.norm_topk_prob, e.act, e.algo,
-                                        want_counts)
+                                        want_counts, e.num_pos, e.num_neg)
         return out, (counts if want_counts else None)
 
     @_no_compile

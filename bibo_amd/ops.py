@@ -288,23 +288,27 @@ def moe_forward_static(x, w_router, bias, w_gate_up, w_down, theta, k, out, norm
     return out
 
 
-def moe_backward(x, d_out, w_router, bias, w_gate_up, w_down, theta, k, norm="sum", act="radial", want_dw=False):
+def moe_backward(x, d_out, w_router, bias, w_gate_up, w_down, theta, k, norm="sum", act="radial", want_dw=False,
+                 n_pos=0, n_neg=0):
     """Gradients of the layer (bibo_moe_backward) for the upstream gradient d_out [T,H] of its output: what autograd
-    derives for BiBoMoELayer.forward (moe.py:157-183) with the selection held fixed.
-    -> d_x [T,H], d_w_router [E,H], d_w_gate_up [E,2I,H], d_w_down [E,H,I] (x.dtype), d_theta fp32 [E], d_w fp32 [T,k]|None."""
+    derives for BiBoMoELayer.forward (moe.py:157-183) with the selection held fixed.  w_router / bias have
+    E = Eg + n_pos + n_neg rows, the expert weights Eg (see experts_fwd).
+    -> d_x [T,H], d_w_router [E,H], d_w_gate_up [Eg,2I,H], d_w_down [Eg,H,I] (x.dtype), d_theta fp32 [Eg],
+    d_w fp32 [T,k]|None."""
     T, H = x.shape
-    E, two_i, _ = w_gate_up.shape
+    Eg, two_i, _ = w_gate_up.shape
+    E = Eg + n_pos + n_neg
     I = two_i // 2
     dc = _dtype_code(x)
     _chk(x, "x"); _chk(d_out, "d_out", x.dtype, (T, H)); _chk(w_router, "w_router", x.dtype, (E, H))
-    _chk(bias, "bias", torch.float32, (E,)); _chk(w_gate_up, "w_gate_up", x.dtype, (E, 2 * I, H))
-    _chk(w_down, "w_down", x.dtype, (E, H, I)); _chk(theta, "theta", torch.float32, (E,))
+    _chk(bias, "bias", torch.float32, (E,)); _chk(w_gate_up, "w_gate_up", x.dtype, (Eg, 2 * I, H))
+    _chk(w_down, "w_down", x.dtype, (Eg, H, I)); _chk(theta, "theta", torch.float32, (Eg,))
     dev = x.device
     d_x = torch.empty_like(x)
     d_wr, d_gu, d_dn = torch.empty_like(w_router), torch.empty_like(w_gate_up), torch.empty_like(w_down)
-    d_theta = torch.empty(E, dtype=torch.float32, device=dev)
+    d_theta = torch.empty(Eg, dtype=torch.float32, device=dev)
     d_w = torch.empty(T, k, dtype=torch.float32, device=dev) if want_dw else None
-    sh = L.Shape(T, H, E, k, I, dc, 0, 0, act_code(act), 0)
+    sh = L.Shape(T, H, E, k, I, dc, n_pos, n_neg, act_code(act), 0)
     nbytes = ctypes.c_size_t(0)
     L.check(L.lib().bibo_moe_backward_workspace_bytes(ctypes.byref(sh), ctypes.byref(nbytes)), "bibo_moe_backward_workspace_bytes")
     ws = workspace(dev, nbytes.value)
@@ -316,11 +320,12 @@ def moe_backward(x, d_out, w_router, bias, w_gate_up, w_down, theta, k, norm="su
     return d_x, d_wr, d_gu, d_dn, d_theta, d_w
 
 
-def experts_backward(x, d_out, idx, w, w_gate_up, w_down, theta, act="radial"):
-    """bibo_moe_experts_backward: gradients of experts_fwd for a caller-owned routing (idx int32 [T,k], w fp32 [T,k]).
-    -> d_x [T,H], d_w fp32 [T,k], d_w_gate_up, d_w_down (x.dtype), d_theta fp32 [E]."""
+def experts_backward(x, d_out, idx, w, w_gate_up, w_down, theta, act="radial", n_pos=0, n_neg=0):
+    """bibo_moe_experts_backward: gradients of experts_fwd for a caller-owned routing (idx int32 [T,k], w fp32 [T,k];
+    expert ids Eg .. Eg+n_pos-1 are +Identity, the next n_neg -Identity, as in experts_fwd).
+    -> d_x [T,H], d_w fp32 [T,k], d_w_gate_up, d_w_down (x.dtype), d_theta fp32 [Eg]."""
     T, H = x.shape
-    E, two_i, _ = w_gate_up.shape
+    E, two_i, _ = w_gate_up.shape          # GLU experts
     I = two_i // 2
     k = idx.shape[1]
     dc = _dtype_code(x)
@@ -331,7 +336,7 @@ def experts_backward(x, d_out, idx, w, w_gate_up, w_down, theta, act="radial"):
     d_x, d_gu, d_dn = torch.empty_like(x), torch.empty_like(w_gate_up), torch.empty_like(w_down)
     d_w = torch.empty(T, k, dtype=torch.float32, device=dev)
     d_theta = torch.empty(E, dtype=torch.float32, device=dev)
-    sh = L.Shape(T, H, E, k, I, dc, 0, 0, act_code(act), 0)
+    sh = L.Shape(T, H, E + n_pos + n_neg, k, I, dc, n_pos, n_neg, act_code(act), 0)
     nbytes = ctypes.c_size_t(0)
     L.check(L.lib().bibo_moe_backward_workspace_bytes(ctypes.byref(sh), ctypes.byref(nbytes)), "bibo_moe_backward_workspace_bytes")
     ws = workspace(dev, nbytes.value)

@@ -267,10 +267,13 @@ int bibo_moe_ffn_forward(const void* h, const float* norm_weight, float eps, con
  * the selection, router.py:38, and gets no gradient; nor does anything flow through which experts were chosen).
  * x is the block's input as in bibo_moe_forward; the routing is recomputed from it by the forward's router kernel,
  * so the selection and the combine weights are those of the forward call on the same operands.
- *   d_x [T,H], d_w_router [E,H], d_w_gate_up [E,2I,H], d_w_down [E,H,I] in `dtype`; d_theta fp32 [E]
+ *   d_x [T,H], d_w_router [E,H], d_w_gate_up [Eg,2I,H], d_w_down [Eg,H,I] in `dtype`; d_theta fp32 [Eg], with
+ *   Eg = E - n_pos - n_neg GLU experts
  *   (reference pins: theta receives gradient, tests/test_moe.py:53-63, ablate/common/test_eager_radial.py:63-69);
  *   d_w_out fp32 [T,k] or NULL: gradient with respect to the combine weights (router.py:47), for inspection.
- * bf16 only, H and I multiples of 128, I <= 512, no +/-Identity experts (BIBO_ERR_UNSUPPORTED otherwise); the
+ * A slot routed to a +/-Identity expert (moe.py:95-99) sends +/- w d_out[t] to d_x and +/- <d_out[t], x[t]> to its
+ * combine weight, and through that to the router.
+ * bf16 only, H and I multiples of 128, I <= 512 (BIBO_ERR_UNSUPPORTED otherwise); the
  * intermediate activations are recomputed, nothing has to be kept from the forward call.  All gradients are
  * overwritten, not accumulated.  Workspace: bibo_moe_backward_workspace_bytes (about 14 bytes per routed slot and
  * column plus one transposed copy of the expert weights).

@@ -41,6 +41,66 @@ def test_backward_matches_oracle(T, H, E, k, I):
         assert _rel(got[name], ref[name]) <= TOL, (name, _rel(got[name], ref[name]))
 
 
+@pytest.mark.parametrize("T,H,Eg,n_pos,n_neg,k,I,norm", [(300, 256, 6, 1, 1, 3, 128, "sum"), (1000, 768, 62, 1, 1, 6, 384, "sum"),
+                                                         (200, 256, 5, 2, 0, 4, 128, "softmax"), (64, 384, 3, 0, 2, 2, 256, False)])
+def test_backward_with_identity_experts_matches_oracle(T, H, Eg, n_pos, n_neg, k, I, norm):
+    """+/-Identity experts (moe.py:95-99, on by default in the reference's configuration): a slot routed to one sends
+    +/- w d_out to d_x and +/- <d_out, x> to its combine weight, hence to the router; its router row gets a gradient,
+    the GLU experts' tensors keep their shapes."""
+    E = Eg + n_pos + n_neg
+    p = O.make_inputs(T=T, H=H, E=Eg, k=k, I=I, theta="normal", seed=T + E)
+    g = torch.Generator().manual_seed(T)
+    p["w_router"] = (torch.randn(E, H, generator=g) * 0.02).bfloat16()
+    p["bias"] = torch.rand(E, generator=g) * 0.02 - 0.01
+    p["bias"][Eg:] += 0.05                                         # the specials get their share of the slots
+    d_out = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    dev = lambda t: t.to(DEV)
+    args = [dev(p[n]) for n in ("w_router", "bias", "w_gate_up", "w_down", "theta")]
+    _, idx, w, _, _ = ops.moe_forward(dev(p["x"]), *args, k, norm=norm, want_routing=True, n_pos=n_pos, n_neg=n_neg)
+    got = ops.moe_backward(dev(p["x"]), dev(d_out), *args, k, norm=norm, want_dw=True, n_pos=n_pos, n_neg=n_neg)
+    torch.cuda.synchronize()
+    idx = idx.cpu().numpy()
+    assert (idx >= Eg).sum() > 0                                   # the case does route to specials
+    ref = O.moe_backward(p["x"], p["w_router"], p["w_gate_up"], p["w_down"], p["theta"], idx, d_out, norm=norm, n_pos=n_pos,
+                         n_neg=n_neg)
+    got = dict(zip(("x", "w_router", "w_gate_up", "w_down", "theta", "w"), got))
+    assert got["w_router"].shape == (E, H) and got["w_gate_up"].shape == (Eg, 2 * I, H) and got["theta"].shape == (Eg,)
+    for name in ("w", "x", "w_down", "w_gate_up", "w_router", "theta"):
+        assert _rel(got[name], ref[name]) <= TOL, (name, _rel(got[name], ref[name]))
+    # the experts alone, with the routing as the caller's: same d_x up to the router's share, same d_w
+    gx, gw, ggu, gdn, gth = ops.experts_backward(dev(p["x"]), dev(d_out), dev(torch.from_numpy(idx)), w, dev(p["w_gate_up"]),
+                                                 dev(p["w_down"]), dev(p["theta"]), n_pos=n_pos, n_neg=n_neg)
+    torch.cuda.synchronize()
+    assert torch.equal(gw, got["w"]) and torch.equal(ggu, got["w_gate_up"]) and torch.equal(gdn, got["w_down"])
+
+
+def test_layer_with_identity_experts_trains():
+    """The reference's default configuration has one +Identity and one -Identity expert: the module's forward under
+    autograd reaches every parameter, with or without hooks on the submodules."""
+    from bibo_amd.config import BiBoMoEConfig
+    from bibo_amd.moe import BiBoMoELayer
+    layer = BiBoMoELayer(BiBoMoEConfig(hidden_size=256, moe_intermediate_size=128, num_routed_experts=8,
+                                       num_experts_per_tok=3, special_expert_pairs=1)).to(DEV).bfloat16()
+    assert layer.experts.num_pos == 1 and layer.experts.num_neg == 1
+    x = torch.randn(2, 40, 256, device=DEV, dtype=torch.bfloat16, requires_grad=True)
+    layer(x).float().square().sum().backward()
+    assert x.grad is not None and bool(torch.isfinite(x.grad.float()).all())
+    grads = {n: prm.grad.clone() for n, prm in layer.named_parameters() if prm.requires_grad}
+    assert all(g is not None and bool(torch.isfinite(g.float()).all()) for g in grads.values())
+    assert float(grads["gate.gate_proj.weight"][-2:].abs().max()) > 0      # the specials' router rows learn
+    # the same through the experts seam (a hook makes the layer call its submodules one by one)
+    for prm in layer.parameters():
+        prm.grad = None
+    hook = layer.experts.register_forward_hook(lambda m, a, o: None)
+    x2 = x.detach().clone().requires_grad_(True)
+    layer(x2).float().square().sum().backward()
+    hook.remove()
+    assert _rel(x2.grad, x.grad.cpu()) <= TOL
+    for n, prm in layer.named_parameters():
+        if prm.requires_grad:
+            assert _rel(prm.grad, grads[n].cpu()) <= TOL, n
+
+
 @pytest.mark.parametrize("norm,act", [("softmax", "radial"), (False, "tanh"), ("sum", "silu"), ("sum", "tanh")])
 def test_backward_norm_modes_and_activations(norm, act):
     got, ref, _ = _run(320, 256, 16, 3, 128, norm=norm, act=act, seed=7)
@@ -89,8 +149,8 @@ def test_backward_rejects_what_it_does_not_cover():
     sh = L.Shape(64, 200, 8, 2, 128, L.DTYPE_BF16)                  # H no multiple of 128
     n = ctypes.c_size_t(0)
     assert L.lib().bibo_moe_backward_workspace_bytes(ctypes.byref(sh), ctypes.byref(n)) == -6
-    sh = L.Shape(64, 256, 8, 2, 128, L.DTYPE_BF16, 1, 1)            # +/-Identity experts
-    assert L.lib().bibo_moe_backward_workspace_bytes(ctypes.byref(sh), ctypes.byref(n)) == -6
+    sh = L.Shape(64, 256, 8, 2, 128, L.DTYPE_BF16, 1, 1)            # +/-Identity experts are covered
+    assert L.lib().bibo_moe_backward_workspace_bytes(ctypes.byref(sh), ctypes.byref(n)) == 0 and n.value > 0
     sh = L.Shape(64, 256, 8, 2, 128, L.DTYPE_F32)
     assert L.lib().bibo_moe_backward_workspace_bytes(ctypes.byref(sh), ctypes.byref(n)) == -6
 
@@ -162,11 +222,11 @@ def test_seam_and_shared_expert_under_autograd():
 def test_what_the_backward_does_not_cover_is_refused():
     from bibo_amd.config import BiBoMoEConfig
     from bibo_amd.moe import BiBoMoELayer
-    layer = BiBoMoELayer(BiBoMoEConfig(hidden_size=256, moe_intermediate_size=128, num_routed_experts=8,
-                                       num_experts_per_tok=2, special_expert_pairs=1)).to(DEV).bfloat16()
-    x = torch.randn(1, 8, 256, device=DEV, dtype=torch.bfloat16)
+    layer = BiBoMoELayer(BiBoMoEConfig(hidden_size=192, moe_intermediate_size=128, num_routed_experts=8,
+                                       num_experts_per_tok=2)).to(DEV).bfloat16()
+    x = torch.randn(1, 8, 192, device=DEV, dtype=torch.bfloat16)
     with pytest.raises(NotImplementedError):
-        layer(x)                                                   # +/-Identity experts: forward only
+        layer(x)                                                   # hidden size no multiple of 128: forward only
     with torch.no_grad():
         layer(x)
     fp32 = _layer().float()

@@ -393,6 +393,42 @@ def test_backward_matches_central_differences(act, norm):
         assert abs(fd - an) <= 1e-6 * max(1.0, abs(an)), (name, fd, an)
 
 
+def test_backward_with_identity_experts_closed_form_and_differences():
+    """+/-Identity experts (moe.py:95-99): out[t] += sign w[t,j] x[t] for a slot routed to one.  Closed form for the
+    part of the gradients that comes from those slots alone: dw[t,j] = sign <d_out[t], x[t]>, and the x gradient of
+    that term is sign w[t,j] d_out[t]; the whole gradient agrees with central differences."""
+    T, H, Eg, k, I = 20, 16, 3, 3, 8
+    n_pos, n_neg = 1, 1
+    E = Eg + n_pos + n_neg
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(T, H, generator=g, dtype=torch.float64)
+    wr = torch.randn(E, H, generator=g, dtype=torch.float64) * 0.3
+    gu = torch.randn(Eg, 2 * I, H, generator=g, dtype=torch.float64) * 0.3
+    dn = torch.randn(Eg, H, I, generator=g, dtype=torch.float64) * 0.3
+    th = torch.randn(Eg, generator=g, dtype=torch.float64)
+    d_out = torch.randn(T, H, generator=g, dtype=torch.float64)
+    idx, _, _ = O.route_from_logits((x @ wr.t()).float().numpy(), np.zeros(E, np.float32), k, "sum")
+    assert (idx >= Eg).any() and (idx == Eg).any() and (idx == Eg + 1).any()
+    grads = O.moe_backward(x, wr, gu, dn, th, idx, d_out, norm="sum", n_pos=n_pos, n_neg=n_neg)
+    dot = (d_out * x).sum(-1)
+    for t in range(T):
+        for j in range(k):
+            if idx[t, j] >= Eg:
+                sign = 1.0 if idx[t, j] < Eg + n_pos else -1.0
+                assert abs(float(grads["w"][t, j]) - sign * float(dot[t])) <= 1e-12 * max(1.0, abs(float(dot[t])))
+
+    def loss(xv, wrv):
+        w = O.route_weights(xv @ wrv.t(), idx, "sum")
+        return float((O.experts_forward(xv, idx, w, gu, dn, th, dtype=torch.float64, n_pos=n_pos, n_neg=n_neg) * d_out).sum())
+    for name, base in (("x", x), ("w_router", wr)):
+        d = torch.randn(base.shape, generator=g, dtype=torch.float64)
+        h = 1e-6
+        lp = loss(x + h * d, wr) if name == "x" else loss(x, wr + h * d)
+        lm = loss(x - h * d, wr) if name == "x" else loss(x, wr - h * d)
+        fd, an = (lp - lm) / (2 * h), float((grads[name] * d).sum())
+        assert abs(fd - an) <= 1e-6 * max(1.0, abs(an)), (name, fd, an)
+
+
 def test_radial_backward_closed_form():
     """h = r^p SiLU(g/r) u, r = sqrt(mean(g^2) + eps), p = sigmoid(theta).  With a = SiLU(z), a' = s (1 + z (1 - s)),
     s = sigmoid(z), z = g / r and q = dh u (all per element):
