@@ -225,6 +225,31 @@ def test_fused_kernel_matches_oracle_and_the_two_kernel_family(T, H, I, k, bias)
     assert rel_err(out, two) <= 1e-2
 
 
+@pytest.mark.parametrize("H,I", [(768, 384), (512, 256), (256, 128)])
+def test_fused_kernel_tiles_of_every_height(H, I):
+    """The fused kernel has one code path per number of 32-row blocks a tile holds (1 to 4) and leaves the missing
+    blocks out of all three phases: experts with 1, 31, 32, 33, 64, 65, 96, 97, 128, 129, 160 and 200 rows make last
+    tiles of every height next to full ones, and every row still matches the oracle and the generic family."""
+    counts = [1, 31, 32, 33, 64, 65, 96, 97, 128, 129, 160, 200, 0, 5]
+    E, k = len(counts), 1
+    T = sum(counts)
+    p = O.make_inputs(T=T, H=H, E=E, k=k, I=I, theta="normal", seed=H + I)
+    rng = np.random.default_rng(H)
+    idx = np.repeat(np.arange(E, dtype=np.int32), counts)
+    rng.shuffle(idx)
+    idx = idx.reshape(T, 1)
+    w = rng.uniform(0.2, 1.0, size=(T, 1)).astype(np.float32)
+    ref = O.experts_forward(p["x"], idx, w, p["w_gate_up"], p["w_down"], p["theta"])
+    out, cnt = _gpu_experts(p, idx, w, "fused")
+    assert np.array_equal(cnt, np.asarray(counts))
+    assert rel_err(out, ref) <= BF16_TOL
+    # row by row, so that a block left out by mistake (zeros or stale rows) cannot hide behind a large row elsewhere
+    err = (out.double() - ref.double()).abs().amax(dim=1) / ref.double().abs().amax(dim=1).clamp_min(1e-30)
+    assert float(err.max()) <= 2 * BF16_TOL, int(err.argmax())
+    gen, _ = _gpu_experts(p, idx, w, "generic")
+    assert rel_err(out, gen) <= 1e-2
+
+
 def test_fused_stage_entry_points_compose_to_the_composite_call():
     """permute -> gateup_down -> combine through the stage ABI equals bibo_moe_experts_fwd(fused) bit for bit;
     the slot buffer holds w[t,j] * expert_j(x_t) (checked against the oracle per slot)."""
