@@ -420,8 +420,8 @@ class BiBoMoELayer(nn.Module):
 
     def _differentiable_forward(self, x: torch.Tensor, want_counts: bool):
         """x [T,H] -> (out [T,H] bf16 with an autograd graph, counts|None).  bf16 compute only (bf16 activations, or
-        fp32 activations under bf16 autocast), GLU experts only, H and I multiples of 128 and I <= 512: what
-        bibo_moe_backward covers."""
+        fp32 activations under bf16 autocast), H and I multiples of 128 and I <= 512, with or without +/-Identity
+        experts: what bibo_moe_backward covers."""
         e = self.experts
         if _compute_dtype(x) != torch.bfloat16:
             raise RuntimeError("the backward pass runs in bf16: use bf16 activations or bf16 autocast, or call the layer "
