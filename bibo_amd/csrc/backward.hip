@@ -20,10 +20,7 @@ namespace bibo {
 namespace {
 
 constexpr int kPad = 64;     // an expert's rows start at a multiple of this in the transposed buffers
-#ifndef BIBO_BWD_BK
-#define BIBO_BWD_BK 64
-#endif
-constexpr int kBwdBK = BIBO_BWD_BK;   // K elements per LDS stage of the GEMMs here: 64 = whole 128-byte lines per row
+constexpr int kBwdBK = 64;   // K elements per LDS stage of the GEMMs here: whole 128-byte lines per row
 
 // ---- grouped GEMM: out[dst(r), n] = sum_k A[src(r), k] W[e][n, k] for the rows r of expert e ------------------
 // src(r) = a_index[r] (GATHER) or r; dst(r) = out_index[r] (SCATTER) or r.  r runs over permuted rows.
@@ -455,10 +452,13 @@ __global__ void router_bwd_kernel(const float* __restrict__ logits, const int32_
 }
 
 // dx[t, c] = sum_j dxs[t k + j, c] + sum_j dl[t, j] W_router[idx[t, j], c]; one thread per 8 columns.  dl == NULL: the
-// slot rows alone (the experts without their router).
+// slot rows alone (the experts without their router).  A slot whose expert id lies outside [0, n_experts) (padding in
+// a caller's indices, which the forward pass skips) has no dxs row and no combine-weight gradient: it is left out of
+// the sum and its dw_slot entry is set to zero here.
 __global__ __launch_bounds__(256) void dx_combine_kernel(const bf16_t* __restrict__ dxs, const float* __restrict__ dl,
                                                          const int32_t* __restrict__ idx,
                                                          const bf16_t* __restrict__ w_router, int T, int H, int k,
+                                                         int n_experts, float* __restrict__ dw_slot,
                                                          bf16_t* __restrict__ dx) {
   const int gpr = H / 8;
   const long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -466,9 +466,14 @@ __global__ __launch_bounds__(256) void dx_combine_kernel(const bf16_t* __restric
   const int t = (int)(gid / gpr), c = (int)(gid - (long long)t * gpr) * 8;
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   for (int j = 0; j < k; ++j) {
+    const int e = idx[t * k + j];
+    if (e < 0 || e >= n_experts) {
+      if (c == 0) dw_slot[t * k + j] = 0.f;
+      continue;
+    }
     const bf16x8 v = *reinterpret_cast<const bf16x8*>(dxs + ((size_t)t * k + j) * H + c);
     if (dl != nullptr) {
-      const bf16x8 r = *reinterpret_cast<const bf16x8*>(w_router + (size_t)idx[t * k + j] * H + c);
+      const bf16x8 r = *reinterpret_cast<const bf16x8*>(w_router + (size_t)e * H + c);
       const float d = dl[t * k + j];
 #pragma unroll
       for (int q = 0; q < 8; ++q) acc[q] += (float)v[q] + d * (float)r[q];
@@ -610,7 +615,7 @@ hipError_t launch_backward(const void* x, const void* d_out, const void* w_route
     hipLaunchKernelGGL(router_bwd_kernel, dim3((T + 255) / 256), dim3(256), 0, s, logits, idx, w, b.dw_slot, T, Et, k, norm_mode,
                        b.dl);
   hipLaunchKernelGGL(dx_combine_kernel, dim3((unsigned)(((long long)T * (H / 8) + 255) / 256)), dim3(256), 0, s, dxs,
-                     with_router ? b.dl : nullptr, idx, wrp, T, H, k, static_cast<bf16_t*>(dx));
+                     with_router ? b.dl : nullptr, idx, wrp, T, H, k, Et, b.dw_slot, static_cast<bf16_t*>(dx));
   if (with_router) {
     hipLaunchKernelGGL(dwr_partial_kernel, dim3((H + 255) / 256, Et, kDwrSplit), dim3(256), 0, s, xp, b.dl, offsets, perm_slot,
                        perm_token, H, b.dwr_part);

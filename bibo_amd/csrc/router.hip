@@ -1,6 +1,8 @@
 // Kernel 1: fused router.  fp32 logits x @ w_router^T, canonical sigmoid, selection on score + bias
 // (ties to the lowest expert index), gather of the unbiased scores, normalisation.
 // Follows BiBoMoERouter.forward, src/modeling/ffn/router.py:25-51 of the reference.
+#include <mutex>
+
 #include "common.h"
 
 namespace bibo {
@@ -554,10 +556,33 @@ __global__ __launch_bounds__(256) void router_mfma_split_kernel(const bf16_t* __
 }  // namespace
 
 // The widest hidden size whose TOK raw rows fit LDS next to the w_router stages (TOK = 32: 64 KB of rows).
+constexpr int kNormRouterMaxH = 1024;
+
 bool router_norm_supported(int H, int dtype, const void* h, const void* w_router, const void* xn) {
   const bool aligned = ((reinterpret_cast<uintptr_t>(h) | reinterpret_cast<uintptr_t>(w_router) |
                          reinterpret_cast<uintptr_t>(xn)) & 15) == 0;
-  return dtype == BIBO_DTYPE_BF16 && (H % kRouterKC) == 0 && H <= 1024 && aligned;
+  return dtype == BIBO_DTYPE_BF16 && (H % kRouterKC) == 0 && H <= kNormRouterMaxH && aligned;
+}
+
+// Dynamic LDS beyond the default limit has to be allowed once per kernel and device (a host-side driver call without
+// a launch): done on the first call on a device, for the widest rows the kernel takes, and remembered, so that later
+// calls (one per layer and step, possibly under graph capture) go straight to the launch.
+constexpr int kMaxDevicesSeen = 64;
+std::mutex g_lds_mutex;
+bool g_lds_allowed[2][kMaxDevicesSeen] = {};
+
+template <int TOK>
+hipError_t allow_dynamic_lds() {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  const bool tracked = dev >= 0 && dev < kMaxDevicesSeen;
+  std::lock_guard<std::mutex> lock(g_lds_mutex);
+  if (tracked && g_lds_allowed[TOK == 32][dev]) return hipSuccess;
+  e = hipFuncSetAttribute(reinterpret_cast<const void*>(&router_norm_mfma_kernel<TOK>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)(TOK * kNormRouterMaxH * sizeof(bf16_t)));
+  if (e == hipSuccess && tracked) g_lds_allowed[TOK == 32][dev] = true;
+  return e;
 }
 
 // RMSNorm + router in one launch (see router_norm_mfma_kernel); `xn` receives the normalised rows.
@@ -569,19 +594,15 @@ hipError_t launch_router_norm(const void* h, const float* norm_weight, float eps
   const bf16_t* hp = static_cast<const bf16_t*>(h);
   const bf16_t* wp = static_cast<const bf16_t*>(w_router);
   bf16_t* xp = static_cast<bf16_t*>(xn);
+  hipError_t e;
   if (T >= 32 * 256) {
     const size_t shm = (size_t)32 * H * sizeof(bf16_t);
-    // (dynamic LDS has to be allowed per kernel and device; a host-side call without a launch)
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&router_norm_mfma_kernel<32>),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm);
-    if (e != hipSuccess) return e;
+    if ((e = allow_dynamic_lds<32>()) != hipSuccess) return e;
     hipLaunchKernelGGL(router_norm_mfma_kernel<32>, dim3((T + 31) / 32), dim3(512), shm, s, hp, norm_weight, eps, wp, bias, T,
                        H, E, k, norm_mode, xp, logits, idx, w, nullptr, chunk_hist);
   } else {
     const size_t shm = (size_t)16 * H * sizeof(bf16_t);
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&router_norm_mfma_kernel<16>),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm);
-    if (e != hipSuccess) return e;
+    if ((e = allow_dynamic_lds<16>()) != hipSuccess) return e;
     hipLaunchKernelGGL(router_norm_mfma_kernel<16>, dim3((T + 15) / 16), dim3(256), shm, s, hp, norm_weight, eps, wp, bias, T,
                        H, E, k, norm_mode, xp, logits, idx, w, nullptr, chunk_hist);
   }

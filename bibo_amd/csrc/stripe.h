@@ -9,10 +9,7 @@
 namespace bibo {
 namespace {
 
-#ifndef BIBO_LOADS_PER_PAIR
-#define BIBO_LOADS_PER_PAIR 1
-#endif
-constexpr int kLoadsPerPair = BIBO_LOADS_PER_PAIR;
+constexpr int kLoadsPerPair = 1;   // load instructions of the next stage issued per (sub-step, N tile) pair
 constexpr int kBK = 32;        // default K elements per LDS stage
 
 struct TileMap {

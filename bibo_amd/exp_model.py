@@ -254,7 +254,10 @@ class BiBoExpDecoderLayer(nn.Module):
             if collect_routing:
                 out = self._moe_with_routing(hs, prefix)
             else:
-                out = self.mlp.ffn_forward(hs, ln.weight, ln.variance_epsilon, residual=prefix)
+                # the reference's block returns its output in the stream's dtype (moe.py:101) before `prefix_sum +
+                # mlp_output` (exp/modeling_bibo.py:666): on a bf16 stream the block is rounded, then the sum
+                out = self.mlp.ffn_forward(hs, ln.weight, ln.variance_epsilon, residual=prefix,
+                                           bf16_moe_out=hs.dtype == torch.bfloat16)
         else:
             out = prefix + self.mlp(ln(hs))
         return out, blocks
@@ -271,7 +274,7 @@ class BiBoExpDecoderLayer(nn.Module):
                                          float(ln.variance_epsilon), m.gate._cache.get("w", m.gate.gate_proj.weight, cd),
                                          m.gate._cache.get("b", m.gate.bias, torch.float32), gu, dn, th,
                                          m.num_experts_per_tok, norm=m.gate.norm_topk_prob, algo=m.experts.algo,
-                                         want_routing=True, act=m.experts.act,
+                                         want_routing=True, act=m.experts.act, round_block_out=cd == torch.bfloat16,
                                          residual=prefix.reshape(-1, H).to(cd).contiguous())
         self.last_routing = (idx, w)
         return out.view(B, S, H).to(hs.dtype)

@@ -33,11 +33,19 @@ class _MoELayerFn(torch.autograd.Function):
     gets none (router.py:38).  The per-expert row counts come out as a second, non-differentiable result."""
 
     @staticmethod
-    def forward(ctx, x, w_router, w_gate_up, w_down, theta, bias, k, norm, act, algo, want_counts, n_pos=0, n_neg=0):
+    def forward(ctx, x, w_router, w_gate_up, w_down, theta, bias, k, norm, act, algo, want_counts, n_pos=0, n_neg=0,
+                casts=None):
         cd = torch.bfloat16
         cast = lambda t, d: (t if t.dtype == d else t.to(d)).contiguous()
-        xb, wr, gu, dn = cast(x.detach(), cd), cast(w_router.detach(), cd), cast(w_gate_up.detach(), cd), cast(w_down.detach(), cd)
-        th, b = cast(theta.detach(), torch.float32), cast(bias.detach(), torch.float32)
+        xb = cast(x.detach(), cd)
+        # `casts`: kernel-dtype copies of the three weight tensors the caller already holds (the layer's cast cache), so
+        # fp32 master weights are rounded once per optimiser step, not once per forward
+        wr, gu, dn = casts if casts is not None else (cast(w_router.detach(), cd), cast(w_gate_up.detach(), cd),
+                                                      cast(w_down.detach(), cd))
+        th = cast(theta.detach(), torch.float32)
+        # A private copy of the E selection biases: the layer's balancing step writes gate.bias in place later in the
+        # same forward (update_bias), and the backward pass has to route with the values the forward saw.
+        b = bias.detach().to(torch.float32).clone()
         out, _, _, counts, _ = ops.moe_forward(xb, wr, b, gu, dn, th, k, norm=norm, algo=algo, want_counts=want_counts, act=act,
                                                n_pos=n_pos, n_neg=n_neg)
         ctx.save_for_backward(xb, wr, gu, dn, th, b)
@@ -54,7 +62,7 @@ class _MoELayerFn(torch.autograd.Function):
         k, norm, act, n_pos, n_neg = ctx.conf
         d = d_out.to(torch.bfloat16).contiguous()
         grads = ops.moe_backward(xb, d, wr, b, gu, dn, th, k, norm=norm, act=act, n_pos=n_pos, n_neg=n_neg)[:5]
-        return tuple(g.to(dt) for g, dt in zip(grads, ctx.in_dtypes)) + (None,) * 8
+        return tuple(g.to(dt) for g, dt in zip(grads, ctx.in_dtypes)) + (None,) * 9
 
 
 class _ExpertsFn(torch.autograd.Function):
@@ -62,10 +70,11 @@ class _ExpertsFn(torch.autograd.Function):
     = bibo_moe_experts_backward.  The gradient of the combine weights (moe.py:93) flows back to whoever made them."""
 
     @staticmethod
-    def forward(ctx, x, top_w, w_gate_up, w_down, theta, idx, act, algo, want_counts, n_pos=0, n_neg=0):
+    def forward(ctx, x, top_w, w_gate_up, w_down, theta, idx, act, algo, want_counts, n_pos=0, n_neg=0, casts=None):
         cd = torch.bfloat16
         cast = lambda t, d: (t if t.dtype == d else t.to(d)).contiguous()
-        xb, gu, dn = cast(x.detach(), cd), cast(w_gate_up.detach(), cd), cast(w_down.detach(), cd)
+        xb = cast(x.detach(), cd)
+        gu, dn = casts if casts is not None else (cast(w_gate_up.detach(), cd), cast(w_down.detach(), cd))
         th, w = cast(theta.detach(), torch.float32), cast(top_w.detach(), torch.float32)
         out, counts = ops.experts_fwd(xb, idx, w, gu, dn, th, algo=algo, want_counts=want_counts, act=act, n_pos=n_pos,
                                       n_neg=n_neg)
@@ -82,7 +91,7 @@ class _ExpertsFn(torch.autograd.Function):
         xb, w, gu, dn, th, idx = ctx.saved_tensors
         grads = ops.experts_backward(xb, d_out.to(torch.bfloat16).contiguous(), idx, w, gu, dn, th, act=ctx.act,
                                      n_pos=ctx.specials[0], n_neg=ctx.specials[1])
-        return tuple(g.to(dt) for g, dt in zip(grads, ctx.in_dtypes)) + (None,) * 6
+        return tuple(g.to(dt) for g, dt in zip(grads, ctx.in_dtypes)) + (None,) * 7
 
 
 def _backward_covers(experts) -> bool:
@@ -258,7 +267,7 @@ class BiBoFusedExperts(nn.Module):
                                           "expert size <= 512")
             out, counts = _ExpertsFn.apply(hidden_states, top_k_weights, self.gate_up_proj, self.down_proj, self.radial_theta,
                                            top_k_indices.detach().to(torch.int32).contiguous(), self.act, self.algo,
-                                           _want_counts, self.num_pos, self.num_neg)
+                                           _want_counts, self.num_pos, self.num_neg, self._weights(torch.bfloat16)[:2])
             out = out if out.dtype == hidden_states.dtype else out.to(hidden_states.dtype)
             return (out, counts) if _want_counts else out
         cd = _compute_dtype(hidden_states)
@@ -429,9 +438,12 @@ class BiBoMoELayer(nn.Module):
         if not _backward_covers(e):
             raise NotImplementedError("the backward pass covers hidden and expert sizes that are multiples of 128 and "
                                       "expert size <= 512")
+        cd = torch.bfloat16
+        gu, dn, _ = e._weights(cd)
+        casts = (self.gate._cache.get("w", self.gate.gate_proj.weight, cd), gu, dn)
         out, counts = _MoELayerFn.apply(x, self.gate.gate_proj.weight, e.gate_up_proj, e.down_proj, e.radial_theta,
                                         self.gate.bias, self.num_experts_per_tok, self.gate.norm_topk_prob, e.act, e.algo,
-                                        want_counts, e.num_pos, e.num_neg)
+                                        want_counts, e.num_pos, e.num_neg, casts)
         return out, (counts if want_counts else None)
 
     @_no_compile

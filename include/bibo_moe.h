@@ -11,8 +11,10 @@
  *
  * Conventions
  *   - Every pointer is a DEVICE pointer on the current HIP device unless stated otherwise.  The caller
- *     allocates inputs, outputs and the workspace; the library allocates nothing, keeps no pointer
- *     after a call returns and has no mutable global state.
+ *     allocates inputs, outputs and the workspace; the library allocates nothing and keeps no pointer
+ *     to a caller's buffer after a call returns.  Its only state across calls is set-up it remembers per
+ *     device behind a mutex: the address of its static scratch array (bibo_moe_forward_static) and
+ *     whether a kernel's dynamic LDS limit has been raised; neither depends on a call's arguments.
  *   - All tensors are dense row-major ("contiguous"); weights are consumed as the reference stores
  *     them: w_router [E,H], w_gate_up [E,2I,H] (rows 0..I-1 gate, I..2I-1 up), w_down [E,H,I].
  *   - `dtype` selects the element type of hidden states and the three weight tensors

@@ -264,3 +264,50 @@ def test_hip_depth_mix_and_row_norm_match_the_stock_operations():
     with torch.enable_grad():
         ref = norm(x.clone().requires_grad_(True)).detach()
     assert got.shape == x.shape and float((got.float() - ref.float()).abs().max()) <= 1e-2 * float(ref.float().abs().max())
+
+
+# ------------------------------------------------------------------ GPU: config 5 at its real dimensions
+def _full_size_case(dtype, seed):
+    """The probe's model as the reference configures it (ablate/tools/tps_probe.sh:30-41, ablate/common/configs.py:63-73):
+    H = 768, 4 query / 2 KV heads of 192, window 128, dense layers 0 and 9 at 2304, E = 64, top-6, I = 384, vocabulary
+    32000, tied head, N(0, 0.02) initialisation.  The parameters that start at a neutral value (norm weights, XSA alpha,
+    carry theta, radial theta, balancing bias) are moved off it so that their paths are live."""
+    cfg = X.BiBoExpConfig(bf16_residual_stream=dtype == torch.bfloat16)
+    assert (cfg.hidden_size, cfg.head_dim, cfg.sliding_window, cfg.moe_intermediate_size, cfg.vocab_size) == (768, 192, 128, 384, 32000)
+    torch.manual_seed(seed)
+    model = X.BiBoExpForCausalLM(cfg)
+    g = torch.Generator().manual_seed(seed)
+    with torch.no_grad():
+        for name, p in model.named_parameters():
+            if name.endswith("norm.weight") or name.endswith("layernorm.weight"):
+                p.copy_(torch.rand(p.shape, generator=g) + 0.5)
+            elif name.endswith("xsa_alpha"):
+                p.copy_(torch.randn(p.shape, generator=g))
+            elif name.endswith("attn_res_carry_theta"):
+                p.copy_(torch.rand(p.shape, generator=g) * 1.5 + 0.25)
+            elif name.endswith("radial_theta"):
+                p.copy_(torch.randn(p.shape, generator=g) * 0.5)
+            elif name.endswith("gate.bias"):
+                p.copy_(torch.rand(p.shape, generator=g) * 0.02 - 0.01)
+    model = model.to("cuda:0").to(dtype).eval()
+    ids = torch.randint(0, cfg.vocab_size, (1, 330), generator=torch.Generator().manual_seed(seed))   # 2.6 windows
+    return cfg, model, ids
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-4), (torch.bfloat16, 5e-2)])
+def test_full_size_model_matches_the_oracle(dtype, tol):
+    """Config 5 at its real dimensions, one sequence of 330 tokens (more than two windows, no multiple of the window):
+    logits of the whole model against the fp32 oracle evaluated with the kernels' routing decisions."""
+    cfg, model, ids = _full_size_case(dtype, 21)
+    logits = model(ids.to("cuda:0"), collect_routing=True)
+    fast = model(ids.to("cuda:0"))
+    torch.cuda.synchronize()
+    assert torch.equal(logits, fast)
+    routing = {l: (i.cpu().numpy(), w.cpu().numpy()) for l, (i, w) in model.routing().items()}
+    assert sorted(routing) == list(range(1, 9))
+    sd = {k: v.detach().cpu() for k, v in model.state_dict().items()}
+    ref = XO.forward(ids, sd, cfg, dtype=torch.float32, routing=routing)
+    err = rel_err(logits.cpu(), ref)
+    print(f"full-size config 5, {dtype}: rel err {err:.3e} (bar {tol:g})")
+    assert logits.shape == (1, 330, 32000) and torch.isfinite(logits).all() and err <= tol

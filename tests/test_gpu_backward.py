@@ -34,7 +34,8 @@ def _run(T, H, E, k, I, norm="sum", act="radial", seed=0, theta="normal", scale=
     return dict(zip(("x", "w_router", "w_gate_up", "w_down", "theta", "w"), got)), ref, idx.cpu().numpy()
 
 
-@pytest.mark.parametrize("T,H,E,k,I", [(300, 256, 16, 4, 128), (512, 512, 64, 6, 256), (64, 384, 8, 2, 384), (1000, 768, 64, 6, 384)])
+@pytest.mark.parametrize("T,H,E,k,I", [(300, 256, 16, 4, 128), (512, 512, 64, 6, 256), (64, 384, 8, 2, 384), (1000, 768, 64, 6, 384),
+                                       (200, 1024, 16, 4, 512)])     # the widest rows the backward pass takes
 def test_backward_matches_oracle(T, H, E, k, I):
     got, ref, _ = _run(T, H, E, k, I, seed=T)
     for name in ("w", "x", "w_down", "w_gate_up", "w_router", "theta"):
@@ -276,3 +277,121 @@ def test_hooks_path_trains_module_by_module():
     for n, p in layer.named_parameters():
         if n in ref:
             assert _rel(p.grad, ref[n].cpu()) <= 3e-2, n
+
+
+def test_experts_backward_with_padded_slots():
+    """Routing indices outside [0, E) (padding in a caller's indices): the forward pass skips those slots, and the
+    backward pass gives them a zero combine-weight gradient and leaves them out of d_x.  The workspace is poisoned
+    first, so a slot row nobody wrote cannot pass by luck."""
+    T, H, E, k, I = 150, 256, 8, 3, 128
+    p = O.make_inputs(T=T, H=H, E=E, k=k, I=I, theta="normal", seed=12)
+    g = torch.Generator().manual_seed(5)
+    idx = torch.randint(0, E, (T, k), generator=g, dtype=torch.int32)
+    idx[:, 1] = E                                                  # one padded slot per token
+    idx[::7, 2] = -1
+    w = torch.rand(T, k, generator=g) + 0.1
+    d_out = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    dev = lambda t: t.to(DEV)
+    ops.workspace(DEV, 256 << 20).fill_(0x7f)                      # bf16 0x7f7f = 3.4e38, fp32 0x7f7f7f7f = 3.4e38
+    got = ops.experts_backward(dev(p["x"]), dev(d_out), dev(idx), dev(w), dev(p["w_gate_up"]), dev(p["w_down"]), dev(p["theta"]))
+    torch.cuda.synchronize()
+    pad = (idx < 0) | (idx >= E)
+    w0, idx0 = w.clone(), idx.clone()
+    w0[pad] = 0.0                                                  # the same slots with weight zero on a real expert
+    idx0[pad] = 0
+    leaf = lambda t: t.double().clone().requires_grad_(True)
+    x, wl, gu, dn, th = leaf(p["x"]), leaf(w0), leaf(p["w_gate_up"]), leaf(p["w_down"]), leaf(p["theta"])
+    (O.experts_forward(x, idx0, wl, gu, dn, th, dtype=torch.float64) * d_out.double()).sum().backward()
+    ref_w = wl.grad.clone()
+    ref_w[pad] = 0.0
+    assert float(got[1].cpu()[pad].abs().max()) == 0.0
+    for a, r, name in zip(got, (x.grad, ref_w, gu.grad, dn.grad, th.grad), ("x", "w", "w_gate_up", "w_down", "theta")):
+        assert bool(torch.isfinite(a.float()).all()), name
+        assert _rel(a, r) <= TOL, (name, _rel(a, r))
+    # the module under autograd takes the same indices
+    from bibo_amd.config import BiBoMoEConfig
+    from bibo_amd.moe import BiBoFusedExperts
+    ex = BiBoFusedExperts(BiBoMoEConfig(hidden_size=H, moe_intermediate_size=I, num_routed_experts=E, num_experts_per_tok=k,
+                                        special_expert_pairs=0)).to(DEV).bfloat16()
+    with torch.no_grad():
+        ex.gate_up_proj.copy_(p["w_gate_up"]); ex.down_proj.copy_(p["w_down"]); ex.radial_theta.copy_(p["theta"])
+    xg, wg = dev(p["x"]).requires_grad_(True), dev(w).requires_grad_(True)
+    ex(xg, dev(idx).long(), wg).backward(dev(d_out))
+    assert torch.equal(xg.grad, got[0]) and torch.equal(wg.grad, got[1])
+
+
+def test_fp32_master_weights_train_while_the_balancing_bias_moves():
+    """fp32 master weights under bf16 autocast with a balancing step that fires in the same forward (token count at the
+    threshold, moe.py:139-155): update_bias writes gate.bias in place after the block ran, the backward pass still
+    routes with the bias the forward saw, and the gradients are those of that selection."""
+    T, H, E, k, I = 256, 256, 16, 4, 128
+    layer = _layer(H=H, I=I, E=E, k=k, bias_update_threshold=T).float().train()
+    with torch.no_grad():
+        layer.gate.bias.copy_(torch.linspace(-0.2, 0.2, E))        # far from balance: the update moves every entry
+        layer.experts.radial_theta.copy_(torch.linspace(-1, 2, E))
+    bias0 = layer.gate.bias.detach().clone()
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(2, T // 2, H, generator=g).to(DEV).requires_grad_(True)
+    d = torch.randn(2, T // 2, H, generator=g).to(DEV)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        out = layer(x)
+    assert not torch.equal(layer.gate.bias.detach(), bias0)         # the balancing step fired inside the forward
+    out.backward(d.to(out.dtype))
+    torch.cuda.synchronize()
+    bf = lambda t: t.detach().to(torch.bfloat16)
+    xb = bf(x).reshape(T, H)
+    _, idx, _, _, _ = ops.moe_forward(xb, bf(layer.gate.gate_proj.weight), bias0.float(), bf(layer.experts.gate_up_proj),
+                                      bf(layer.experts.down_proj), layer.experts.radial_theta.detach().float(), k,
+                                      want_routing=True)
+    _, idx_new, _, _, _ = ops.moe_forward(xb, bf(layer.gate.gate_proj.weight), layer.gate.bias.detach().float(),
+                                          bf(layer.experts.gate_up_proj), bf(layer.experts.down_proj),
+                                          layer.experts.radial_theta.detach().float(), k, want_routing=True)
+    assert not torch.equal(idx, idx_new)                            # the moved bias would select differently
+    ref = O.moe_backward(xb.cpu(), bf(layer.gate.gate_proj.weight).cpu(), bf(layer.experts.gate_up_proj).cpu(),
+                         bf(layer.experts.down_proj).cpu(), layer.experts.radial_theta.detach().float().cpu(),
+                         idx.cpu().numpy(), bf(d).cpu().reshape(T, H))
+    assert x.grad.dtype == torch.float32 and layer.experts.gate_up_proj.grad.dtype == torch.float32
+    assert _rel(x.grad.reshape(T, H), ref["x"]) <= TOL
+    assert _rel(layer.gate.gate_proj.weight.grad, ref["w_router"]) <= TOL
+    assert _rel(layer.experts.gate_up_proj.grad, ref["w_gate_up"]) <= TOL
+    assert _rel(layer.experts.down_proj.grad, ref["w_down"]) <= TOL
+    assert _rel(layer.experts.radial_theta.grad, ref["theta"]) <= TOL
+
+
+@pytest.mark.parametrize("seam", ["layer", "ffn"])
+def test_layer_under_activation_checkpointing(seam):
+    """The reference wraps its decoder layers in torch.utils.checkpoint (src/modeling/layers.py:97-98): the block runs
+    once in the forward pass and once more when the backward pass recomputes it.  Gradients equal those of the plain
+    run bit for bit (the kernels are deterministic), and the balancing state stays consistent."""
+    from torch.utils.checkpoint import checkpoint
+    H = 256
+    layer = _layer(H=H, I=128, E=16, k=4, bias_update_threshold=10 ** 9).train()   # no bias step inside this test
+    nw = (1 + 0.1 * torch.randn(H, device=DEV)).requires_grad_(True)
+    g = torch.Generator().manual_seed(9)
+    x0 = torch.randn(2, 60, H, generator=g).to(torch.bfloat16).to(DEV)
+    d = torch.randn(2, 60, H, generator=g).to(torch.bfloat16).to(DEV)
+    fn = (lambda t: layer(t)) if seam == "layer" else (lambda t: layer.ffn_forward(t, nw, 1e-6))
+
+    def run(wrapped):
+        layer.zero_grad()
+        nw.grad = None
+        layer.accumulated_tpe.zero_()
+        layer._fwd_step = 0
+        x = x0.clone().requires_grad_(True)
+        out = checkpoint(fn, x, use_reentrant=False) if wrapped else fn(x)
+        out.backward(d)
+        torch.cuda.synchronize()
+        grads = {n: p.grad.clone() for n, p in layer.named_parameters() if p.grad is not None}
+        return (out.detach(), x.grad.clone(), grads, (None if nw.grad is None else nw.grad.clone()),
+                (layer._fwd_step, float(layer.accumulated_tpe.sum())))
+
+    out_a, gx_a, gp_a, gn_a, steps_a = run(False)
+    out_b, gx_b, gp_b, gn_b, steps_b = run(True)
+    assert torch.equal(out_a, out_b) and torch.equal(gx_a, gx_b)
+    assert sorted(gp_a) == sorted(gp_b) and all(torch.equal(gp_a[n], gp_b[n]) for n in gp_a)
+    if seam == "ffn":
+        assert gn_a is not None and torch.equal(gn_a, gn_b)
+    # The balancing state counts calls of the layer.  The recomputation calls it again, but torch stops it as soon as
+    # the last tensor the backward pass needs exists again, which may be before the balancing step: one or two steps,
+    # each with all of the forward's 120 * 4 selections.
+    assert steps_a == (1, 120.0 * 4) and steps_b in ((1, 120.0 * 4), (2, 2 * 120.0 * 4))
