@@ -314,7 +314,8 @@ def test_experts_backward_with_padded_slots():
     ex = BiBoFusedExperts(BiBoMoEConfig(hidden_size=H, moe_intermediate_size=I, num_routed_experts=E, num_experts_per_tok=k,
                                         special_expert_pairs=0)).to(DEV).bfloat16()
     with torch.no_grad():
-        ex.gate_up_proj.copy_(p["w_gate_up"]); ex.down_proj.copy_(p["w_down"]); ex.radial_theta.copy_(p["theta"])
+        ex.gate_up_proj.copy_(p["w_gate_up"]); ex.down_proj.copy_(p["w_down"])
+    ex.radial_theta.data = dev(p["theta"])                         # fp32, so both calls see the same exponents
     xg, wg = dev(p["x"]).requires_grad_(True), dev(w).requires_grad_(True)
     ex(xg, dev(idx).long(), wg).backward(dev(d_out))
     assert torch.equal(xg.grad, got[0]) and torch.equal(wg.grad, got[1])
