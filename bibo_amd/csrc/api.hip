@@ -50,13 +50,15 @@ int check_dims(int T, int H, int E, int k, int I, int dtype, int n_pos = 0, int 
   return BIBO_OK;
 }
 
-// Rows per expert at or below which the weight-streaming kernels are preferred (measured against the MFMA tile
-// kernels at E = 64, k = 6).  With H and I up to 512 a wave's 16 weight rows stay in registers for all of the
-// expert's rows and a further 16-row pass only costs its staging (crossover near 40 rows); wider rows are
-// streamed again, from L2, for every pass (crossover near 32 rows at H = 768, near 24 at H = 1024).
-inline long long stream_rows_per_expert(int H, int I) {
-  if (H <= 512 && I <= 512) return 40;
-  return H <= 768 ? 32 : 24;
+// Rows per expert at or below which the weight-streaming kernels are preferred (measured against the tile kernels
+// at E = 64, k = 6, whole layer).  With H and I up to 512 a wave's 16 weight rows stay in registers for all of the
+// expert's rows and a further 16-row pass only costs its staging: the crossover against the fused kernel is near 24
+// rows.  Wider rows are streamed again, from L2, for every pass: against the fused kernel they win up to about 10
+// rows (H = 768, I = 384), against the two-kernel MFMA path (shapes the fused kernel does not take) up to about 17
+// (H = 1024, I = 512).
+inline long long stream_rows_per_expert(int H, int I, int dtype) {
+  if (H <= 512 && I <= 512) return 24;
+  return fused_supported(H, I, dtype) ? 10 : 17;
 }
 
 // `distinct`: the k experts of a token are known to differ (indices that come straight from the router kernel), so
@@ -65,9 +67,15 @@ inline long long stream_rows_per_expert(int H, int I) {
 // the fused kernel addresses hidden-state rows with 32-bit byte offsets
 inline bool fused_fits(int T, int H) { return (long long)T * H < (1LL << 31); }
 
+// what the streaming kernels can run: the slots fit a workgroup's scan and an expert's rows its row list
+inline bool stream_possible(int T, int H, int E, int k, int I, int dtype, bool distinct) {
+  return stream_supported(H, I, dtype) && (long long)T * k <= kStreamMaxSlots &&
+         (distinct ? T : (long long)T * k) <= kStreamMaxRows;
+}
+
+// what `auto` gives them: few enough rows per expert that streaming beats the tile kernels
 inline bool stream_eligible(int T, int H, int E, int k, int I, int dtype, bool distinct) {
-  return stream_supported(H, I, dtype) && (long long)T * k <= stream_rows_per_expert(H, I) * E &&
-         (long long)T * k <= kStreamMaxSlots && (distinct ? T : (long long)T * k) <= kStreamMaxRows;
+  return stream_possible(T, H, E, k, I, dtype, distinct) && (long long)T * k <= stream_rows_per_expert(H, I, dtype) * E;
 }
 
 // `composite`: the caller is bibo_moe_experts_fwd / bibo_moe_forward, the only entry points that can run
@@ -87,7 +95,7 @@ int resolve_algo(int algo, int T, int H, int E, int k, int I, int dtype, bool co
       break;
     case BIBO_ALGO_STREAM:
       // more rows per expert than the limit: refused here, before anything is launched
-      if (!composite || !stream_eligible(T, H, E, k, I, dtype, distinct)) return BIBO_ERR_UNSUPPORTED;
+      if (!composite || !stream_possible(T, H, E, k, I, dtype, distinct)) return BIBO_ERR_UNSUPPORTED;
       *out = BIBO_ALGO_STREAM;
       break;
     case BIBO_ALGO_FUSED:
@@ -119,7 +127,7 @@ Workspace carve(int T, int H, int E, int k, int I, int dtype) {
   ws.perm_token = o; o += align_up(S * sizeof(int32_t));
   ws.hidden = o;     o += align_up(S * (size_t)I * elt_size(dtype));
   // bf16 gate/up pre-activations, only ever used when the streaming kernels are eligible
-  ws.gu = o;         o += align_up(stream_eligible(T, H, E, k, I, dtype, true) ? S * (size_t)2 * I * sizeof(bf16_t) : 0);
+  ws.gu = o;         o += align_up(stream_possible(T, H, E, k, I, dtype, true) ? S * (size_t)2 * I * sizeof(bf16_t) : 0);
   ws.yw = o;         o += align_up(S * (size_t)H * sizeof(float));
   ws.total = o;
   return ws;
@@ -170,7 +178,7 @@ int experts_dispatch(const void* x, const void* wgu, const void* wd, const float
   if (!idx_trusted || np + nn > 0) { ca.idx = idx; ca.w = w; ca.x = x; ca.E_glu = Eg; ca.n_pos = np; ca.n_neg = nn; }
   if (algo == BIBO_ALGO_STREAM) {
     if (!aligned16(x) || !aligned16(wgu) || !aligned16(wd)) return BIBO_ERR_MISALIGNED;
-    if (!stream_eligible(T, H, Eg + np + nn, k, I, dtype, idx_trusted)) return BIBO_ERR_UNSUPPORTED;   // no pre-activation segment carved, or more rows than a row list holds
+    if (!stream_possible(T, H, Eg + np + nn, k, I, dtype, idx_trusted)) return BIBO_ERR_UNSUPPORTED;   // no pre-activation segment carved, or more rows than a row list holds
     void* gu = base + ws.gu;
     hipError_t e = launch_gateup_stream(x, wgu, idx, T, H, Eg, k, I, gu, s);
     if (e != hipSuccess) return (int)e;

@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <mutex>
+
 #include "../../include/bibo_moe.h"
 
 namespace bibo {
@@ -135,6 +137,25 @@ __device__ __forceinline__ int xcd_tile(int bid, int total) {
   if (slot >= per) return total;   // no tile
   return (bid & 7) * per + slot;
 }
+
+// A kernel that wants more dynamic LDS than the default limit has to be allowed to, once per device, by a host-side
+// driver call (hipFuncSetAttribute).  One of these per kernel instantiation remembers the devices on which that has
+// been done, so that later launches, possibly under graph capture, go straight to the launch.
+struct LdsLimitOnce {
+  std::mutex m;
+  bool done[64] = {};
+  hipError_t raise(const void* kernel, int bytes) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    const bool tracked = dev >= 0 && dev < 64;
+    std::lock_guard<std::mutex> lock(m);
+    if (tracked && done[dev]) return hipSuccess;
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipSuccess && tracked) done[dev] = true;
+    return e;
+  }
+};
 
 // ---- host-side launchers (one per translation unit) -------------------------------------------
 // `chunk_hist` (or NULL): per-workgroup histograms of the selected experts, [ceil(T / *hist_tokens)][64]; *hist_tokens

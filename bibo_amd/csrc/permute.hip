@@ -121,9 +121,9 @@ __global__ __launch_bounds__(256) void scatter_kernel(const int32_t* __restrict_
   }
 }
 
-// Small inputs (T*k <= kSmallSlots): histogram, scan and scatter by ONE wave in one launch; the two
-// passes over the slots cost less than a second kernel launch.
-constexpr int kSmallSlots = 2048;
+// Small inputs (T*k <= kSmallSlots): histogram, scan and scatter by ONE wave in one launch.  The wave spends about
+// 0.7 us per 64 slots; from about 600 slots on the multi-workgroup kernels (6 us whatever the size) are faster.
+constexpr int kSmallSlots = 512;
 
 __global__ __launch_bounds__(64) void permute_small_kernel(const int32_t* __restrict__ idx, int S, int E, int k,
                                                            int32_t* __restrict__ counts, int32_t* __restrict__ offsets,

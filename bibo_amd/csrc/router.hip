@@ -1,8 +1,6 @@
 // Kernel 1: fused router.  fp32 logits x @ w_router^T, canonical sigmoid, selection on score + bias
 // (ties to the lowest expert index), gather of the unbiased scores, normalisation.
 // Follows BiBoMoERouter.forward, src/modeling/ffn/router.py:25-51 of the reference.
-#include <mutex>
-
 #include "common.h"
 
 namespace bibo {
@@ -564,25 +562,11 @@ bool router_norm_supported(int H, int dtype, const void* h, const void* w_router
   return dtype == BIBO_DTYPE_BF16 && (H % kRouterKC) == 0 && H <= kNormRouterMaxH && aligned;
 }
 
-// Dynamic LDS beyond the default limit has to be allowed once per kernel and device (a host-side driver call without
-// a launch): done on the first call on a device, for the widest rows the kernel takes, and remembered, so that later
-// calls (one per layer and step, possibly under graph capture) go straight to the launch.
-constexpr int kMaxDevicesSeen = 64;
-std::mutex g_lds_mutex;
-bool g_lds_allowed[2][kMaxDevicesSeen] = {};
-
+// the kernel's TOK whole rows sit in dynamic LDS: allowed once per device, for the widest rows it takes
 template <int TOK>
 hipError_t allow_dynamic_lds() {
-  int dev = -1;
-  hipError_t e = hipGetDevice(&dev);
-  if (e != hipSuccess) return e;
-  const bool tracked = dev >= 0 && dev < kMaxDevicesSeen;
-  std::lock_guard<std::mutex> lock(g_lds_mutex);
-  if (tracked && g_lds_allowed[TOK == 32][dev]) return hipSuccess;
-  e = hipFuncSetAttribute(reinterpret_cast<const void*>(&router_norm_mfma_kernel<TOK>),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)(TOK * kNormRouterMaxH * sizeof(bf16_t)));
-  if (e == hipSuccess && tracked) g_lds_allowed[TOK == 32][dev] = true;
-  return e;
+  static LdsLimitOnce once;
+  return once.raise(reinterpret_cast<const void*>(&router_norm_mfma_kernel<TOK>), (int)(TOK * kNormRouterMaxH * sizeof(bf16_t)));
 }
 
 // RMSNorm + router in one launch (see router_norm_mfma_kernel); `xn` receives the normalised rows.

@@ -108,13 +108,13 @@ def test_ffn_forward_at_full_prefill_size(name):
 @pytest.mark.parametrize("algo", ["auto", "stream"])
 def test_every_slot_on_one_expert_with_repeats(algo):
     """A caller's indices may name one expert in every slot of every token (the reference's loop accepts that,
-    moe.py:46-71): 2560 rows on expert 9, more than the row list of a streaming workgroup holds.  `auto` must not
+    moe.py:46-71): 2560 rows on expert 9, more than the row list of a streaming workgroup holds.  `auto` does not
     pick the streaming kernels for such a call and `stream` is refused before anything is launched."""
     T, k, H, I, E = 320, 8, 256, 256, 64
     p = O.make_inputs(T=T, H=H, E=E, k=k, I=I, theta="normal", seed=320)
     idx = np.full((T, k), 9, np.int32)
     w = np.random.default_rng(4).random((T, k)).astype(np.float32)
-    assert ops.select_algo(T, H, E, k, I) == "stream"          # what the layer call (distinct experts) would run
+    assert ops.select_algo(T, H, E, k, I) == "fused"           # 40 slots per expert on average: past the streaming range
     args = (p["x"].to(DEV), torch.from_numpy(idx).to(DEV), torch.from_numpy(w).to(DEV), p["w_gate_up"].to(DEV),
             p["w_down"].to(DEV), p["theta"].to(DEV))
     if algo == "stream":

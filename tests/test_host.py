@@ -89,8 +89,12 @@ def test_kernel_family_selection_is_exported():
     assert ops.select_algo(16384, 768, 64, 6, 384) == "fused"
     assert ops.select_algo(64, 1024, 64, 6, 512) == "stream"            # decode workload: 6 rows per expert
     assert ops.select_algo(512, 512, 64, 6, 256) == "fused"             # 48 rows per expert: past the streaming limit
-    assert ops.select_algo(400, 512, 64, 6, 256) == "stream"            # 37.5 rows, register-resident weight rows
-    assert ops.select_algo(341, 1024, 64, 6, 512) == "mfma"             # 32 rows of 2 KB: tiles win, I = 512 is not fused
+    assert ops.select_algo(250, 512, 64, 6, 256) == "stream"            # 23.4 rows, register-resident weight rows
+    assert ops.select_algo(300, 512, 64, 6, 256) == "fused"             # 28 rows: the fused kernel wins from about 24
+    assert ops.select_algo(100, 768, 64, 6, 384) == "stream"            # 9.4 rows of 1.5 KB
+    assert ops.select_algo(128, 768, 64, 6, 384) == "fused"             # 12 rows: wider rows are re-streamed per pass
+    assert ops.select_algo(170, 1024, 64, 6, 512) == "stream"           # 16 rows; I = 512 is not fused, the tile path is slow
+    assert ops.select_algo(341, 1024, 64, 6, 512) == "mfma"             # 32 rows of 2 KB: tiles win
     assert ops.select_algo(8192, 768, 64, 6, 384, L.DTYPE_F32) == "generic"
     assert ops.select_algo(8192, 768, 64, 6, 384, algo="mfma") == "mfma"
     with pytest.raises(RuntimeError, match="does not support"):
