@@ -255,12 +255,12 @@ int forward_impl(const void* x, const void* w_router, const float* bias, const v
 
 
 struct BackwardWorkspace {
-  size_t hist, idx, w, logits, counts, offsets, perm_slot, perm_token, pad_off, dw_slot, dl, dtheta_row, dwr_part, wd_t, wgu_t, gu, dhp, dgu,
-      hidden, dxs, p_t, q_t, total;
+  size_t hist, idx, w, logits, counts, offsets, perm_slot, perm_token, dw_slot, dl, dtheta_row, dwr_part, zrow, gu, dhp, dgu,
+      hidden, dxs, total;
 };
 
 BackwardWorkspace carve_backward(int T, int H, int E, int k, int I) {
-  const size_t S = (size_t)T * k, ld = backward_padded_rows(T, E, k), b = sizeof(bf16_t);
+  const size_t S = (size_t)T * k, b = sizeof(bf16_t);
   BackwardWorkspace ws;
   size_t o = 0;
   ws.hist = o;       o += align_up(permute_workspace_bytes(T) > router_hist_bytes(T) ? permute_workspace_bytes(T)
@@ -272,20 +272,16 @@ BackwardWorkspace carve_backward(int T, int H, int E, int k, int I) {
   ws.offsets = o;    o += align_up((kMaxE + 1) * sizeof(int32_t));
   ws.perm_slot = o;  o += align_up(S * sizeof(int32_t));
   ws.perm_token = o; o += align_up(S * sizeof(int32_t));
-  ws.pad_off = o;    o += align_up((kMaxE + 1) * sizeof(int32_t));
   ws.dw_slot = o;    o += align_up(S * sizeof(float));
   ws.dl = o;         o += align_up(S * sizeof(float));
   ws.dtheta_row = o; o += align_up(S * sizeof(float));
   ws.dwr_part = o;   o += align_up((size_t)E * backward_dwr_split() * H * sizeof(float));
-  ws.wd_t = o;       o += align_up((size_t)E * I * H * b);
-  ws.wgu_t = o;      o += align_up((size_t)E * H * 2 * I * b);
+  ws.zrow = o;       o += align_up(backward_zero_row_bytes(H, I));
   ws.gu = o;         o += align_up(S * 2 * I * b);
   ws.dhp = o;        o += align_up(S * I * b);
   ws.dgu = o;        o += align_up(S * 2 * I * b);
   ws.hidden = o;     o += align_up(S * I * b);
   ws.dxs = o;        o += align_up(S * H * b);
-  ws.p_t = o;        o += align_up((size_t)(H > 2 * I ? H : 2 * I) * ld * b);
-  ws.q_t = o;        o += align_up((size_t)(H > I ? H : I) * ld * b);
   ws.total = o;
   return ws;
 }
@@ -572,13 +568,12 @@ int bibo_moe_backward(const void* x, const void* d_out, const void* w_router, co
   if ((rc = hip_rc(launch_permute(idx, T, E, k, counts, offsets, perm_slot, perm_token, base + ws.hist, s))) != BIBO_OK)
     return rc;
   BackwardBuffers b;
-  b.wd_t = base + ws.wd_t; b.wgu_t = base + ws.wgu_t; b.gu = base + ws.gu; b.dhp = base + ws.dhp; b.dgu = base + ws.dgu;
-  b.hidden = base + ws.hidden; b.dxs = base + ws.dxs; b.p_t = base + ws.p_t; b.q_t = base + ws.q_t;
+  b.gu = base + ws.gu; b.dhp = base + ws.dhp; b.dgu = base + ws.dgu;
+  b.hidden = base + ws.hidden; b.dxs = base + ws.dxs; b.zrow = base + ws.zrow;
   b.dw_slot = d_w_out ? d_w_out : reinterpret_cast<float*>(base + ws.dw_slot);
   b.dl = reinterpret_cast<float*>(base + ws.dl);
   b.dtheta_row = reinterpret_cast<float*>(base + ws.dtheta_row);
   b.dwr_part = reinterpret_cast<float*>(base + ws.dwr_part);
-  b.pad_off = reinterpret_cast<int32_t*>(base + ws.pad_off);
   return hip_rc(launch_backward(x, d_out, w_router, w_gate_up, w_down, theta, logits, idx, w, offsets, perm_slot, perm_token,
                                 T, H, E - sh->n_pos - sh->n_neg, sh->n_pos, sh->n_neg, k, I, norm_mode, sh->act, b, d_x,
                                 d_w_router, d_w_gate_up, d_w_down, d_theta, s));
@@ -610,13 +605,12 @@ int bibo_moe_experts_backward(const void* x, const void* d_out, const int32_t* i
   if ((rc = hip_rc(launch_permute(idx, T, E, k, counts, offsets, perm_slot, perm_token, base + ws.hist, s))) != BIBO_OK)
     return rc;
   BackwardBuffers b;
-  b.wd_t = base + ws.wd_t; b.wgu_t = base + ws.wgu_t; b.gu = base + ws.gu; b.dhp = base + ws.dhp; b.dgu = base + ws.dgu;
-  b.hidden = base + ws.hidden; b.dxs = base + ws.dxs; b.p_t = base + ws.p_t; b.q_t = base + ws.q_t;
+  b.gu = base + ws.gu; b.dhp = base + ws.dhp; b.dgu = base + ws.dgu;
+  b.hidden = base + ws.hidden; b.dxs = base + ws.dxs; b.zrow = base + ws.zrow;
   b.dw_slot = d_w;
   b.dl = reinterpret_cast<float*>(base + ws.dl);
   b.dtheta_row = reinterpret_cast<float*>(base + ws.dtheta_row);
   b.dwr_part = reinterpret_cast<float*>(base + ws.dwr_part);
-  b.pad_off = reinterpret_cast<int32_t*>(base + ws.pad_off);
   return hip_rc(launch_backward(x, d_out, nullptr, w_gate_up, w_down, theta, nullptr, idx, w, offsets, perm_slot, perm_token,
                                 T, H, E - sh->n_pos - sh->n_neg, sh->n_pos, sh->n_neg, k, I, BIBO_NORM_SUM, sh->act, b, d_x,
                                 nullptr, d_w_gate_up, d_w_down, d_theta, s));

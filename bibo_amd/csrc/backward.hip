@@ -9,17 +9,16 @@
 //     dx_t += W_gate_up[e]^T [dg, du]  (grouped GEMM over the TRANSPOSED gate/up weights)
 //     dW_down[e] += (w d_t) h^T,  dW_gate_up[e] += [dg, du] x_t^T   (grouped GEMMs that contract over an expert's rows)
 //     dlogit from dw (router.py:41-47), dW_router += dlogit^T x, dx += dlogit W_router.
-// Every GEMM here runs on the LDS-DMA / MFMA stripe machinery of the forward kernels, which wants both operands
-// contiguous along the contraction: the weights are transposed once per call, and the row-major activations that
-// are contracted over ROWS (the weight gradients) are transposed into [columns][rows] buffers in which each
-// expert's rows start at a multiple of 64 and are zero-padded to the next one, so that a K step never straddles
-// two experts.
-#include "stripe.h"
+// Every GEMM here runs on LDS-DMA stages and 32x32x16 MFMAs.  The pre-activations are recomputed with the forward's
+// operand layout (both operands contiguous along the contraction).  The input gradients contract over the middle
+// dimension of the weight tensors and the weight gradients over the ROWS of row-major activations: those operands go
+// to LDS as they lie in memory and are read through transposing LDS reads (kmajor.h), so nothing is transposed in
+// memory and an expert's rows need no padding: a K stage that runs past an expert's last row reads a row of zeros.
+#include "kmajor.h"
 
 namespace bibo {
 namespace {
 
-constexpr int kPad = 64;     // an expert's rows start at a multiple of this in the transposed buffers
 constexpr int kBwdBK = 64;   // K elements per LDS stage of the GEMMs here: whole 128-byte lines per row
 
 // ---- grouped GEMM: out[dst(r), n] = sum_k A[src(r), k] W[e][n, k] for the rows r of expert e ------------------
@@ -130,174 +129,50 @@ hipError_t launch_ggemm(const bf16_t* A, const int32_t* a_index, const bf16_t* W
   return launch_ggemm_t<1, GATHER, SCATTER>(A, a_index, W, offsets, out_index, S_rows, K, N, E, out, s);
 }
 
-// ---- transposes ---------------------------------------------------------------------------------------------
-// A 64 x 64 tile goes through LDS (row stride 66 elements: the eight column reads behind one 16-byte store touch
-// different banks); global memory is read and written 16 bytes per thread, 128 contiguous bytes per row.
-constexpr int kTS = 66;
-
-// rows j = t / 8 and j + 32 of the tile, columns 8 (t % 8) .. + 8: row j of the tile is in[src(j)], scaled; src < 0: zeros
-template <typename RowPtr, typename Scale>
-__device__ __forceinline__ void tile_load(bf16_t (&tile)[64][kTS], RowPtr row_ptr, Scale scale) {
-  const int t = threadIdx.x, cg = (t & 7) * 8;
-#pragma unroll
-  for (int h = 0; h < 2; ++h) {
-    const int j = (t >> 3) + 32 * h;
-    const bf16_t* src = row_ptr(j);
-    bf16x8 v;
-    if (src != nullptr) {
-      v = *reinterpret_cast<const bf16x8*>(src + cg);
-      const float sc = scale(j);
-      if (sc != 1.f) {
-#pragma unroll
-        for (int q = 0; q < 8; ++q) v[q] = (bf16_t)(sc * (float)v[q]);
-      }
-    } else {
-#pragma unroll
-      for (int q = 0; q < 8; ++q) v[q] = (bf16_t)0.f;
-    }
-#pragma unroll
-    for (int q = 0; q < 8; q += 2)          // 4-byte LDS writes (the row stride is not a multiple of 16 bytes)
-      *reinterpret_cast<bf16x2*>(&tile[j][cg + q]) = bf16x2{v[q], v[q + 1]};
-  }
-}
-
-// column c = t / 8 and c + 32 of the tile, rows 8 (t % 8) .. + 8, to out_row(c) + 8 (t % 8)
-template <typename OutPtr>
-__device__ __forceinline__ void tile_store_transposed(const bf16_t (&tile)[64][kTS], OutPtr out_row) {
-  const int t = threadIdx.x, pg = (t & 7) * 8;
-#pragma unroll
-  for (int h = 0; h < 2; ++h) {
-    const int c = (t >> 3) + 32 * h;
-    bf16x8 v;
-#pragma unroll
-    for (int q = 0; q < 8; ++q) v[q] = tile[pg + q][c];
-    *reinterpret_cast<bf16x8*>(out_row(c) + pg) = v;
-  }
-}
-
-// out[b][c][r] = in[b][r][c] for b < batch.  grid = (C / 64, R / 64, batch), 256 threads.
-__global__ __launch_bounds__(256) void transpose_batched_kernel(const bf16_t* __restrict__ in, int R, int C,
-                                                                bf16_t* __restrict__ out) {
-  __shared__ __attribute__((aligned(16))) bf16_t tile[64][kTS];
-  const size_t base = (size_t)blockIdx.z * R * C;
-  const int c0 = blockIdx.x * 64, r0 = blockIdx.y * 64;
-  tile_load(tile, [&](int j) { return in + base + (size_t)(r0 + j) * C + c0; }, [](int) { return 1.f; });
-  __syncthreads();
-  tile_store_transposed(tile, [&](int c) { return out + base + (size_t)(c0 + c) * R + r0; });
-}
-
-// pad_off[e] = sum over e' < e of the rows of e' rounded up to kPad (one wave; E <= 64)
-__global__ void pad_offsets_kernel(const int32_t* __restrict__ offsets, int E, int32_t* __restrict__ pad_off) {
-  const int lane = threadIdx.x;
-  int n = 0;
-  if (lane < E) n = (offsets[lane + 1] - offsets[lane] + kPad - 1) / kPad * kPad;
-  const int incl = wave_inclusive_scan(n);
-  if (lane < E) pad_off[lane + 1] = incl;
-  if (lane == 0) pad_off[0] = 0;
-}
-
-// outT[c][pad_off[e] + j] = scale * in[src(offsets[e] + j)][c] for the j-th row of expert e, zero in an expert's
-// padding columns.  src(r) = index[r] (or r); scale = scale_by_slot[slot_of_row[r]] (or 1).  grid = (ld / 64, C / 64):
-// a workgroup owns 64 columns of the padded row axis, which lie within one expert.
-__global__ __launch_bounds__(256) void transpose_rows_kernel(const bf16_t* __restrict__ in,
-                                                             const int32_t* __restrict__ index,
-                                                             const float* __restrict__ scale_by_slot,
-                                                             const int32_t* __restrict__ slot_of_row,
-                                                             const int32_t* __restrict__ offsets,
-                                                             const int32_t* __restrict__ pad_off, int E, int C, int ld,
-                                                             bf16_t* __restrict__ outT) {
-  __shared__ __attribute__((aligned(16))) bf16_t tile[64][kTS];
-  __shared__ int src_s[64];
-  __shared__ float scale_s[64];
-  const int p0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
-  if (p0 >= pad_off[E]) return;
-  int e = 0;
-  while (pad_off[e + 1] <= p0) ++e;                            // E <= 64 steps, uniform
-  if (threadIdx.x < 64) {
-    const int r = offsets[e] + (p0 - pad_off[e]) + threadIdx.x;
-    const bool live = r < offsets[e + 1];
-    src_s[threadIdx.x] = live ? (index ? index[r] : r) : -1;
-    scale_s[threadIdx.x] = (live && scale_by_slot) ? scale_by_slot[slot_of_row[r]] : 1.f;
-  }
-  __syncthreads();
-  tile_load(tile, [&](int j) { return src_s[j] >= 0 ? in + (size_t)src_s[j] * C + c0 : nullptr; },
-            [&](int j) { return scale_s[j]; });
-  __syncthreads();
-  tile_store_transposed(tile, [&](int c) { return outT + (size_t)(c0 + c) * ld + p0; });
-}
-
-// ---- weight gradients: dW[e][n][m] = sum over the padded rows kc of expert e of PT[n][kc] QT[m][kc] --------------
-// grid = (N / BM, M / BN, E).  Both operands are row-major with leading dimension ld and contiguous along kc.
-template <int MT, int NTW, int WM>
-__global__ __launch_bounds__(256 * WM) void wgrad_kernel(const bf16_t* __restrict__ PT, const bf16_t* __restrict__ QT,
-                                                         const int32_t* __restrict__ pad_off, int N, int M, int ld,
-                                                         bf16_t* __restrict__ dW) {
-  using S = Stripe<MT, NTW, WM, kBwdBK>;
-  constexpr int BM = S::BM, BN = S::BN;
-  __shared__ __attribute__((aligned(16))) bf16_t st0[S::kStageElems];
-  __shared__ __attribute__((aligned(16))) bf16_t st1[S::kStageElems];
-  const int e = blockIdx.z;
-  const int n0 = blockIdx.x * BM, m0 = blockIdx.y * BN;
-  const int k_lo = pad_off[e], K = pad_off[e + 1] - k_lo;
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const int wn = wave & 3, wm = wave >> 2;
-  floatx16 acc[MT][NTW];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-    for (int j = 0; j < NTW; ++j)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) acc[mt][j][i] = 0.f;
-  if (K > 0) {                                                   // an idle expert's gradient is zero
-    const int chunk = S::dma_chunk(tid);
-    StripeLoader<S> ldr;
-#pragma unroll
-    for (int i = 0; i < S::A_PER; ++i)
-      ldr.a_src[i] = PT + (size_t)(n0 + S::dma_row(tid) + i * S::kRowsPerInstr) * ld + k_lo + chunk * 8;
-    ldr.b_src = QT + (size_t)(m0 + S::dma_row(tid)) * ld + k_lo + chunk * 8;
-    ldr.bstep = (size_t)S::kRowsPerInstr * ld;
-    ldr.issue_stage(0, st0);
-    auto frag_row = [&](int j) { return (wn * NTW + j) * 32; };
-    stripe_mainloop_dma<MT, NTW, WM, S::BK, true>(acc, ldr, K, st0, st1, wm, frag_row);
-  }
-  // accumulators transposed: lane = row n0 + mbase + 32 mt + lane % 32, register 4 q + r = column
-  // m0 + (wn NTW + j) 32 + 8 q + 4 (lane / 32) + r
-  const int n = lane & 31, hh = lane >> 5;
-  bf16_t* orow = dW + ((size_t)e * N + n0 + wm * MT * 32 + n) * M + m0 + wn * NTW * 32 + 4 * hh;
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-    for (int j = 0; j < NTW; ++j)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        bf16x4 v;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) v[r] = (bf16_t)acc[mt][j][4 * q + r];
-        *reinterpret_cast<bf16x4*>(orow + (size_t)mt * 32 * M + j * 32 + 8 * q) = v;
-      }
-}
-
-template <int NTW>
-hipError_t launch_wgrad_t(const bf16_t* PT, const bf16_t* QT, const int32_t* pad_off, int N, int M, int ld, int E,
-                          bf16_t* dW, hipStream_t s) {
-  constexpr int MT = 2, WM = 2;
-  using St = Stripe<MT, NTW, WM, kBwdBK>;
-  hipLaunchKernelGGL((wgrad_kernel<MT, NTW, WM>), dim3(N / St::BM, M / St::BN, E), dim3(256 * WM), 0, s, PT, QT, pad_off, N,
-                     M, ld, dW);
+template <int NTW, bool GATHER, bool SCATTER>
+hipError_t launch_dgrad_t(const bf16_t* A, const int32_t* a_index, const bf16_t* W, const int32_t* offsets,
+                          const int32_t* out_index, int S_rows, int K, int N, int E, bf16_t* out, hipStream_t s) {
+  constexpr int BM = 128, BN = kSubW * NTW;
+  const int nblk_n = N / BN;
+  const int tiles = (S_rows / BM + E) * nblk_n;
+  const int grid = ((tiles + 7) & ~7) + 8;
+  hipLaunchKernelGGL((dgrad_kmajor_kernel<NTW, GATHER, SCATTER>), dim3(grid), dim3(512), 0, s, A, a_index, W, offsets,
+                     out_index, K, N, E, nblk_n, out);
   return hipGetLastError();
 }
 
-hipError_t launch_wgrad(const bf16_t* PT, const bf16_t* QT, const int32_t* pad_off, int N, int M, int ld, int E,
-                        bf16_t* dW, hipStream_t s) {
-  if (M % 384 == 0) return launch_wgrad_t<3>(PT, QT, pad_off, N, M, ld, E, dW, s);
-  if (M % 256 == 0) return launch_wgrad_t<2>(PT, QT, pad_off, N, M, ld, E, dW, s);
-  return launch_wgrad_t<1>(PT, QT, pad_off, N, M, ld, E, dW, s);
+// out[dst(r)] = A[src(r)] W[e] with W [E, K, N] as stored (kmajor.h)
+template <bool GATHER, bool SCATTER>
+hipError_t launch_dgrad(const bf16_t* A, const int32_t* a_index, const bf16_t* W, const int32_t* offsets,
+                        const int32_t* out_index, int S_rows, int K, int N, int E, bf16_t* out, hipStream_t s) {
+  if (N % 384 == 0) return launch_dgrad_t<3, GATHER, SCATTER>(A, a_index, W, offsets, out_index, S_rows, K, N, E, out, s);
+  if (N % 256 == 0) return launch_dgrad_t<2, GATHER, SCATTER>(A, a_index, W, offsets, out_index, S_rows, K, N, E, out, s);
+  return launch_dgrad_t<1, GATHER, SCATTER>(A, a_index, W, offsets, out_index, S_rows, K, N, E, out, s);
+}
+
+// dW[e] = P(rows of e)^T Q(rows of e), P [.., N] and Q [.., M] row-major (kmajor.h)
+template <bool GATHER_P, bool GATHER_Q>
+hipError_t launch_wgrad(const bf16_t* P, const bf16_t* Q, const int32_t* index, const int32_t* offsets, const bf16_t* zrow,
+                        int N, int M, int S_rows, int E, bf16_t* dW, hipStream_t s) {
+  const dim3 block(512);
+  auto grid = [&](int bn) { return dim3((unsigned)((E * (N / 128) * (M / bn) + 7) & ~7)); };
+  if (M % 384 == 0)
+    hipLaunchKernelGGL((wgrad_kmajor_kernel<3, GATHER_P, GATHER_Q>), grid(384), block, 0, s, P, Q, index, offsets, zrow, N, M, E,
+                       dW);
+  else if (M % 256 == 0)
+    hipLaunchKernelGGL((wgrad_kmajor_kernel<2, GATHER_P, GATHER_Q>), grid(256), block, 0, s, P, Q, index, offsets, zrow, N, M, E,
+                       dW);
+  else
+    hipLaunchKernelGGL((wgrad_kmajor_kernel<1, GATHER_P, GATHER_Q>), grid(128), block, 0, s, P, Q, index, offsets, zrow, N, M, E,
+                       dW);
+  return hipGetLastError();
 }
 
 // ---- Radial NormSiLU backward (moe.py:87-92), one wave per permuted row ----------------------------------------
 // h = r^p a u, a = SiLU(z) = z s, s = sigmoid(z), z = g / r, a' = s (1 + z (1 - s)); with q = dh u:
 //   du = dh r^p a;  dg = q r^(p-1) a' + g / (I r) sum_i q_i (p r^(p-1) a_i - r^(p-2) a'_i g_i);
 //   dtheta (the row's share) = p'(theta) ln r sum_i q_i r^p a_i;  dw = <dh', h>, dh = w dh'.
+// `hidden` receives w h, the row the down projection's weight gradient contracts with d_out.
 // act = SiLU: h = SiLU(g) u, dg = q a'(g), no theta.  Rows of I <= kActMaxI elements.
 constexpr int kActMaxI = 512;   // one 16-byte granule of the row per lane
 
@@ -370,7 +245,7 @@ __global__ __launch_bounds__(256) void act_bwd_kernel(const bf16_t* __restrict__
       if (radial) dg = fmaf(g[q] * rinv / (float)I, inner, dg);
       og[q] = (bf16_t)dg;
       ou[q] = (bf16_t)(dh * gain * a_[q]);
-      oh[q] = (bf16_t)(gain * a_[q] * u[q]);
+      oh[q] = (bf16_t)(ws * gain * a_[q] * u[q]);              // w h: the weight gradient's operand (moe.py:92-93)
     }
     *reinterpret_cast<bf16x8*>(dgu + (size_t)row * 2 * I + lane * 8) = og;
     *reinterpret_cast<bf16x8*>(dgu + (size_t)row * 2 * I + I + lane * 8) = ou;
@@ -555,12 +430,12 @@ bool backward_supported(int H, int I, int k, int dtype) {
 
 int backward_dwr_split() { return kDwrSplit; }
 
-// leading dimension of the transposed activation buffers: every expert's rows padded to a multiple of kPad
-size_t backward_padded_rows(int T, int E, int k) { return ((size_t)T * k + (size_t)E * (kPad - 1) + kPad - 1) / kPad * kPad; }
+// a row of zeros as wide as the widest weight-gradient operand: what a K stage reads past an expert's last row
+size_t backward_zero_row_bytes(int H, int I) { return (size_t)(H > 2 * I ? H : 2 * I) * sizeof(bf16_t); }
 
-// The launches after routing and permutation.  Buffers (bf16 unless noted): wd_t [E,I,H], wgu_t [E,H,2I], gu [S,2I],
-// dhp [S,I], dgu [S,2I], hidden [S,I], dxs [S,H], p_t [max(H,2I), ld], q_t [max(H,I), ld], dw_slot [S] f32,
-// dl [S] f32, dtheta_row [S] f32, dwr_part [E, backward_dwr_split(), H] f32, pad_off [E+1] i32.
+// The launches after routing and permutation.  Buffers (bf16 unless noted): gu [S,2I], dhp [S,I], dgu [S,2I],
+// hidden [S,I], dxs [S,H], zrow [max(H, 2I)] (zeroed here), dw_slot [S] f32, dl [S] f32, dtheta_row [S] f32,
+// dwr_part [E, backward_dwr_split(), H] f32.
 hipError_t launch_backward(const void* x, const void* d_out, const void* w_router, const void* wgu, const void* wd,
                            const float* theta, const float* logits, const int32_t* idx, const float* w,
                            const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token, int T, int H, int E,
@@ -572,16 +447,14 @@ hipError_t launch_backward(const void* x, const void* d_out, const void* w_route
   const bf16_t* xp = static_cast<const bf16_t*>(x);
   const bf16_t* dop = static_cast<const bf16_t*>(d_out);
   const bf16_t* wrp = static_cast<const bf16_t*>(w_router);
-  bf16_t* wd_t = static_cast<bf16_t*>(b.wd_t);
-  bf16_t* wgu_t = static_cast<bf16_t*>(b.wgu_t);
+  const bf16_t* wgup = static_cast<const bf16_t*>(wgu);
+  const bf16_t* wdp = static_cast<const bf16_t*>(wd);
   bf16_t* gu = static_cast<bf16_t*>(b.gu);
   bf16_t* dhp = static_cast<bf16_t*>(b.dhp);
   bf16_t* dgu = static_cast<bf16_t*>(b.dgu);
   bf16_t* hidden = static_cast<bf16_t*>(b.hidden);
   bf16_t* dxs = static_cast<bf16_t*>(b.dxs);
-  bf16_t* p_t = static_cast<bf16_t*>(b.p_t);
-  bf16_t* q_t = static_cast<bf16_t*>(b.q_t);
-  const int ld = (int)backward_padded_rows(T, Et, k);
+  bf16_t* zrow = static_cast<bf16_t*>(b.zrow);
   hipError_t err = hipSuccess;
   if (S == 0) {
     zero_bytes(d_theta, (size_t)E * sizeof(float), s);
@@ -590,22 +463,18 @@ hipError_t launch_backward(const void* x, const void* d_out, const void* w_route
     zero_bytes(d_wd, (size_t)E * H * I * sizeof(bf16_t), s);
     return hipGetLastError();
   }
-  hipLaunchKernelGGL(pad_offsets_kernel, dim3(1), dim3(64), 0, s, offsets, E, b.pad_off);
-  // transposed weights: wd [E,H,I] -> [E,I,H]; wgu [E,2I,H] -> [E,H,2I]
-  hipLaunchKernelGGL(transpose_batched_kernel, dim3(I / 64, H / 64, E), dim3(256), 0, s, static_cast<const bf16_t*>(wd), H, I,
-                     wd_t);
-  hipLaunchKernelGGL(transpose_batched_kernel, dim3(H / 64, 2 * I / 64, E), dim3(256), 0, s,
-                     static_cast<const bf16_t*>(wgu), 2 * I, H, wgu_t);
-  // pre-activations again (moe.py:84) and dh' = d W_down (both gather their rows by token)
-  err = launch_ggemm<true, false>(xp, perm_token, static_cast<const bf16_t*>(wgu), offsets, nullptr, S, H, 2 * I, E, gu, s);
+  zero_bytes(zrow, backward_zero_row_bytes(H, I), s);
+  // pre-activations again (moe.py:84): x W_gate_up^T, both contiguous along H
+  err = launch_ggemm<true, false>(xp, perm_token, wgup, offsets, nullptr, S, H, 2 * I, E, gu, s);
   if (err != hipSuccess) return err;
-  err = launch_ggemm<true, false>(dop, perm_token, wd_t, offsets, nullptr, S, H, I, E, dhp, s);
+  // dh' = d W_down: contracts over H, the middle dimension of w_down [E, H, I]
+  err = launch_dgrad<true, false>(dop, perm_token, wdp, offsets, nullptr, S, H, I, E, dhp, s);
   if (err != hipSuccess) return err;
   hipLaunchKernelGGL(act_bwd_kernel, dim3((S + 3) / 4), dim3(256), 0, s, gu, dhp, w, theta, offsets, perm_slot, S, E, I, act,
                      dgu, hidden, b.dw_slot, b.dtheta_row);
   hipLaunchKernelGGL(dtheta_reduce_kernel, dim3(E), dim3(256), 0, s, b.dtheta_row, offsets, d_theta);
-  // dx of every slot, in slot order: [dg, du] W_gate_up
-  err = launch_ggemm<false, true>(dgu, nullptr, wgu_t, offsets, perm_slot, S, 2 * I, H, E, dxs, s);
+  // dx of every slot, in slot order: [dg, du] W_gate_up, contracts over the 2I rows of w_gate_up [E, 2I, H]
+  err = launch_dgrad<false, true>(dgu, nullptr, wgup, offsets, perm_slot, S, 2 * I, H, E, dxs, s);
   if (err != hipSuccess) return err;
   if (n_pos + n_neg > 0)   // (as many waves as there could be rows: how many there are is only known on the device)
     hipLaunchKernelGGL(special_bwd_kernel, dim3((S + 3) / 4), dim3(256), 0, s, xp, dop, w, offsets, perm_slot, perm_token, E,
@@ -622,19 +491,11 @@ hipError_t launch_backward(const void* x, const void* d_out, const void* w_route
     hipLaunchKernelGGL(dwr_sum_kernel, dim3((Et * H + 255) / 256), dim3(256), 0, s, b.dwr_part, H, Et * H,
                        static_cast<bf16_t*>(d_w_router));
   }
-  // weight gradients: dW_down[e] = (w d)^T h, dW_gate_up[e] = [dg, du]^T x, contracted over the expert's rows
-  const dim3 tgrid_h(ld / 64, H / 64), tgrid_i(ld / 64, I / 64), tgrid_2i(ld / 64, 2 * I / 64);
-  hipLaunchKernelGGL(transpose_rows_kernel, tgrid_h, dim3(256), 0, s, dop, perm_token, w, perm_slot, offsets, b.pad_off, E, H,
-                     ld, p_t);
-  hipLaunchKernelGGL(transpose_rows_kernel, tgrid_i, dim3(256), 0, s, hidden, nullptr, nullptr, nullptr, offsets, b.pad_off, E,
-                     I, ld, q_t);
-  err = launch_wgrad(p_t, q_t, b.pad_off, H, I, ld, E, static_cast<bf16_t*>(d_wd), s);
+  // weight gradients, contracted over each expert's rows: dW_down[e] = d^T (w h) (d gathered by token, `hidden`
+  // already carries w), dW_gate_up[e] = [dg, du]^T x (x gathered by token)
+  err = launch_wgrad<true, false>(dop, hidden, perm_token, offsets, zrow, H, I, S, E, static_cast<bf16_t*>(d_wd), s);
   if (err != hipSuccess) return err;
-  hipLaunchKernelGGL(transpose_rows_kernel, tgrid_2i, dim3(256), 0, s, dgu, nullptr, nullptr, nullptr, offsets, b.pad_off, E,
-                     2 * I, ld, p_t);
-  hipLaunchKernelGGL(transpose_rows_kernel, tgrid_h, dim3(256), 0, s, xp, perm_token, nullptr, nullptr, offsets, b.pad_off, E,
-                     H, ld, q_t);
-  err = launch_wgrad(p_t, q_t, b.pad_off, 2 * I, H, ld, E, static_cast<bf16_t*>(d_wgu), s);
+  err = launch_wgrad<false, true>(dgu, xp, perm_token, offsets, zrow, 2 * I, H, S, E, static_cast<bf16_t*>(d_wgu), s);
   if (err != hipSuccess) return err;
   return hipGetLastError();
 }

@@ -217,13 +217,12 @@ hipError_t launch_attn_res(const void* const* cands, int n_cand, const float* sc
 
 // ---- backward pass (backward.hip) ----
 struct BackwardBuffers {
-  void *wd_t, *wgu_t, *gu, *dhp, *dgu, *hidden, *dxs, *p_t, *q_t;   // bf16 device buffers, sizes in launch_backward's comment
+  void *gu, *dhp, *dgu, *hidden, *dxs, *zrow;                       // bf16 device buffers, sizes in launch_backward's comment
   float *dw_slot, *dl, *dtheta_row;                                 // [T*k] each
   float* dwr_part;                                                  // [E, backward_dwr_split(), H]
-  int32_t* pad_off;                                                 // [E + 1]
 };
 bool backward_supported(int H, int I, int k, int dtype);
-size_t backward_padded_rows(int T, int E, int k);
+size_t backward_zero_row_bytes(int H, int I);
 int backward_dwr_split();
 hipError_t launch_backward(const void* x, const void* d_out, const void* w_router, const void* wgu, const void* wd,
                            const float* theta, const float* logits, const int32_t* idx, const float* w,
