@@ -18,31 +18,22 @@ namespace {
 typedef short v4i16 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) v4i16 lds_v4i16;
 
-constexpr int kKS = 64;                 // k rows per LDS stage
+constexpr int kKS = 32;                 // k rows per LDS stage
+constexpr int kRing = 4;                // stages in LDS: one being multiplied, two on their way, one being requested
 constexpr int kSubW = 128;              // n elements per sub-tile row (256 bytes: whole 128-byte lines per DMA row)
-constexpr int kSubElems = kKS * kSubW;  // 16 KB
+constexpr int kSubElems = kKS * kSubW;  // 8 KB: one LDS-DMA instruction of the 512 threads
+constexpr int kATile = 128 * kKS;       // row-major operand tile, 128 rows: 8 KB as well
 
-// LDS layout of a K-major sub-tile [64 k][128 n]: 16-byte granule G of row k sits at position G ^ ((k & 3) << 2).
+// LDS layout of a K-major sub-tile [32 k][128 n]: 16-byte granule G of row k sits at position G ^ ((k & 3) << 2).
 // The four k rows one transposed read touches then lie in four different 64-byte quarters of the 256-byte bank
-// period, so the read has no bank conflicts.
+// period, so the read has no bank conflicts.  Thread t of the fill writes row t / 16, position t % 16, and therefore
+// fetches granule (t % 16) ^ (((t / 16) & 3) << 2) of that row.
+__device__ __forceinline__ int kfill_granule(int tid) { return (tid & 15) ^ (((tid >> 4) & 3) << 2); }
 
-// What a thread contributes to the fill of K-major sub-tiles: with 512 threads an instruction moves 512 granules =
-// 32 rows of 16, so thread t handles rows t / 16 and 32 + t / 16, position t % 16.
-struct KFill {
-  int krow;        // t / 16
-  int gcol;        // logical granule this thread fetches for row krow AND row krow + 32 (both have the same k & 3)
-  __device__ __forceinline__ void init(int tid) {
-    krow = tid >> 4;
-    gcol = (tid & 15) ^ ((krow & 3) << 2);
-  }
-};
-
-// Fill one sub-tile from two row pointers (the rows krow and krow + 32 of the stage, already offset to the sub-tile's
-// first column).
-__device__ __forceinline__ void kfill_subtile(const KFill& f, const bf16_t* row_a, const bf16_t* row_b, bf16_t* sub) {
-  const int wave_elems = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)) * 64 * 8;
-  dma16(row_a + f.gcol * 8, sub + wave_elems);
-  dma16(row_b + f.gcol * 8, sub + 512 * 8 + wave_elems);
+// Fill one sub-tile: `row` = this thread's row (tid / 16) of the stage, already offset to the sub-tile's first
+// column and to this thread's granule.
+__device__ __forceinline__ void kfill_subtile(const bf16_t* row, bf16_t* sub) {
+  dma16(row, sub + __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)) * 64 * 8);
 }
 
 // Per-lane element offset, inside a sub-tile, of the first transposed read of the 32 (n) x 16 (k) fragment whose
@@ -66,24 +57,25 @@ __device__ __forceinline__ bf16x8 kfrag_read(const bf16_t* sub, int off) {
   return __builtin_bit_cast(bf16x8, v);
 }
 
-// the same with the step as a loop variable of an unrolled loop (folds to one of the four)
+// the same with the step as a loop variable of an unrolled loop (folds to one of the two)
 __device__ __forceinline__ bf16x8 kfrag_read_s(const bf16_t* sub, int off, int s) {
-  return s == 0 ? kfrag_read<0>(sub, off) : s == 1 ? kfrag_read<1>(sub, off) : s == 2 ? kfrag_read<2>(sub, off)
-                                                                                      : kfrag_read<3>(sub, off);
+  return s == 0 ? kfrag_read<0>(sub, off) : kfrag_read<1>(sub, off);
 }
 
-// One K stage (four k16 steps) of a wave's MT x NTW tiles as a software pipeline: the fragments of step s + 1 are read
-// while step s is multiplied, two LDS reads behind every MFMA.  read_a(s, mt) / read_b(s, j) return the fragments.
+// One K stage (two k16 steps) of a wave's MT x NTW tiles as a software pipeline: the fragments of the second step
+// are read while the first is multiplied, two LDS reads behind every MFMA.  read_a(s, mt) / read_b(s, j) return the
+// fragments.
 template <int MT, int NTW, typename ReadA, typename ReadB>
 __device__ __forceinline__ void multiply_stage(floatx16 (&acc)[MT][NTW], ReadA read_a, ReadB read_b) {
+  constexpr int kSteps = kKS / 16;
   bf16x8 af[2][MT], bfr[2][NTW];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) af[0][mt] = read_a(0, mt);
 #pragma unroll
   for (int j = 0; j < NTW; ++j) bfr[0][j] = read_b(0, j);
 #pragma unroll
-  for (int s = 0; s < 4; ++s) {
-    if (s < 3) {
+  for (int s = 0; s < kSteps; ++s) {
+    if (s + 1 < kSteps) {
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) af[(s + 1) & 1][mt] = read_a(s + 1, mt);
 #pragma unroll
@@ -98,25 +90,29 @@ __device__ __forceinline__ void multiply_stage(floatx16 (&acc)[MT][NTW], ReadA r
 #pragma unroll
     for (int i = 0; i < MT * NTW; ++i) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      if (s < 3) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      if (s + 1 < kSteps) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
     }
   }
 }
 
-// Row-major A tile [128 rows][64 k] in the stripe layout (granule c of row r at c ^ ((r >> 1) & 7)): fill by 512
-// threads, two instructions; thread t handles rows t / 8 and 64 + t / 8.
-__device__ __forceinline__ void afill(const bf16_t* row_a, const bf16_t* row_b, bf16_t* tile) {
-  const int tid = threadIdx.x;
-  const int wave_elems = __builtin_amdgcn_readfirstlane(tid >> 6) * 64 * 8;
-  const int g = (tid & 7) ^ ((tid >> 4) & 7);                  // rows t / 8 and 64 + t / 8 have the same (row >> 1) & 7
-  dma16(row_a + g * 8, tile + wave_elems);
-  dma16(row_b + g * 8, tile + 512 * 8 + wave_elems);
+// Row-major operand tile [128 rows][32 k] in the stripe layout for 64-byte rows (granule c of row r at
+// c ^ ((r >> 2) & 3)): thread t of the fill writes row t / 4, position t % 4.  `row` = that row's K extent, already
+// offset to the stage's first k and to this thread's granule (afill_granule).
+__device__ __forceinline__ int afill_granule(int tid) { return (tid & 3) ^ ((tid >> 4) & 3); }
+__device__ __forceinline__ void afill(const bf16_t* row, bf16_t* tile) {
+  dma16(row, tile + __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)) * 64 * 8);
 }
+
+// The stages form a ring of four, each a __shared__ variable of its own (the compiler orders an LDS-DMA transfer
+// against later reads of the same variable with a full wait).  Step i of the K loop waits until the transfers of
+// stage i have landed (those of stages i + 1 and i + 2 may stay in flight: loads complete in order), meets the other
+// waves, requests stage i + 3 into the buffer stage i - 1 was read from, and multiplies stage i.  Every step issues
+// the same number of transfers (a request past the last stage repeats the last one), so the wait count is a constant.
 
 // ---- input gradients: out[dst(r), n] = sum_k A[src(r), k] W[e][k, n] for the rows r of expert e ----------------
 // A row-major (K contiguous), W K-major as stored: [K, N] per expert.  src(r) = a_index[r] (GATHER) or r; dst(r) =
 // out_index[r] (SCATTER) or r.  Workgroup = 128 rows x 128 NTW columns, 2 x 4 waves, 32x32x16 MFMA, operands swapped
-// so that a lane owns one output row.
+// so that a lane owns one output row.  K is a multiple of 128.
 template <int NTW, bool GATHER, bool SCATTER>
 __global__ __launch_bounds__(512) void dgrad_kmajor_kernel(const bf16_t* __restrict__ A, const int32_t* __restrict__ a_index,
                                                            const bf16_t* __restrict__ W,
@@ -124,11 +120,15 @@ __global__ __launch_bounds__(512) void dgrad_kmajor_kernel(const bf16_t* __restr
                                                            const int32_t* __restrict__ out_index, int K, int N, int E,
                                                            int nblk_n, bf16_t* __restrict__ out) {
   constexpr int MT = 2, BM = 128, BN = kSubW * NTW;
-  constexpr int kATile = BM * kKS;
+  constexpr int kOps = 1 + NTW;                          // transfers per thread and stage
   __shared__ __attribute__((aligned(16))) bf16_t a0[kATile];
   __shared__ __attribute__((aligned(16))) bf16_t a1[kATile];
+  __shared__ __attribute__((aligned(16))) bf16_t a2[kATile];
+  __shared__ __attribute__((aligned(16))) bf16_t a3[kATile];
   __shared__ __attribute__((aligned(16))) bf16_t b0[NTW * kSubElems];
   __shared__ __attribute__((aligned(16))) bf16_t b1[NTW * kSubElems];
+  __shared__ __attribute__((aligned(16))) bf16_t b2[NTW * kSubElems];
+  __shared__ __attribute__((aligned(16))) bf16_t b3[NTW * kSubElems];
   __shared__ int dst_s[BM];
 
   const TileMap tm = make_tile_map(offsets, E, BM);
@@ -146,23 +146,30 @@ __global__ __launch_bounds__(512) void dgrad_kmajor_kernel(const bf16_t* __restr
     dst_s[tid] = SCATTER ? out_index[r] : r;
   }
   // fill side
-  const bf16_t* arow[2];
-#pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int r = row0 + min((tid >> 3) + 64 * i, rows - 1);        // rows past the end re-read the last one
-    arow[i] = A + (size_t)(GATHER ? a_index[r] : r) * K;
-  }
-  KFill kf;
-  kf.init(tid);
+  const int ar = row0 + min(tid >> 2, rows - 1);                   // rows past the end re-read the last one
+  const bf16_t* arow = A + (size_t)(GATHER ? a_index[ar] : ar) * K + afill_granule(tid) * 8;
   const int n0 = nb * BN;
-  const bf16_t* wrow = W + (size_t)e * K * N + (size_t)kf.krow * N + n0;   // row krow of the first stage; + 32 N: the other
-  auto fill = [&](int k0, bf16_t* at, bf16_t* bt) {
-    afill(arow[0] + k0, arow[1] + k0, at);
+  const bf16_t* wrow = W + (size_t)e * K * N + (size_t)(tid >> 4) * N + n0 + kfill_granule(tid) * 8;
+  const int nstages = K / kKS;
+  auto abuf = [&](auto bc) -> bf16_t* {
+    constexpr int b = decltype(bc)::value;
+    if constexpr (b == 0) return a0; else if constexpr (b == 1) return a1; else if constexpr (b == 2) return a2; else return a3;
+  };
+  auto bbuf = [&](auto bc) -> bf16_t* {
+    constexpr int b = decltype(bc)::value;
+    if constexpr (b == 0) return b0; else if constexpr (b == 1) return b1; else if constexpr (b == 2) return b2; else return b3;
+  };
+  auto fill = [&](auto bc, int stage) {
+    const int k0 = min(stage, nstages - 1) * kKS;
+    afill(arow + k0, abuf(bc));
     const bf16_t* w0 = wrow + (size_t)k0 * N;
 #pragma unroll
-    for (int j = 0; j < NTW; ++j) kfill_subtile(kf, w0 + j * kSubW, w0 + (size_t)32 * N + j * kSubW, bt + j * kSubElems);
+    for (int j = 0; j < NTW; ++j) kfill_subtile(w0 + j * kSubW, bbuf(bc) + j * kSubElems);
   };
-  fill(0, a0, b0);
+  using std::integral_constant;
+  fill(integral_constant<int, 0>{}, 0);
+  fill(integral_constant<int, 1>{}, 1);
+  fill(integral_constant<int, 2>{}, 2);
 
   floatx16 acc[MT][NTW];
 #pragma unroll
@@ -176,7 +183,7 @@ __global__ __launch_bounds__(512) void dgrad_kmajor_kernel(const bf16_t* __restr
   // columns (wn NTW + j) 32 of the block = sub-tile (wn NTW + j) / 4, column ((wn NTW + j) % 4) 32 inside it.
   const int n = lane & 31, h = lane >> 5;
   const int mbase = wm * MT * 32;
-  const int apos0 = (h ^ ((n >> 1) & 7)) * 8;
+  const int apos0 = (h ^ ((n >> 2) & 3)) * 8;
   const int aoff = (mbase + n) * kKS;
   int boff[NTW];
 #pragma unroll
@@ -184,31 +191,33 @@ __global__ __launch_bounds__(512) void dgrad_kmajor_kernel(const bf16_t* __restr
     const int t32 = wn * NTW + j;
     boff[j] = (t32 >> 2) * kSubElems + kfrag_offset(lane, (t32 & 3) * 32);
   }
-  auto multiply = [&](const bf16_t* at, const bf16_t* bt) {
+  auto step = [&](auto bc, auto nc, int stage) {
+    sync_keep_loads<2 * kOps>();
+    fill(nc, stage + 3);
+    const bf16_t* at = abuf(bc);
+    const bf16_t* bt = bbuf(bc);
     multiply_stage<MT, NTW>(
         acc,
         [&](int s, int mt) { return *reinterpret_cast<const bf16x8*>(at + aoff + mt * 32 * kKS + (apos0 ^ (s * 16))); },
         [&](int s, int j) { return kfrag_read_s(bt, boff[j], s); });
   };
-  for (int k0 = 0; k0 < K; k0 += 2 * kKS) {
-    wait_loads_and_sync();
-    if (k0 + kKS < K) fill(k0 + kKS, a1, b1);
-    multiply(a0, b0);
-    if (k0 + kKS < K) {
-      wait_loads_and_sync();
-      if (k0 + 2 * kKS < K) fill(k0 + 2 * kKS, a0, b0);
-      multiply(a1, b1);
-    }
+  for (int i = 0; i < nstages; i += 4) {                           // nstages is a multiple of 4
+    step(integral_constant<int, 0>{}, integral_constant<int, 3>{}, i);
+    step(integral_constant<int, 1>{}, integral_constant<int, 0>{}, i + 1);
+    step(integral_constant<int, 2>{}, integral_constant<int, 1>{}, i + 2);
+    step(integral_constant<int, 3>{}, integral_constant<int, 2>{}, i + 3);
   }
+  wait_loads_and_sync();                 // the repeated requests of the last steps have landed; every wave is done reading
 
   // Epilogue (accumulators transposed: lane = row, four consecutive columns per register quad): 32 rows at a time
   // through a wave-private LDS tile, out as 16-byte row segments.
   const int hh = lane >> 5;
   constexpr int kOutCols = NTW * 32;
   constexpr int kOutStride = kOutCols + 8;          // +16 bytes staggers the rows over the banks
-  static_assert(4 * 32 * kOutStride <= NTW * kSubElems, "output staging does not fit a weight stage");
-  __syncthreads();                       // every wave is done reading the stage buffers
-  bf16_t* otile = (wave < 4 ? b0 : b1) + (wave & 3) * (32 * kOutStride);
+  static_assert(2 * 32 * kOutStride <= NTW * kSubElems, "output staging does not fit a weight stage");
+  bf16_t* otile = bbuf(integral_constant<int, 0>{});
+  if (wave >= 6) otile = b3; else if (wave >= 4) otile = b2; else if (wave >= 2) otile = b1;
+  otile += (wave & 1) * (32 * kOutStride);
   constexpr int kGranPerRow = kOutCols / 8;
   const int colbase = n0 + wn * kOutCols;
 #pragma unroll
@@ -238,8 +247,9 @@ __global__ __launch_bounds__(512) void dgrad_kmajor_kernel(const bf16_t* __restr
 
 // ---- weight gradients: dW[e][n][m] = sum over the rows r of expert e of P[srcP(r)][n] Q[srcQ(r)][m] ------------
 // Both operands row-major activations, contracted over their rows: K-major both.  srcP(r) = index[r] (GATHER_P) or r,
-// likewise Q.  A K stage is 64 rows; rows past the expert's end read `zrow` (zeros, at least 128 elements) on the P
-// side.  One workgroup per (expert, 128 rows of dW, 128 NTW columns of dW).
+// likewise Q.  A K stage is 32 rows; rows past the expert's end read `zrow` (zeros, at least 128 elements) on the P
+// side and the expert's last row on the Q side (memory that is certainly finite, whatever the rows behind the
+// expert's hold).  One workgroup per (expert, 128 rows of dW, 128 NTW columns of dW).
 template <int NTW, bool GATHER_P, bool GATHER_Q>
 __global__ __launch_bounds__(512) void wgrad_kmajor_kernel(const bf16_t* __restrict__ P, const bf16_t* __restrict__ Q,
                                                            const int32_t* __restrict__ index,
@@ -247,10 +257,15 @@ __global__ __launch_bounds__(512) void wgrad_kmajor_kernel(const bf16_t* __restr
                                                            const bf16_t* __restrict__ zrow, int N, int M, int E,
                                                            bf16_t* __restrict__ dW) {
   constexpr int MT = 2, BM = 128, BN = kSubW * NTW;
+  constexpr int kOps = 1 + NTW;
   __shared__ __attribute__((aligned(16))) bf16_t p0[kSubElems];
   __shared__ __attribute__((aligned(16))) bf16_t p1[kSubElems];
+  __shared__ __attribute__((aligned(16))) bf16_t p2[kSubElems];
+  __shared__ __attribute__((aligned(16))) bf16_t p3[kSubElems];
   __shared__ __attribute__((aligned(16))) bf16_t q0[NTW * kSubElems];
   __shared__ __attribute__((aligned(16))) bf16_t q1[NTW * kSubElems];
+  __shared__ __attribute__((aligned(16))) bf16_t q2[NTW * kSubElems];
+  __shared__ __attribute__((aligned(16))) bf16_t q3[NTW * kSubElems];
   // Workgroup ids congruent mod 8 run on one XCD: they walk a contiguous range of (expert, m block, n block) triples,
   // so the workgroups that read the same rows of Q (and of P) share that XCD's L2.
   const int nblk_n = N / BM, nblk_m = M / BN;
@@ -258,7 +273,7 @@ __global__ __launch_bounds__(512) void wgrad_kmajor_kernel(const bf16_t* __restr
   if (item >= E * nblk_n * nblk_m) return;
   const int e = item / (nblk_n * nblk_m), rest = item - e * (nblk_n * nblk_m);
   const int n0 = (rest % nblk_n) * BM, m0 = (rest / nblk_n) * BN;
-  const int lo = offsets[e], hi = offsets[e + 1];
+  const int lo = __builtin_amdgcn_readfirstlane(offsets[e]), hi = __builtin_amdgcn_readfirstlane(offsets[e + 1]);
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int wn = wave & 3, wm = wave >> 2;
   floatx16 acc[MT][NTW];
@@ -269,23 +284,30 @@ __global__ __launch_bounds__(512) void wgrad_kmajor_kernel(const bf16_t* __restr
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[mt][j][i] = 0.f;
 
-  KFill kf;
-  kf.init(tid);
-  // rows lo + k0 + krow and + 32 of every stage; their source rows, one stage ahead of the fill that uses them
-  // (a row past the expert's end reads zeros on the P side and, on the Q side, the expert's last row: memory that is
-  // certainly finite, whatever the rows behind the expert's hold)
-  auto source = [&](int r, const bf16_t*& prow, const bf16_t*& qrow) {
+  auto pbuf = [&](auto bc) -> bf16_t* {
+    constexpr int b = decltype(bc)::value;
+    if constexpr (b == 0) return p0; else if constexpr (b == 1) return p1; else if constexpr (b == 2) return p2; else return p3;
+  };
+  auto qbuf = [&](auto bc) -> bf16_t* {
+    constexpr int b = decltype(bc)::value;
+    if constexpr (b == 0) return q0; else if constexpr (b == 1) return q1; else if constexpr (b == 2) return q2; else return q3;
+  };
+  const int nstages = (hi - lo + kKS - 1) / kKS;
+  const int gofs = kfill_granule(tid) * 8;
+  // This thread's row of stage `stage` (row tid / 16 of the stage's 32), the expert's last row past its end.
+  auto stage_row = [&](int stage) { return lo + min(stage, nstages - 1) * kKS + (tid >> 4); };
+  auto lookup = [&](int stage) {
+    return (GATHER_P || GATHER_Q) ? index[min(stage_row(stage), hi - 1)] : 0;
+  };
+  auto fill = [&](auto bc, int stage, int ix) {
+    const int r = stage_row(stage);
     const bool live = r < hi;
     const int rc = live ? r : hi - 1;
-    const int ix = (GATHER_P || GATHER_Q) ? index[rc] : 0;
-    prow = live ? P + (size_t)(GATHER_P ? ix : rc) * N + n0 : zrow;
-    qrow = Q + (size_t)(GATHER_Q ? ix : rc) * M + m0;
-  };
-  const bf16_t *pa, *pb, *qa, *qb;
-  auto fill = [&](bf16_t* pt, bf16_t* qt) {
-    kfill_subtile(kf, pa, pb, pt);
+    const bf16_t* prow = live ? P + (size_t)(GATHER_P ? ix : rc) * N + n0 : zrow;
+    const bf16_t* qrow = Q + (size_t)(GATHER_Q ? ix : rc) * M + m0;
+    kfill_subtile(prow + gofs, pbuf(bc));
 #pragma unroll
-    for (int j = 0; j < NTW; ++j) kfill_subtile(kf, qa + j * kSubW, qb + j * kSubW, qt + j * kSubElems);
+    for (int j = 0; j < NTW; ++j) kfill_subtile(qrow + j * kSubW + gofs, qbuf(bc) + j * kSubElems);
   };
   int poff[MT], qoff[NTW];
 #pragma unroll
@@ -295,37 +317,41 @@ __global__ __launch_bounds__(512) void wgrad_kmajor_kernel(const bf16_t* __restr
     const int t32 = wn * NTW + j;
     qoff[j] = (t32 >> 2) * kSubElems + kfrag_offset(lane, (t32 & 3) * 32);
   }
-  auto multiply = [&](const bf16_t* pt, const bf16_t* qt) {
-    multiply_stage<MT, NTW>(
-        acc, [&](int s, int mt) { return kfrag_read_s(pt, poff[mt], s); },
-        [&](int s, int j) { return kfrag_read_s(qt, qoff[j], s); });
-  };
-  if (hi > lo) {                                                   // an idle expert's gradient is zero
-    // The source rows of a stage (two index loads per thread when an operand is gathered) are looked up a stage
-    // before the fill that uses them, right after the fill before it, so the loads fly during a multiply.
-    const int r_a = lo + kf.krow;
-    auto sources = [&](int k0) { source(r_a + k0, pa, qa); source(r_a + k0 + 32, pb, qb); };
-    sources(0);
-    fill(p0, q0);
-    if (lo + kKS < hi) sources(kKS);
-    for (int k0 = 0; lo + k0 < hi; k0 += 2 * kKS) {
-      const bool more1 = lo + k0 + kKS < hi;
-      wait_loads_and_sync();
-      if (more1) {
-        fill(p1, q1);
-        if (lo + k0 + 2 * kKS < hi) sources(k0 + 2 * kKS);
+  using std::integral_constant;
+  if (nstages > 0) {                                               // an idle expert's gradient is zero
+    // The row index of a gathered operand is loaded three steps before the transfers that use it (four values
+    // rotate through ix[]): step s requests stage s + 3 with the index loaded at step s - 3 and loads the one of
+    // stage s + 6.  That load is one more vector-memory operation per step, so the ring's wait counts it.
+    constexpr int kVm = kOps + ((GATHER_P || GATHER_Q) ? 1 : 0);
+    int ix[4];
+    ix[0] = lookup(0); ix[1] = lookup(1); ix[2] = lookup(2);
+    fill(integral_constant<int, 0>{}, 0, ix[0]);
+    ix[3] = lookup(3);
+    fill(integral_constant<int, 1>{}, 1, ix[1]);
+    ix[0] = lookup(4);
+    fill(integral_constant<int, 2>{}, 2, ix[2]);
+    ix[1] = lookup(5);
+    // now in flight, oldest first: stage 0, index 3, stage 1, index 4, stage 2, index 5
+    auto step = [&](auto bc, auto nc, int stage) {
+      constexpr int b = decltype(bc)::value;
+      sync_keep_loads<2 * kVm>();
+      fill(nc, stage + 3, ix[(b + 3) & 3]);
+      ix[(b + 2) & 3] = lookup(stage + 6);
+      if (stage < nstages) {
+        const bf16_t* pt = pbuf(bc);
+        const bf16_t* qt = qbuf(bc);
+        multiply_stage<MT, NTW>(
+            acc, [&](int s, int mt) { return kfrag_read_s(pt, poff[mt], s); },
+            [&](int s, int j) { return kfrag_read_s(qt, qoff[j], s); });
       }
-      multiply(p0, q0);
-      if (more1) {
-        const bool more2 = lo + k0 + 2 * kKS < hi;
-        wait_loads_and_sync();
-        if (more2) {
-          fill(p0, q0);
-          if (lo + k0 + 3 * kKS < hi) sources(k0 + 3 * kKS);
-        }
-        multiply(p1, q1);
-      }
+    };
+    for (int i = 0; i < nstages; i += 4) {
+      step(integral_constant<int, 0>{}, integral_constant<int, 3>{}, i);
+      step(integral_constant<int, 1>{}, integral_constant<int, 0>{}, i + 1);
+      step(integral_constant<int, 2>{}, integral_constant<int, 1>{}, i + 2);
+      step(integral_constant<int, 3>{}, integral_constant<int, 2>{}, i + 3);
     }
+    __builtin_amdgcn_s_waitcnt(0);       // the repeated requests of the last steps land before the workgroup ends
   }
   // accumulators transposed: lane = row n0 + wm MT 32 + 32 mt + lane % 32, register 4 q + r = column
   // m0 + (wn NTW + j) 32 + 8 q + 4 (lane / 32) + r
