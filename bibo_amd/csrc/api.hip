@@ -562,11 +562,17 @@ int bibo_moe_backward(const void* x, const void* d_out, const void* w_router, co
   int32_t* perm_slot = reinterpret_cast<int32_t*>(base + ws.perm_slot);
   int32_t* perm_token = reinterpret_cast<int32_t*>(base + ws.perm_token);
   // the routing of the forward pass again: same kernel, same inputs, hence the same selection and weights
+  // (the router kernel leaves per-workgroup histograms of its selections for the permutation, as in the forward pass)
+  int32_t* hist = reinterpret_cast<int32_t*>(base + ws.hist);
+  int hist_tokens = 0;
+  const bool want_hist = T > 0 && permute_takes_router_hist(T, k);
   if (T > 0 && (rc = hip_rc(launch_router(x, w_router, bias, T, H, E, k, sh->dtype, norm_mode, logits, idx, w, nullptr,
-                                          nullptr, nullptr, s))) != BIBO_OK)
+                                          want_hist ? hist : nullptr, &hist_tokens, s))) != BIBO_OK)
     return rc;
-  if ((rc = hip_rc(launch_permute(idx, T, E, k, counts, offsets, perm_slot, perm_token, base + ws.hist, s))) != BIBO_OK)
-    return rc;
+  rc = hip_rc((want_hist && hist_tokens > 0)
+                  ? launch_permute_from_hist(idx, T, E, k, hist, hist_tokens, counts, offsets, perm_slot, perm_token, s)
+                  : launch_permute(idx, T, E, k, counts, offsets, perm_slot, perm_token, hist, s));
+  if (rc != BIBO_OK) return rc;
   BackwardBuffers b;
   b.gu = base + ws.gu; b.dhp = base + ws.dhp; b.dgu = base + ws.dgu;
   b.hidden = base + ws.hidden; b.dxs = base + ws.dxs; b.zrow = base + ws.zrow;

@@ -181,7 +181,11 @@ __global__ __launch_bounds__(256) void act_bwd_kernel(const bf16_t* __restrict__
                                                       const int32_t* __restrict__ offsets,
                                                       const int32_t* __restrict__ perm_slot, int S, int E, int I, int act,
                                                       bf16_t* __restrict__ dgu, bf16_t* __restrict__ hidden,
-                                                      float* __restrict__ dw_slot, float* __restrict__ dtheta_row) {
+                                                      float* __restrict__ dw_slot, float* __restrict__ dtheta_row,
+                                                      uint32_t* __restrict__ zero_words, int n_zero_words) {
+  // (the first workgroup also clears the row of zeros the weight-gradient kernels read past an expert's last row)
+  if (blockIdx.x == 0)
+    for (int i = threadIdx.x; i < n_zero_words; i += 256) zero_words[i] = 0u;
   const int lane = threadIdx.x & 63;
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= S || row >= offsets[E]) return;                   // E = GLU experts: rows behind theirs have no activation
@@ -434,7 +438,7 @@ int backward_dwr_split() { return kDwrSplit; }
 size_t backward_zero_row_bytes(int H, int I) { return (size_t)(H > 2 * I ? H : 2 * I) * sizeof(bf16_t); }
 
 // The launches after routing and permutation.  Buffers (bf16 unless noted): gu [S,2I], dhp [S,I], dgu [S,2I],
-// hidden [S,I], dxs [S,H], zrow [max(H, 2I)] (zeroed here), dw_slot [S] f32, dl [S] f32, dtheta_row [S] f32,
+// hidden [S,I], dxs [S,H], zrow [max(H, 2I)] (cleared by act_bwd_kernel), dw_slot [S] f32, dl [S] f32, dtheta_row [S] f32,
 // dwr_part [E, backward_dwr_split(), H] f32.
 hipError_t launch_backward(const void* x, const void* d_out, const void* w_router, const void* wgu, const void* wd,
                            const float* theta, const float* logits, const int32_t* idx, const float* w,
@@ -463,7 +467,6 @@ hipError_t launch_backward(const void* x, const void* d_out, const void* w_route
     zero_bytes(d_wd, (size_t)E * H * I * sizeof(bf16_t), s);
     return hipGetLastError();
   }
-  zero_bytes(zrow, backward_zero_row_bytes(H, I), s);
   // pre-activations again (moe.py:84): x W_gate_up^T, both contiguous along H
   err = launch_ggemm<true, false>(xp, perm_token, wgup, offsets, nullptr, S, H, 2 * I, E, gu, s);
   if (err != hipSuccess) return err;
@@ -471,7 +474,8 @@ hipError_t launch_backward(const void* x, const void* d_out, const void* w_route
   err = launch_dgrad<true, false>(dop, perm_token, wdp, offsets, nullptr, S, H, I, E, dhp, s);
   if (err != hipSuccess) return err;
   hipLaunchKernelGGL(act_bwd_kernel, dim3((S + 3) / 4), dim3(256), 0, s, gu, dhp, w, theta, offsets, perm_slot, S, E, I, act,
-                     dgu, hidden, b.dw_slot, b.dtheta_row);
+                     dgu, hidden, b.dw_slot, b.dtheta_row, reinterpret_cast<uint32_t*>(zrow),
+                     (int)(backward_zero_row_bytes(H, I) / 4));
   hipLaunchKernelGGL(dtheta_reduce_kernel, dim3(E), dim3(256), 0, s, b.dtheta_row, offsets, d_theta);
   // dx of every slot, in slot order: [dg, du] W_gate_up, contracts over the 2I rows of w_gate_up [E, 2I, H]
   err = launch_dgrad<false, true>(dgu, nullptr, wgup, offsets, perm_slot, S, 2 * I, H, E, dxs, s);
