@@ -15,9 +15,9 @@
 // Order of the memory requests.  A CU serves its vector loads first in, first out, and its share of the
 // HBM rate is about 23 GB/s, so a small load issued behind 64 KB of weight requests waits about 3 us for
 // them (and behind 192 KB about 8 us).  Every small load the multiplication depends on is therefore issued
-// AHEAD of the weights it would otherwise queue behind: the routing indices before the first weight
-// chunk, the operand rows before the second, and only as much weight data is requested in between as the
-// dependent work (finding the rows) takes to complete.
+// AHEAD of the weights it would otherwise queue behind: the routing indices before any weights, the operand
+// rows before the second half of the first chunk and the second chunk, and only as much weight data is
+// requested in between (kFirstLines lines per lane) as the dependent work (finding the rows) takes to complete.
 //
 //   gateup_stream_kernel : raw gate/up pre-activations gu[slot, 0..2I) bf16        (src/modeling/ffn/moe.py:84)
 //   down_stream_kernel   : streams w_down and writes routing-weighted rows in slot order (moe.py:92-93);
@@ -87,14 +87,20 @@ __device__ __forceinline__ int scan_finish(const ScanRegs& r, int S, int e, unsi
 struct WChunk {
   bf16x8 w0[kChunk], w1[kChunk];
 };
+// Lines of the first chunk a wave requests before its rows are known; the other lines follow the row requests.  All
+// four up front put 128 KB of weight requests per CU ahead of every workgroup's row loads, which then wait for them;
+// with two, the rows are back about 1.5 us earlier and the weights still keep HBM busy from the first microsecond
+// (one line was as slow as four: too little in flight while the rows are found).
+constexpr int kFirstLines = 2;
 
 // this lane's 32 bytes of lines l .. l+kChunk-1 of its weight row.  kWhole: the row is a whole number of
 // chunks, and a chunk that starts past its end is skipped as a whole; otherwise line by line.
-template <bool kWhole>
+// (U0, U1: only lines l + U0 .. l + U1 - 1 of the chunk)
+template <bool kWhole, int U0 = 0, int U1 = kChunk>
 __device__ __forceinline__ void load_chunk(WChunk& c, const bf16_t* __restrict__ wp, int l, int nlines) {
   if (kWhole && l >= nlines) return;
 #pragma unroll
-  for (int u = 0; u < kChunk; ++u)
+  for (int u = U0; u < U1; ++u)
     if (kWhole || l + u < nlines) {
       c.w0[u] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(wp + (l + u) * kLine));
       c.w1[u] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(wp + (l + u) * kLine + 8));
@@ -145,21 +151,25 @@ typedef __attribute__((address_space(3))) void stream_lds_void;
 typedef const __attribute__((address_space(1))) void stream_gbl_void;
 
 // wait until at most the kChunk lines of weights requested last are still on their way (loads complete in order)
+// (EXTRA: further loads requested behind the rows, the rest of the first chunk; s_waitcnt vmcnt(8 + EXTRA) in the gfx9
+// encoding: vmcnt in bits 3:0 and 15:14, expcnt and lgkmcnt left at "no wait")
+template <int EXTRA>
 __device__ __forceinline__ void wait_all_but_chunk(bool chunk_requested) {
-  if (chunk_requested) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+  constexpr int kN = 8 + EXTRA;
+  if (chunk_requested) __builtin_amdgcn_s_waitcnt((kN & 0xF) | ((kN >> 4) << 14) | (0x7 << 4) | (0xF << 8));
   else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   static_assert(2 * kChunk == 8, "the wait above counts the two loads per line of one chunk");
 }
 
 // Operand rows of slots rows_s[r0 .. r0+nrow), row (slot / div) of `src` (row length K), into xs[t][0..K) (row
 // stride K + 8), by LDS-DMA: one wave instruction moves 1 KB of one row (lane L's 16 bytes land at base + 16 L),
-// no registers hold the data.  The rows are requested, then chunk `b` of the weights (lines kChunk..), and the
-// wave then waits for its rows only.  Rows past nrow keep whatever LDS held: they only feed accumulator
+// no registers hold the data.  The rows are requested, then (a_rest: the first pass) the lines of chunk `a` that were
+// held back, then chunk `b` of the weights (lines kChunk..), and the wave then waits for its rows only.  Rows past nrow keep whatever LDS held: they only feed accumulator
 // columns nobody stores.  The caller's barrier makes the rows visible to the other waves.
-template <bool kWhole>
+template <bool kWhole, int kFirst>
 __device__ __forceinline__ void stage_rows(const bf16_t* __restrict__ src, const unsigned short* rows_s, int r0,
                                            int nrow, int div, int K, bf16_t* xs, WChunk& b,
-                                           const bf16_t* __restrict__ wp, int nlines, bool load_b) {
+                                           const bf16_t* __restrict__ wp, int nlines, bool load_b, WChunk& a, bool a_rest) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int gran = K / 8;                                      // 16-byte granules per row
@@ -173,8 +183,15 @@ __device__ __forceinline__ void stage_rows(const bf16_t* __restrict__ src, const
       __builtin_amdgcn_global_load_lds((stream_gbl_void*)(src + (size_t)row * K + c * 8),
                                        (stream_lds_void*)(xs + t * (K + 8) + sg * 512), 16, 0, 0);
   }
+  if (a_rest) {
+    load_chunk<kWhole, kFirst, kChunk>(a, wp, 0, nlines);
+    if (load_b) load_chunk<kWhole>(b, wp, kChunk, nlines);
+    if (kWhole) wait_all_but_chunk<2 * (kChunk - kFirst)>(load_b && nlines > kChunk);
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    return;
+  }
   if (load_b) load_chunk<kWhole>(b, wp, kChunk, nlines);
-  wait_all_but_chunk(load_b && kWhole && nlines > kChunk);
+  wait_all_but_chunk<0>(load_b && kWhole && nlines > kChunk);
 }
 
 // grid = (2I / 64, E).  gu[slot, c] = x[slot / k] . w_gate_up[e, c, :].  kWhole: H is a whole number of chunks.
@@ -196,7 +213,7 @@ void gateup_stream_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict
   ScanRegs sr;
   scan_issue(sr, idx, S);
   WChunk ca, cb;
-  load_chunk<kWhole>(ca, wp, 0, nlines);                       // keeps HBM busy while the rows are found
+  load_chunk<kWhole, 0, kFirstLines>(ca, wp, 0, nlines);             // keeps HBM busy while the rows are found
   const int n = scan_finish(sr, S, e, rows_s, cnt_s);
   for (int r0 = 0; r0 < n; r0 += kTok) {
     const int nrow = min(kTok, n - r0);
@@ -205,7 +222,7 @@ void gateup_stream_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict
       __syncthreads();                                         // the pass before is done with xs
       if (reload) load_chunk<kWhole>(ca, wp, 0, nlines);       // a further pass starts the weight rows again
     }
-    stage_rows<kWhole>(x, rows_s, r0, nrow, k, H, xs, cb, wp, nlines, reload);
+    stage_rows<kWhole, kFirstLines>(x, rows_s, r0, nrow, k, H, xs, cb, wp, nlines, reload, ca, r0 == 0 && kFirstLines < kChunk);
     __syncthreads();
     const floatx4 acc = stream_rows<kWhole>(wp, xs, H, lane, ca, cb);
     // accumulator: lane holds row lane%16 of the pass, weight rows 4*(lane/16) + i
@@ -244,12 +261,14 @@ __global__ __launch_bounds__(256) void activate_rows_kernel(const bf16_t* __rest
 // from the bf16 pre-activations, r = sqrt(mean(g^2) + eps), hidden = r^p SiLU(g/r) up, p = sigmoid(theta)
 // (moe.py:87-92), into hs[t][0..I) (row stride I + 8).  tpr = 32 or 64 threads share a row, so the workgroup
 // covers 8 (or 4) rows per round; a thread owns granules part, part + tpr of the gate and of the up half.  The
-// first round's loads are requested ahead of chunk `b` of the weights, like the rows in stage_rows.
+// first round's loads are requested ahead of the held-back lines of chunk `a` and of chunk `b`, like the rows in
+// stage_rows.
 // I <= kFusedActMaxI.
-template <bool kWhole>
+template <bool kWhole, int kFirst>
 __device__ __forceinline__ void stage_activated(const bf16_t* __restrict__ gu, float p, int act,
                                                 const unsigned short* rows_s, int r0, int nrow, int I, bf16_t* hs,
-                                                WChunk& b, const bf16_t* __restrict__ wp, int nlines, bool load_b) {
+                                                WChunk& b, const bf16_t* __restrict__ wp, int nlines, bool load_b,
+                                                WChunk& a, bool a_rest) {
   constexpr int kPer = kFusedActMaxI / 8 / 32;                 // granules per thread and half at 32 threads per row
   const int tid = threadIdx.x;
   const int tpr = nrow <= 4 ? 64 : 32;
@@ -268,6 +287,7 @@ __device__ __forceinline__ void stage_activated(const bf16_t* __restrict__ gu, f
         u[j] = *reinterpret_cast<const bf16x8*>(grow + I + c * 8);
       }
     }
+    if (rb == 0 && a_rest) load_chunk<kWhole, kFirst, kChunk>(a, wp, 0, nlines);
     if (rb == 0 && load_b) load_chunk<kWhole>(b, wp, kChunk, nlines);
     float ss = 0.f;
 #pragma unroll
@@ -321,7 +341,7 @@ void down_stream_kernel(const bf16_t* __restrict__ rows_in, const bf16_t* __rest
   scan_issue(sr, idx, S);
   const float p_e = kFusedAct ? radial_exponent(theta, e, act) : 0.f;                       // moe.py:89
   WChunk ca, cb;
-  load_chunk<kWhole>(ca, wp, 0, nlines);
+  load_chunk<kWhole, 0, kFirstLines>(ca, wp, 0, nlines);
   const int n = scan_finish(sr, S, e, rows_s, cnt_s);
   for (int r0 = 0; r0 < n; r0 += kTok) {
     const int nrow = min(kTok, n - r0);
@@ -330,8 +350,9 @@ void down_stream_kernel(const bf16_t* __restrict__ rows_in, const bf16_t* __rest
       __syncthreads();
       if (reload) load_chunk<kWhole>(ca, wp, 0, nlines);
     }
-    if (kFusedAct) stage_activated<kWhole>(rows_in, p_e, act, rows_s, r0, nrow, I, hs, cb, wp, nlines, reload);
-    else stage_rows<kWhole>(rows_in, rows_s, r0, nrow, 1, I, hs, cb, wp, nlines, reload);
+    const bool rest = r0 == 0 && kFirstLines < kChunk;
+    if (kFusedAct) stage_activated<kWhole, kFirstLines>(rows_in, p_e, act, rows_s, r0, nrow, I, hs, cb, wp, nlines, reload, ca, rest);
+    else stage_rows<kWhole, kFirstLines>(rows_in, rows_s, r0, nrow, 1, I, hs, cb, wp, nlines, reload, ca, rest);
     __syncthreads();
     // the fused activation is only used up to I = kFusedActMaxI = two chunks
     const floatx4 acc = stream_rows<kWhole, kFusedAct>(wp, hs, I, lane, ca, cb);
