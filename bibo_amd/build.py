@@ -14,7 +14,7 @@ CSRC = HERE / "csrc"
 BUILD = HERE / "csrc" / "build"
 LIB = HERE / "libbibo_moe.so"
 
-SOURCES = ["router.hip", "permute.hip", "experts_generic.hip", "experts_mfma.hip", "experts_fused.hip", "experts_stream.hip", "ffn.hip", "backward.hip", "api.hip"]
+SOURCES = ["router.hip", "permute.hip", "experts_generic.hip", "experts_mfma.hip", "experts_fused.hip", "experts_stream.hip", "ffn.hip", "backward.hip", "backward_generic.hip", "api.hip"]
 
 # -packed-fp32-ops is switched off on purpose: hipcc -O3 otherwise forms v_pk_*_f32 from scalar float code.
 HIPCC_FLAGS = [

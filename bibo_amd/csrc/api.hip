@@ -286,13 +286,44 @@ BackwardWorkspace carve_backward(int T, int H, int E, int k, int I) {
   return ws;
 }
 
+// the generic family keeps its intermediates in fp32: [dg, du], w h and the per-slot dx rows
+struct GenericBackwardWorkspace {
+  size_t hist, idx, w, logits, counts, offsets, perm_slot, perm_token, dw_slot, dl, dtheta_row, dgu, hw, dxs, total;
+};
+
+GenericBackwardWorkspace carve_backward_generic(int T, int H, int E, int k, int I) {
+  const size_t S = (size_t)T * k;
+  GenericBackwardWorkspace ws;
+  size_t o = 0;
+  ws.hist = o;       o += align_up(permute_workspace_bytes(T) > router_hist_bytes(T) ? permute_workspace_bytes(T)
+                                                                                    : router_hist_bytes(T));
+  ws.idx = o;        o += align_up(S * sizeof(int32_t));
+  ws.w = o;          o += align_up(S * sizeof(float));
+  ws.logits = o;     o += align_up((size_t)T * E * sizeof(float));
+  ws.counts = o;     o += align_up(kMaxE * sizeof(int32_t));
+  ws.offsets = o;    o += align_up((kMaxE + 1) * sizeof(int32_t));
+  ws.perm_slot = o;  o += align_up(S * sizeof(int32_t));
+  ws.perm_token = o; o += align_up(S * sizeof(int32_t));
+  ws.dw_slot = o;    o += align_up(S * sizeof(float));
+  ws.dl = o;         o += align_up(S * sizeof(float));
+  ws.dtheta_row = o; o += align_up(S * sizeof(float));
+  ws.dgu = o;        o += align_up(S * 2 * I * sizeof(float));
+  ws.hw = o;         o += align_up(S * I * sizeof(float));
+  ws.dxs = o;        o += align_up(S * H * sizeof(float));
+  ws.total = o;
+  return ws;
+}
+
+// which backward family a shape runs: the MFMA kernels (bf16, H and I multiples of 128, I <= 512) or the generic ones
+inline bool backward_fast(const bibo_moe_shape* sh) { return backward_supported(sh->H, sh->I, sh->k, sh->dtype); }
+
 int backward_check(const bibo_moe_shape* sh, int norm_mode) {
   if (sh == nullptr) return BIBO_ERR_NULL_POINTER;
   const int rc = check_dims(sh->T, sh->H, sh->E, sh->k, sh->I, sh->dtype, sh->n_pos, sh->n_neg);
   if (rc != BIBO_OK) return rc;
   if (norm_mode < BIBO_NORM_NONE || norm_mode > BIBO_NORM_SOFTMAX || !act_ok(sh->act)) return BIBO_ERR_UNSUPPORTED;
-  // bf16, dimensions the MFMA tiles divide
-  if (!backward_supported(sh->H, sh->I, sh->k, sh->dtype)) return BIBO_ERR_UNSUPPORTED;
+  // the MFMA family (bf16, dimensions its tiles divide) or the generic one (a row of 2H + 5I floats within 64 KB)
+  if (!backward_fast(sh) && !backward_generic_supported(sh->H, sh->I, sh->k)) return BIBO_ERR_UNSUPPORTED;
   return BIBO_OK;
 }
 
@@ -531,7 +562,8 @@ int bibo_moe_backward_workspace_bytes(const bibo_moe_shape* sh, size_t* bytes) {
   if (bytes == nullptr) return BIBO_ERR_NULL_POINTER;
   const int rc = backward_check(sh, BIBO_NORM_SUM);
   if (rc != BIBO_OK) return rc;
-  *bytes = carve_backward(sh->T, sh->H, sh->E, sh->k, sh->I).total;
+  *bytes = backward_fast(sh) ? carve_backward(sh->T, sh->H, sh->E, sh->k, sh->I).total
+                             : carve_backward_generic(sh->T, sh->H, sh->E, sh->k, sh->I).total;
   return BIBO_OK;
 }
 
@@ -547,6 +579,32 @@ int bibo_moe_backward(const void* x, const void* d_out, const void* w_router, co
   if (!d_w_router || !d_w_gate_up || !d_w_down || !d_theta) return BIBO_ERR_NULL_POINTER;
   if (T > 0 && (!x || !d_out || !w_router || !bias || !w_gate_up || !w_down || !d_x)) return BIBO_ERR_NULL_POINTER;
   if (T > 0 && !theta && sh->act != BIBO_ACT_SILU) return BIBO_ERR_NULL_POINTER;
+  if (!backward_fast(sh)) {
+    const GenericBackwardWorkspace gw = carve_backward_generic(T, H, E, k, I);
+    if (workspace_bytes < gw.total) return BIBO_ERR_WORKSPACE_TOO_SMALL;
+    char* gb = static_cast<char*>(workspace);
+    hipStream_t gs = static_cast<hipStream_t>(stream);
+    int32_t* g_idx = reinterpret_cast<int32_t*>(gb + gw.idx);
+    float* g_w = reinterpret_cast<float*>(gb + gw.w);
+    float* g_logits = reinterpret_cast<float*>(gb + gw.logits);
+    int32_t* g_offsets = reinterpret_cast<int32_t*>(gb + gw.offsets);
+    int32_t* g_slot = reinterpret_cast<int32_t*>(gb + gw.perm_slot);
+    int32_t* g_token = reinterpret_cast<int32_t*>(gb + gw.perm_token);
+    if (T > 0 && (rc = hip_rc(launch_router(x, w_router, bias, T, H, E, k, sh->dtype, norm_mode, g_logits, g_idx, g_w, nullptr,
+                                            nullptr, nullptr, gs))) != BIBO_OK)
+      return rc;
+    if ((rc = hip_rc(launch_permute(g_idx, T, E, k, reinterpret_cast<int32_t*>(gb + gw.counts), g_offsets, g_slot, g_token,
+                                    gb + gw.hist, gs))) != BIBO_OK)
+      return rc;
+    GenericBackwardBuffers g;
+    g.dgu = reinterpret_cast<float*>(gb + gw.dgu); g.hw = reinterpret_cast<float*>(gb + gw.hw);
+    g.dxs = reinterpret_cast<float*>(gb + gw.dxs);
+    g.dw_slot = d_w_out ? d_w_out : reinterpret_cast<float*>(gb + gw.dw_slot);
+    g.dl = reinterpret_cast<float*>(gb + gw.dl); g.dtheta_row = reinterpret_cast<float*>(gb + gw.dtheta_row);
+    return hip_rc(launch_backward_generic(x, d_out, w_router, w_gate_up, w_down, theta, g_logits, g_idx, g_w, g_offsets, g_slot,
+                                          g_token, T, H, E - sh->n_pos - sh->n_neg, sh->n_pos, sh->n_neg, k, I, sh->dtype,
+                                          norm_mode, sh->act, g, d_x, d_w_router, d_w_gate_up, d_w_down, d_theta, gs));
+  }
   if (!aligned16(x) || !aligned16(d_out) || !aligned16(w_router) || !aligned16(w_gate_up) || !aligned16(w_down) ||
       !aligned16(d_x) || !aligned16(d_w_gate_up) || !aligned16(d_w_down))
     return BIBO_ERR_MISALIGNED;
@@ -597,6 +655,26 @@ int bibo_moe_experts_backward(const void* x, const void* d_out, const int32_t* i
   if (!d_w_gate_up || !d_w_down || !d_theta) return BIBO_ERR_NULL_POINTER;
   if (T > 0 && (!x || !d_out || !idx || !w || !w_gate_up || !w_down || !d_x || !d_w)) return BIBO_ERR_NULL_POINTER;
   if (T > 0 && !theta && sh->act != BIBO_ACT_SILU) return BIBO_ERR_NULL_POINTER;
+  if (!backward_fast(sh)) {
+    const GenericBackwardWorkspace gw = carve_backward_generic(T, H, E, k, I);
+    if (workspace_bytes < gw.total) return BIBO_ERR_WORKSPACE_TOO_SMALL;
+    char* gb = static_cast<char*>(workspace);
+    hipStream_t gs = static_cast<hipStream_t>(stream);
+    int32_t* g_offsets = reinterpret_cast<int32_t*>(gb + gw.offsets);
+    int32_t* g_slot = reinterpret_cast<int32_t*>(gb + gw.perm_slot);
+    int32_t* g_token = reinterpret_cast<int32_t*>(gb + gw.perm_token);
+    if ((rc = hip_rc(launch_permute(idx, T, E, k, reinterpret_cast<int32_t*>(gb + gw.counts), g_offsets, g_slot, g_token,
+                                    gb + gw.hist, gs))) != BIBO_OK)
+      return rc;
+    GenericBackwardBuffers g;
+    g.dgu = reinterpret_cast<float*>(gb + gw.dgu); g.hw = reinterpret_cast<float*>(gb + gw.hw);
+    g.dxs = reinterpret_cast<float*>(gb + gw.dxs);
+    g.dw_slot = d_w;
+    g.dl = reinterpret_cast<float*>(gb + gw.dl); g.dtheta_row = reinterpret_cast<float*>(gb + gw.dtheta_row);
+    return hip_rc(launch_backward_generic(x, d_out, nullptr, w_gate_up, w_down, theta, nullptr, idx, w, g_offsets, g_slot, g_token,
+                                          T, H, E - sh->n_pos - sh->n_neg, sh->n_pos, sh->n_neg, k, I, sh->dtype, BIBO_NORM_SUM,
+                                          sh->act, g, d_x, nullptr, d_w_gate_up, d_w_down, d_theta, gs));
+  }
   if (!aligned16(x) || !aligned16(d_out) || !aligned16(w_gate_up) || !aligned16(w_down) || !aligned16(d_x) ||
       !aligned16(d_w_gate_up) || !aligned16(d_w_down))
     return BIBO_ERR_MISALIGNED;

@@ -224,6 +224,18 @@ struct BackwardBuffers {
 bool backward_supported(int H, int I, int k, int dtype);
 size_t backward_zero_row_bytes(int H, int I);
 int backward_dwr_split();
+// the generic family (backward_generic.hip): any sizes, bf16 or fp32 operands; every buffer fp32
+struct GenericBackwardBuffers {
+  float *dgu, *hw, *dxs;                                            // [S,2I], [S,I], [S,H]
+  float *dw_slot, *dl, *dtheta_row;                                 // [T*k] each
+};
+bool backward_generic_supported(int H, int I, int k);
+hipError_t launch_backward_generic(const void* x, const void* d_out, const void* w_router, const void* wgu, const void* wd,
+                                   const float* theta, const float* logits, const int32_t* idx, const float* w,
+                                   const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token, int T, int H,
+                                   int E, int n_pos, int n_neg, int k, int I, int dtype, int norm_mode, int act,
+                                   const GenericBackwardBuffers& b, void* dx, void* d_w_router, void* d_wgu, void* d_wd,
+                                   float* d_theta, hipStream_t s);
 hipError_t launch_backward(const void* x, const void* d_out, const void* w_router, const void* wgu, const void* wd,
                            const float* theta, const float* logits, const int32_t* idx, const float* w,
                            const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token, int T, int H, int E,

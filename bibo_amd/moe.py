@@ -3,9 +3,10 @@
 Class names, constructor argument, attribute names, parameter shapes and state_dict keys follow
 src/modeling/ffn/router.py and src/modeling/ffn/moe.py of the reference, so a reference checkpoint
 loads with strict=True and code that pokes at `layer.gate.bias` or `layer.experts.radial_theta`
-keeps working.  The modules are differentiable for bf16 compute: `BiBoMoELayer.forward` is one autograd node
-(backward = bibo_moe_backward); with hooks present, or called on their own, `BiBoFusedExperts` is one node (backward =
-bibo_moe_experts_backward) and `BiBoMoERouter` returns the kernel's selection with differentiable weights."""
+keeps working.  The modules are differentiable: `BiBoMoELayer.forward` is one autograd node (backward =
+bibo_moe_backward); with hooks present, or called on their own, `BiBoFusedExperts` is one node (backward =
+bibo_moe_experts_backward) and `BiBoMoERouter` returns the kernel's selection with differentiable weights.  bf16
+compute on sizes that are multiples of 128 trains on the MFMA kernels, fp32 compute and other sizes on generic ones."""
 from __future__ import annotations
 
 import torch
@@ -30,12 +31,12 @@ class _MoELayerFn(torch.autograd.Function):
     """The whole layer as one autograd node: forward = bibo_moe_forward, backward = bibo_moe_backward, which recomputes
     the routing and the activations from the saved input, so nothing but the input rows is kept.  Gradients are what
     autograd gives the reference's eager layer with the selection held fixed (moe.py:157-183); the balancing bias
-    gets none (router.py:38).  The per-expert row counts come out as a second, non-differentiable result."""
+    gets none (router.py:38).  The per-expert row counts come out as a second, non-differentiable result.  `cd` is the
+    compute dtype: bf16 runs the MFMA backward where its tiles divide the sizes, anything else the generic kernels."""
 
     @staticmethod
     def forward(ctx, x, w_router, w_gate_up, w_down, theta, bias, k, norm, act, algo, want_counts, n_pos=0, n_neg=0,
-                casts=None):
-        cd = torch.bfloat16
+                casts=None, cd=torch.bfloat16):
         cast = lambda t, d: (t if t.dtype == d else t.to(d)).contiguous()
         xb = cast(x.detach(), cd)
         # `casts`: kernel-dtype copies of the three weight tensors the caller already holds (the layer's cast cache), so
@@ -60,9 +61,9 @@ class _MoELayerFn(torch.autograd.Function):
     def backward(ctx, d_out, _d_counts):
         xb, wr, gu, dn, th, b = ctx.saved_tensors
         k, norm, act, n_pos, n_neg = ctx.conf
-        d = d_out.to(torch.bfloat16).contiguous()
+        d = d_out.to(xb.dtype).contiguous()
         grads = ops.moe_backward(xb, d, wr, b, gu, dn, th, k, norm=norm, act=act, n_pos=n_pos, n_neg=n_neg)[:5]
-        return tuple(g.to(dt) for g, dt in zip(grads, ctx.in_dtypes)) + (None,) * 9
+        return tuple(g.to(dt) for g, dt in zip(grads, ctx.in_dtypes)) + (None,) * 10
 
 
 class _ExpertsFn(torch.autograd.Function):
@@ -70,8 +71,8 @@ class _ExpertsFn(torch.autograd.Function):
     = bibo_moe_experts_backward.  The gradient of the combine weights (moe.py:93) flows back to whoever made them."""
 
     @staticmethod
-    def forward(ctx, x, top_w, w_gate_up, w_down, theta, idx, act, algo, want_counts, n_pos=0, n_neg=0, casts=None):
-        cd = torch.bfloat16
+    def forward(ctx, x, top_w, w_gate_up, w_down, theta, idx, act, algo, want_counts, n_pos=0, n_neg=0, casts=None,
+                cd=torch.bfloat16):
         cast = lambda t, d: (t if t.dtype == d else t.to(d)).contiguous()
         xb = cast(x.detach(), cd)
         gu, dn = casts if casts is not None else (cast(w_gate_up.detach(), cd), cast(w_down.detach(), cd))
@@ -89,14 +90,22 @@ class _ExpertsFn(torch.autograd.Function):
     @staticmethod
     def backward(ctx, d_out, _d_counts):
         xb, w, gu, dn, th, idx = ctx.saved_tensors
-        grads = ops.experts_backward(xb, d_out.to(torch.bfloat16).contiguous(), idx, w, gu, dn, th, act=ctx.act,
+        grads = ops.experts_backward(xb, d_out.to(xb.dtype).contiguous(), idx, w, gu, dn, th, act=ctx.act,
                                      n_pos=ctx.specials[0], n_neg=ctx.specials[1])
-        return tuple(g.to(dt) for g, dt in zip(grads, ctx.in_dtypes)) + (None,) * 7
+        return tuple(g.to(dt) for g, dt in zip(grads, ctx.in_dtypes)) + (None,) * 8
 
 
-def _backward_covers(experts) -> bool:
-    return (experts.hidden_size % 128 == 0 and experts.intermediate_size % 128 == 0
-            and experts.intermediate_size <= 512)
+def _backward_covers(experts, cd) -> bool:
+    """Whether bibo_moe_backward takes this size in compute dtype cd, as the library itself answers: the MFMA kernels
+    for bf16 with hidden and expert sizes that are multiples of 128 (expert size up to 512), the generic kernels for
+    everything else that keeps a row's 2H + 5I floats within 64 KB of LDS."""
+    return ops.backward_supported(experts.hidden_size, experts.intermediate_size, experts.num_routed_experts, cd,
+                                  experts.num_pos, experts.num_neg)
+
+
+_NO_BACKWARD = ("no backward pass for this size: the MFMA kernels take bf16 with hidden and expert sizes that are multiples "
+                "of 128 and expert sizes up to 512, the generic ones rows of 2 * hidden_size + 5 * moe_intermediate_size "
+                "floats up to 64 KB")
 
 
 class _CastCache:
@@ -259,15 +268,12 @@ class BiBoFusedExperts(nn.Module):
     def forward(self, hidden_states: torch.Tensor, top_k_indices: torch.Tensor, top_k_weights: torch.Tensor,
                 _want_counts: bool = False):
         if _wants_grad(hidden_states, top_k_weights, self.gate_up_proj, self.down_proj, self.radial_theta):
-            if _compute_dtype(hidden_states) != torch.bfloat16:
-                raise RuntimeError("the backward pass runs in bf16: use bf16 activations or bf16 autocast, or call the "
-                                   "experts under torch.no_grad()")
-            if not _backward_covers(self):
-                raise NotImplementedError("the backward pass covers hidden and expert sizes that are multiples of 128 and "
-                                          "expert size <= 512")
+            cd = _compute_dtype(hidden_states)
+            if not _backward_covers(self, cd):
+                raise NotImplementedError(_NO_BACKWARD)
             out, counts = _ExpertsFn.apply(hidden_states, top_k_weights, self.gate_up_proj, self.down_proj, self.radial_theta,
                                            top_k_indices.detach().to(torch.int32).contiguous(), self.act, self.algo,
-                                           _want_counts, self.num_pos, self.num_neg, self._weights(torch.bfloat16)[:2])
+                                           _want_counts, self.num_pos, self.num_neg, self._weights(cd)[:2], cd)
             out = out if out.dtype == hidden_states.dtype else out.to(hidden_states.dtype)
             return (out, counts) if _want_counts else out
         cd = _compute_dtype(hidden_states)
@@ -428,22 +434,18 @@ class BiBoMoELayer(nn.Module):
         return out
 
     def _differentiable_forward(self, x: torch.Tensor, want_counts: bool):
-        """x [T,H] -> (out [T,H] bf16 with an autograd graph, counts|None).  bf16 compute only (bf16 activations, or
-        fp32 activations under bf16 autocast), H and I multiples of 128 and I <= 512, with or without +/-Identity
-        experts: what bibo_moe_backward covers."""
+        """x [T,H] -> (out [T,H] in the compute dtype with an autograd graph, counts|None).  bf16 compute (bf16
+        activations, or fp32 activations under bf16 autocast) with H and I multiples of 128 and I <= 512 runs the MFMA
+        backward; fp32 compute and every other size run the generic kernels."""
         e = self.experts
-        if _compute_dtype(x) != torch.bfloat16:
-            raise RuntimeError("the backward pass runs in bf16: use bf16 activations or bf16 autocast, or call the layer "
-                               "under torch.no_grad()")
-        if not _backward_covers(e):
-            raise NotImplementedError("the backward pass covers hidden and expert sizes that are multiples of 128 and "
-                                      "expert size <= 512")
-        cd = torch.bfloat16
+        cd = _compute_dtype(x)
+        if not _backward_covers(e, cd):
+            raise NotImplementedError(_NO_BACKWARD)
         gu, dn, _ = e._weights(cd)
         casts = (self.gate._cache.get("w", self.gate.gate_proj.weight, cd), gu, dn)
         out, counts = _MoELayerFn.apply(x, self.gate.gate_proj.weight, e.gate_up_proj, e.down_proj, e.radial_theta,
                                         self.gate.bias, self.num_experts_per_tok, self.gate.norm_topk_prob, e.act, e.algo,
-                                        want_counts, e.num_pos, e.num_neg, casts)
+                                        want_counts, e.num_pos, e.num_neg, casts, cd)
         return out, (counts if want_counts else None)
 
     @_no_compile

@@ -47,6 +47,14 @@ def select_algo(T, H, E, k, I, dtype_code=L.DTYPE_BF16, algo="auto", n_pos=0, n_
     return {v: n for n, v in _ALGO.items()}[out.value]
 
 
+def backward_supported(H, I, E, dtype, n_pos=0, n_neg=0) -> bool:
+    """Whether bibo_moe_backward takes hidden size H and expert size I in `dtype` (torch.bfloat16 or torch.float32): the
+    answer bibo_moe_backward_workspace_bytes gives for a single token."""
+    sh = L.Shape(1, H, E, 1, I, L.DTYPE_BF16 if dtype == torch.bfloat16 else L.DTYPE_F32, n_pos, n_neg)
+    n = ctypes.c_size_t(0)
+    return L.lib().bibo_moe_backward_workspace_bytes(ctypes.byref(sh), ctypes.byref(n)) == 0
+
+
 def _dtype_code(t: torch.Tensor) -> int:
     if t.dtype == torch.bfloat16:
         return L.DTYPE_BF16

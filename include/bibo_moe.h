@@ -275,10 +275,13 @@ int bibo_moe_ffn_forward(const void* h, const float* norm_weight, float eps, con
  *   d_w_out fp32 [T,k] or NULL: gradient with respect to the combine weights (router.py:47), for inspection.
  * A slot routed to a +/-Identity expert (moe.py:95-99) sends +/- w d_out[t] to d_x and +/- <d_out[t], x[t]> to its
  * combine weight, and through that to the router.
- * bf16 only, H and I multiples of 128, I <= 512 (BIBO_ERR_UNSUPPORTED otherwise); the
- * intermediate activations are recomputed, nothing has to be kept from the forward call.  All gradients are
- * overwritten, not accumulated.  Workspace: bibo_moe_backward_workspace_bytes (about 14 bytes per routed slot and
- * column plus one transposed copy of the expert weights).
+ * Two kernel families: bf16 with H and I multiples of 128 and I <= 512 runs grouped MFMA GEMMs (bf16 operands, fp32
+ * accumulation, results rounded once); every other size and fp32 run generic kernels that compute in fp32 throughout
+ * (fp32 operands give fp32-exact gradients, the regime of the reference's own gradient tests) and keep
+ * 2H + 5I floats of a row in LDS: BIBO_ERR_UNSUPPORTED when neither applies, i.e. off the MFMA sizes with
+ * (2H + 5I) * 4 > 65536.  The intermediate activations are recomputed, nothing has to be kept from the forward
+ * call.  All gradients are overwritten, not accumulated.  Workspace: bibo_moe_backward_workspace_bytes (MFMA family:
+ * about 12 I + 2 H bytes per routed slot; generic family: 12 I + 4 H).
  */
 int bibo_moe_backward_workspace_bytes(const bibo_moe_shape* shape, size_t* bytes);
 int bibo_moe_backward(const void* x, const void* d_out, const void* w_router, const float* bias, const void* w_gate_up,

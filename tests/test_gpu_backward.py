@@ -144,16 +144,96 @@ def test_backward_is_linear_in_the_upstream_gradient():
     assert all(bool(torch.isfinite(t.float()).all()) for t in a[:5])
 
 
-def test_backward_rejects_what_it_does_not_cover():
+def test_backward_families_and_what_neither_covers():
+    """bf16 with H and I multiples of 128 runs the MFMA backward; other sizes and fp32 run the generic kernels, whose
+    workspace holds fp32 intermediates; a row of more than 64 KB (2H + 5I floats) is refused."""
     from bibo_amd import _lib as L
     import ctypes
-    sh = L.Shape(64, 200, 8, 2, 128, L.DTYPE_BF16)                  # H no multiple of 128
     n = ctypes.c_size_t(0)
-    assert L.lib().bibo_moe_backward_workspace_bytes(ctypes.byref(sh), ctypes.byref(n)) == -6
-    sh = L.Shape(64, 256, 8, 2, 128, L.DTYPE_BF16, 1, 1)            # +/-Identity experts are covered
-    assert L.lib().bibo_moe_backward_workspace_bytes(ctypes.byref(sh), ctypes.byref(n)) == 0 and n.value > 0
-    sh = L.Shape(64, 256, 8, 2, 128, L.DTYPE_F32)
-    assert L.lib().bibo_moe_backward_workspace_bytes(ctypes.byref(sh), ctypes.byref(n)) == -6
+    size = lambda *a: (L.lib().bibo_moe_backward_workspace_bytes(ctypes.byref(L.Shape(*a)), ctypes.byref(n)), n.value)
+    rc_fast, fast = size(64, 256, 8, 2, 128, L.DTYPE_BF16)
+    rc_odd, odd = size(64, 200, 8, 2, 128, L.DTYPE_BF16)           # H no multiple of 128: generic
+    rc_f32, f32 = size(64, 256, 8, 2, 128, L.DTYPE_F32)            # fp32: generic
+    assert (rc_fast, rc_odd, rc_f32) == (0, 0, 0) and min(fast, odd, f32) > 0
+    assert size(64, 256, 8, 2, 128, L.DTYPE_BF16, 1, 1)[0] == 0    # +/-Identity experts are covered
+    assert size(64, 4096, 8, 2, 2048, L.DTYPE_BF16)[0] == -6       # MFMA family: I > 512; generic: 72 KB per row
+
+
+def _run_generic(T, H, E, k, I, dtype, norm="sum", act="radial", seed=0, n_pos=0, n_neg=0):
+    """bibo_moe_backward on a shape or dtype the generic kernels take, against the fp64 autograd oracle."""
+    Et = E + n_pos + n_neg
+    p = O.make_inputs(T=T, H=H, E=E, k=k, I=I, theta="normal", seed=seed)
+    g = torch.Generator().manual_seed(seed + 50)
+    p["w_router"] = (torch.randn(Et, H, generator=g) * 0.05).bfloat16()
+    p["bias"] = torch.rand(Et, generator=g) * 0.02 - 0.01
+    if n_pos + n_neg:
+        p["bias"][E:] += 0.05
+    d_out = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    dev = lambda t: (t.to(dtype) if t.dtype == torch.bfloat16 else t).to(DEV)     # bf16-representable values either way
+    args = [dev(p[n]) for n in ("w_router", "bias", "w_gate_up", "w_down", "theta")]
+    _, idx, w, _, _ = ops.moe_forward(dev(p["x"]), *args, k, norm=norm, act=act, want_routing=True, n_pos=n_pos, n_neg=n_neg)
+    got = ops.moe_backward(dev(p["x"]), dev(d_out), *args, k, norm=norm, act=act, want_dw=True, n_pos=n_pos, n_neg=n_neg)
+    torch.cuda.synchronize()
+    ref = O.moe_backward(p["x"], p["w_router"], p["w_gate_up"], p["w_down"], p["theta"], idx.cpu().numpy(), d_out, norm=norm,
+                         act=act, n_pos=n_pos, n_neg=n_neg)
+    return dict(zip(("x", "w_router", "w_gate_up", "w_down", "theta", "w"), got)), ref, idx.cpu().numpy()
+
+
+@pytest.mark.parametrize("T,H,E,k,I", [(40, 48, 6, 2, 40), (130, 100, 16, 4, 72), (64, 256, 8, 2, 128)])
+def test_generic_backward_in_fp32_matches_oracle(T, H, E, k, I):
+    """fp32 operands, fp32 arithmetic, sizes that are no multiples of anything: every gradient against the fp64 oracle
+    at the tolerance the reference uses for its fp32 eager path against fp64 (ablate/common/test_eager_radial.py:61)."""
+    got, ref, _ = _run_generic(T, H, E, k, I, torch.float32, seed=T)
+    for name in ("w", "x", "w_down", "w_gate_up", "w_router", "theta"):
+        assert got[name].dtype == torch.float32
+        assert _rel(got[name], ref[name]) <= 1e-4, (name, _rel(got[name], ref[name]))
+
+
+@pytest.mark.parametrize("norm,act,n_pos,n_neg", [("softmax", "tanh", 0, 0), (False, "silu", 0, 0), ("sum", "radial", 1, 1)])
+def test_generic_backward_modes_and_identity_experts(norm, act, n_pos, n_neg):
+    got, ref, idx = _run_generic(90, 72, 6, 3, 48, torch.float32, norm=norm, act=act, seed=11, n_pos=n_pos, n_neg=n_neg)
+    if n_pos + n_neg:
+        assert (idx >= 6).sum() > 0
+    for name in ("w", "x", "w_down", "w_gate_up", "w_router") + (() if act == "silu" else ("theta",)):
+        assert _rel(got[name], ref[name]) <= 1e-4, (name, _rel(got[name], ref[name]))
+
+
+def test_generic_backward_in_bf16_on_odd_sizes():
+    """bf16 operands whose sizes the MFMA tiles do not divide: the generic kernels, bf16 results."""
+    got, ref, idx = _run_generic(150, 200, 8, 3, 96, torch.bfloat16, seed=3)
+    for name in ("w", "x", "w_down", "w_gate_up", "w_router", "theta"):
+        assert _rel(got[name], ref[name]) <= TOL, (name, _rel(got[name], ref[name]))
+    idle = np.setdiff1d(np.arange(8), np.unique(idx))
+    for e in idle:
+        assert float(got["w_down"][e].abs().max()) == 0.0
+
+
+def test_generic_experts_backward_with_padded_slots():
+    """The experts alone in fp32 with padding ids in a caller's indices: zero combine-weight gradient for those slots,
+    nothing of theirs in d_x (workspace poisoned first)."""
+    T, H, E, k, I = 60, 40, 5, 3, 24
+    p = O.make_inputs(T=T, H=H, E=E, k=k, I=I, theta="normal", seed=2)
+    g = torch.Generator().manual_seed(6)
+    idx = torch.randint(0, E, (T, k), generator=g, dtype=torch.int32)
+    idx[:, 0] = -1
+    w = torch.rand(T, k, generator=g) + 0.1
+    d_out = torch.randn(T, H, generator=g)
+    f = lambda t: t.float().to(DEV)
+    ops.workspace(DEV, 64 << 20).fill_(0x7f)
+    got = ops.experts_backward(f(p["x"]), f(d_out), idx.to(DEV), f(w), f(p["w_gate_up"]), f(p["w_down"]), f(p["theta"]))
+    torch.cuda.synchronize()
+    pad = idx < 0
+    w0, idx0 = w.clone(), idx.clone()
+    w0[pad] = 0.0
+    idx0[pad] = 0
+    leaf = lambda t: t.double().clone().requires_grad_(True)
+    x, wl, gu, dn, th = leaf(p["x"]), leaf(w0), leaf(p["w_gate_up"]), leaf(p["w_down"]), leaf(p["theta"])
+    (O.experts_forward(x, idx0, wl, gu, dn, th, dtype=torch.float64) * d_out.double()).sum().backward()
+    ref_w = wl.grad.clone()
+    ref_w[pad] = 0.0
+    assert float(got[1].cpu()[pad].abs().max()) == 0.0
+    for a, r, name in zip(got, (x.grad, ref_w, gu.grad, dn.grad, th.grad), ("x", "w", "w_gate_up", "w_down", "theta")):
+        assert bool(torch.isfinite(a.float()).all()) and _rel(a, r) <= 1e-4, (name, _rel(a, r))
 
 
 # ---- the module: BiBoMoELayer.forward under autograd ----
@@ -220,22 +300,45 @@ def test_seam_and_shared_expert_under_autograd():
             assert prm.grad is not None and bool(torch.isfinite(prm.grad.float()).all())
 
 
-def test_what_the_backward_does_not_cover_is_refused():
+def test_fp32_and_odd_sized_layers_train():
+    """The regimes of the reference's own gradient tests (tests/test_moe.py:53-63, ablate/common/test_eager_radial.py:
+    63-89): an fp32 layer of small, odd sizes under autograd.  theta starts at 0, receives a non-zero gradient, and
+    moving it moves the output; fp32 master weights under bf16 autocast train as well; only rows too long for the
+    generic kernels' LDS are refused."""
     from bibo_amd.config import BiBoMoEConfig
     from bibo_amd.moe import BiBoMoELayer
-    layer = BiBoMoELayer(BiBoMoEConfig(hidden_size=192, moe_intermediate_size=128, num_routed_experts=8,
-                                       num_experts_per_tok=2)).to(DEV).bfloat16()
-    x = torch.randn(1, 8, 192, device=DEV, dtype=torch.bfloat16)
-    with pytest.raises(NotImplementedError):
-        layer(x)                                                   # hidden size no multiple of 128: forward only
+    torch.manual_seed(1)
+    layer = BiBoMoELayer(BiBoMoEConfig(hidden_size=96, moe_intermediate_size=40, num_routed_experts=6,
+                                       num_experts_per_tok=2, special_expert_pairs=0)).to(DEV)
+    th = layer.experts.radial_theta
+    assert th.requires_grad and float(th.detach().abs().max()) == 0.0
+    x = torch.randn(2, 6, 96, device=DEV, requires_grad=True)
+    out = layer(x)
+    assert out.dtype == torch.float32
+    (out * torch.randn(2, 6, 96, device=DEV)).sum().backward()
+    assert th.grad is not None and float(th.grad.abs().max()) > 0 and x.grad is not None
+    for prm in layer.parameters():
+        if prm.requires_grad:
+            assert prm.grad is not None and prm.grad.dtype == torch.float32 and bool(torch.isfinite(prm.grad).all())
     with torch.no_grad():
-        layer(x)
+        base = layer(x).clone()
+        th += 2.0
+        assert float((layer(x) - base).abs().max()) > 1e-5
+    bf = BiBoMoELayer(BiBoMoEConfig(hidden_size=192, moe_intermediate_size=128, num_routed_experts=8,
+                                    num_experts_per_tok=2)).to(DEV).bfloat16()
+    xb = torch.randn(1, 8, 192, device=DEV, dtype=torch.bfloat16, requires_grad=True)
+    bf(xb).float().square().sum().backward()                       # hidden size no multiple of 128: generic kernels
+    assert xb.grad is not None and bf.experts.down_proj.grad is not None
     fp32 = _layer().float()
-    with pytest.raises(RuntimeError):
-        fp32(torch.randn(1, 8, 256, device=DEV))                   # fp32 compute: forward only
     with torch.autocast("cuda", dtype=torch.bfloat16):
-        fp32(torch.randn(1, 8, 256, device=DEV)).sum().backward()  # fp32 master weights under bf16 autocast train
+        fp32(torch.randn(1, 8, 256, device=DEV)).sum().backward()  # fp32 master weights under bf16 autocast
     assert fp32.experts.gate_up_proj.grad is not None and fp32.experts.gate_up_proj.grad.dtype == torch.float32
+    huge = BiBoMoELayer(BiBoMoEConfig(hidden_size=4096, moe_intermediate_size=2048, num_routed_experts=2,
+                                      num_experts_per_tok=1, special_expert_pairs=0)).to(DEV).bfloat16()
+    with pytest.raises(NotImplementedError):
+        huge(torch.randn(1, 4, 4096, device=DEV, dtype=torch.bfloat16))
+    with torch.no_grad():
+        huge(torch.randn(1, 4, 4096, device=DEV, dtype=torch.bfloat16))
 
 
 def test_experts_backward_with_caller_owned_routing():

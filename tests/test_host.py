@@ -243,13 +243,12 @@ def test_specials_and_shared_expert_follow_the_reference_layout():
     assert (asym.experts.num_glu_experts, asym.experts.pos_end, asym.experts.neg_end) == (5, 8, 8)
 
 
-def test_forward_refuses_to_drop_gradients():
-    """What has no backward says so instead of returning a result without a graph: fp32 compute in the layer and in
-    the experts module called on its own."""
+def test_forward_under_autograd_has_no_cpu_path_either():
+    """With gradients wanted the modules go to the library as without: host tensors are refused, not computed here."""
     layer = bibo_amd.BiBoMoELayer(make_config())
-    with pytest.raises(RuntimeError, match="backward pass runs in bf16"):
+    with pytest.raises(RuntimeError, match="no CPU path"):
         layer(torch.zeros(1, 4, 64))
-    with pytest.raises(RuntimeError, match="backward pass runs in bf16"):
+    with pytest.raises(RuntimeError, match="no CPU path"):
         layer.experts(torch.zeros(4, 64), torch.zeros(4, 2, dtype=torch.long), torch.ones(4, 2))
 
 
