@@ -125,6 +125,28 @@ def test_backward_idle_experts_and_ragged_rows():
     assert _rel(got["x"], ref["x"]) <= TOL and _rel(got["theta"], ref["theta"]) <= TOL
 
 
+@pytest.mark.parametrize("H,I,dtype", [(256, 128, torch.bfloat16), (48, 40, torch.float32)])
+def test_backward_of_a_few_tokens_and_of_none(H, I, dtype):
+    """One token, three tokens (far fewer rows than a tile holds) and an empty batch, in both kernel families: an
+    empty batch gives zero gradients for every parameter."""
+    E, k = 8, 2
+    tol = TOL if dtype == torch.bfloat16 else 1e-4
+    for T in (1, 3):
+        got, ref, _ = _run_generic(T, H, E, k, I, dtype, seed=T)
+        for name in ("w", "x", "w_down", "w_gate_up", "w_router", "theta"):
+            assert _rel(got[name], ref[name]) <= tol, (T, name, _rel(got[name], ref[name]))
+    p = O.make_inputs(T=4, H=H, E=E, k=k, I=I, seed=0)
+    dev = lambda t: (t.to(dtype) if t.dtype == torch.bfloat16 else t).to(DEV)
+    none = torch.empty(0, H, dtype=dtype, device=DEV)
+    ops.workspace(DEV, 1 << 20).fill_(0x7f)
+    got = ops.moe_backward(none, none, dev(p["w_router"]), dev(p["bias"]), dev(p["w_gate_up"]), dev(p["w_down"]),
+                           dev(p["theta"]), k)
+    torch.cuda.synchronize()
+    assert got[0].shape == (0, H)
+    for g in got[1:5]:
+        assert float(g.float().abs().max()) == 0.0
+
+
 def test_backward_is_linear_in_the_upstream_gradient():
     """Size-independent property at the full c2 shape: the gradients of 2 d are twice those of d (every path is linear
     in d_out), to bf16 rounding; and nothing is accumulated between calls."""
