@@ -236,7 +236,9 @@ def test_model_with_hip_moe_layers_matches_the_oracle(dtype, tol):
     assert sorted(routing) == list(range(1, 9))
     sd = {k: v.detach().cpu() for k, v in model.state_dict().items()}
     ref = XO.forward(ids, sd, cfg, dtype=torch.float32, routing=routing)
-    assert torch.isfinite(logits).all() and rel_err(logits.cpu(), ref) <= tol
+    err = rel_err(logits.cpu(), ref)
+    print(f"reduced config 5, {dtype}: rel err {err:.3e} (bar {tol:g})")
+    assert torch.isfinite(logits).all() and err <= tol
 
 
 @pytest.mark.gpu

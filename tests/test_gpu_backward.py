@@ -12,6 +12,7 @@ from oracle import bibo_moe_oracle as O
 pytestmark = pytest.mark.gpu
 DEV = torch.device("cuda:0")
 TOL = 2e-2          # bf16 operands, fp32 accumulation, bf16 results
+F32_TOL = 1e-5      # fp32 operands and arithmetic against the fp64 oracle (measured below 1e-6)
 
 
 def _rel(a, ref):
@@ -130,7 +131,7 @@ def test_backward_of_a_few_tokens_and_of_none(H, I, dtype):
     """One token, three tokens (far fewer rows than a tile holds) and an empty batch, in both kernel families: an
     empty batch gives zero gradients for every parameter."""
     E, k = 8, 2
-    tol = TOL if dtype == torch.bfloat16 else 1e-4
+    tol = TOL if dtype == torch.bfloat16 else F32_TOL
     for T in (1, 3):
         got, ref, _ = _run_generic(T, H, E, k, I, dtype, seed=T)
         for name in ("w", "x", "w_down", "w_gate_up", "w_router", "theta"):
@@ -204,11 +205,13 @@ def _run_generic(T, H, E, k, I, dtype, norm="sum", act="radial", seed=0, n_pos=0
 @pytest.mark.parametrize("T,H,E,k,I", [(40, 48, 6, 2, 40), (130, 100, 16, 4, 72), (64, 256, 8, 2, 128)])
 def test_generic_backward_in_fp32_matches_oracle(T, H, E, k, I):
     """fp32 operands, fp32 arithmetic, sizes that are no multiples of anything: every gradient against the fp64 oracle
-    at the tolerance the reference uses for its fp32 eager path against fp64 (ablate/common/test_eager_radial.py:61)."""
+    at 1e-5 of each tensor's maximum."""
     got, ref, _ = _run_generic(T, H, E, k, I, torch.float32, seed=T)
-    for name in ("w", "x", "w_down", "w_gate_up", "w_router", "theta"):
+    errs = {name: _rel(got[name], ref[name]) for name in ("w", "x", "w_down", "w_gate_up", "w_router", "theta")}
+    print("fp32 backward", (T, H, E, k, I), {n: f"{e:.1e}" for n, e in errs.items()})
+    for name, err in errs.items():
         assert got[name].dtype == torch.float32
-        assert _rel(got[name], ref[name]) <= 1e-4, (name, _rel(got[name], ref[name]))
+        assert err <= F32_TOL, (name, err)
 
 
 @pytest.mark.parametrize("norm,act,n_pos,n_neg", [("softmax", "tanh", 0, 0), (False, "silu", 0, 0), ("sum", "radial", 1, 1)])
@@ -217,7 +220,7 @@ def test_generic_backward_modes_and_identity_experts(norm, act, n_pos, n_neg):
     if n_pos + n_neg:
         assert (idx >= 6).sum() > 0
     for name in ("w", "x", "w_down", "w_gate_up", "w_router") + (() if act == "silu" else ("theta",)):
-        assert _rel(got[name], ref[name]) <= 1e-4, (name, _rel(got[name], ref[name]))
+        assert _rel(got[name], ref[name]) <= F32_TOL, (name, _rel(got[name], ref[name]))
 
 
 def test_generic_backward_in_bf16_on_odd_sizes():
@@ -255,7 +258,7 @@ def test_generic_experts_backward_with_padded_slots():
     ref_w[pad] = 0.0
     assert float(got[1].cpu()[pad].abs().max()) == 0.0
     for a, r, name in zip(got, (x.grad, ref_w, gu.grad, dn.grad, th.grad), ("x", "w", "w_gate_up", "w_down", "theta")):
-        assert bool(torch.isfinite(a.float()).all()) and _rel(a, r) <= 1e-4, (name, _rel(a, r))
+        assert bool(torch.isfinite(a.float()).all()) and _rel(a, r) <= F32_TOL, (name, _rel(a, r))
 
 
 # ---- the module: BiBoMoELayer.forward under autograd ----
