@@ -37,7 +37,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_shape_struct_matches_the_header_and_the_documented_binding():
     """bibo_moe_shape is read by pointer: a binding with fewer fields makes the library read past the caller's
-    struct.  The ctypes structure, the header and the example in INTEGRATION.md must agree field for field."""
+    struct.  The ctypes structure, the header and the example in the integration guide at the repository root must agree field for field."""
     header = (ROOT / "include" / "bibo_moe.h").read_text()
     body = re.search(r"typedef struct bibo_moe_shape \{(.*?)\} bibo_moe_shape;", header, re.S).group(1)
     fields = re.findall(r"int32_t\s+(\w+);", body)
