@@ -299,9 +299,10 @@ hipError_t launch_t(const void* x_, const void* d_out_, const void* w_router_, c
 
 }  // namespace
 
-// the row kernel keeps 2H + 5I floats of a row in LDS
+// the row kernel keeps 2H + 5I floats of a row in dynamic LDS next to a few words of its own; 64 KB per workgroup
+// need no raised limit
 bool backward_generic_supported(int H, int I, int k) {
-  return (size_t)(2 * H + 5 * I) * sizeof(float) <= 64 * 1024 && k <= kMaxK;
+  return (size_t)(2 * H + 5 * I) * sizeof(float) + 64 <= 64 * 1024 && k <= kMaxK;
 }
 
 // Buffers (fp32): dgu [S,2I], hw [S,I], dxs [S,H], dw_slot [S], dl [S], dtheta_row [S].

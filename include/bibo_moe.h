@@ -279,7 +279,7 @@ int bibo_moe_ffn_forward(const void* h, const float* norm_weight, float eps, con
  * accumulation, results rounded once); every other size and fp32 run generic kernels that compute in fp32 throughout
  * (fp32 operands give fp32-exact gradients, the regime of the reference's own gradient tests) and keep
  * 2H + 5I floats of a row in LDS: BIBO_ERR_UNSUPPORTED when neither applies, i.e. off the MFMA sizes with
- * (2H + 5I) * 4 > 65536.  The intermediate activations are recomputed, nothing has to be kept from the forward
+ * (2H + 5I) * 4 + 64 > 65536.  The intermediate activations are recomputed, nothing has to be kept from the forward
  * call.  All gradients are overwritten, not accumulated.  Workspace: bibo_moe_backward_workspace_bytes (MFMA family:
  * about 12 I + 2 H bytes per routed slot; generic family: 12 I + 4 H).
  */

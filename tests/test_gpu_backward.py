@@ -233,6 +233,14 @@ def test_generic_backward_in_bf16_on_odd_sizes():
         assert float(got["w_down"][e].abs().max()) == 0.0
 
 
+def test_generic_backward_at_the_lds_limit():
+    """The longest rows the generic kernels take: 2H + 5I floats just under 64 KB of LDS."""
+    got, ref, _ = _run_generic(4, 4096, 2, 1, 1616, torch.bfloat16, seed=9)
+    for name in ("w", "x", "w_down", "w_gate_up", "w_router", "theta"):
+        assert _rel(got[name], ref[name]) <= TOL, (name, _rel(got[name], ref[name]))
+    assert not ops.backward_supported(4096, 1664, 2, torch.bfloat16)
+
+
 def test_generic_experts_backward_with_padded_slots():
     """The experts alone in fp32 with padding ids in a caller's indices: zero combine-weight gradient for those slots,
     nothing of theirs in d_x (workspace poisoned first)."""
