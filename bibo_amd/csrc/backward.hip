@@ -129,15 +129,23 @@ hipError_t launch_ggemm(const bf16_t* A, const int32_t* a_index, const bf16_t* W
   return launch_ggemm_t<1, GATHER, SCATTER>(A, a_index, W, offsets, out_index, S_rows, K, N, E, out, s);
 }
 
+// 256-row tiles once the experts hold 192 rows on average (a 256-row tile then is at least half full where it matters)
+inline bool tall_tiles(int S_rows, int E) { return (long long)S_rows >= 192ll * E; }
+
 template <int NTW, bool GATHER, bool SCATTER>
 hipError_t launch_dgrad_t(const bf16_t* A, const int32_t* a_index, const bf16_t* W, const int32_t* offsets,
                           const int32_t* out_index, int S_rows, int K, int N, int E, bf16_t* out, hipStream_t s) {
-  constexpr int BM = 128, BN = kSubW * NTW;
+  constexpr int BN = kSubW * NTW;
   const int nblk_n = N / BN;
-  const int tiles = (S_rows / BM + E) * nblk_n;
+  const bool tall = tall_tiles(S_rows, E);
+  const int tiles = (S_rows / (tall ? 256 : 128) + E) * nblk_n;
   const int grid = ((tiles + 7) & ~7) + 8;
-  hipLaunchKernelGGL((dgrad_kmajor_kernel<NTW, GATHER, SCATTER>), dim3(grid), dim3(512), 0, s, A, a_index, W, offsets,
-                     out_index, K, N, E, nblk_n, out);
+  if (tall)
+    hipLaunchKernelGGL((dgrad_kmajor_kernel<4, NTW, GATHER, SCATTER>), dim3(grid), dim3(512), 0, s, A, a_index, W, offsets,
+                       out_index, K, N, E, nblk_n, out);
+  else
+    hipLaunchKernelGGL((dgrad_kmajor_kernel<2, NTW, GATHER, SCATTER>), dim3(grid), dim3(512), 0, s, A, a_index, W, offsets,
+                       out_index, K, N, E, nblk_n, out);
   return hipGetLastError();
 }
 

@@ -95,6 +95,33 @@ __device__ __forceinline__ void multiply_stage(floatx16 (&acc)[MT][NTW], ReadA r
   }
 }
 
+// The same for a tall tile (MT = 4 row tiles per wave): 192 accumulator registers leave no room for two sets of every
+// fragment, so the row operand is read one fragment ahead and only the column operand is held for a whole k16 step;
+// the column fragments of the next step are read during the first NTW pairs of this one.  kARd = LDS reads per row
+// fragment (1: a 16-byte read, 2: a pair of transposing reads).
+template <int MT, int NTW, int kARd, typename ReadA, typename ReadB>
+__device__ __forceinline__ void multiply_stage_tall(floatx16 (&acc)[MT][NTW], ReadA read_a, ReadB read_b) {
+  constexpr int kSteps = kKS / 16, kPairs = kSteps * MT;
+  static_assert(MT >= NTW, "a step's pairs carry the next step's column fragments");
+  bf16x8 af[2], bfr[2][NTW];
+#pragma unroll
+  for (int j = 0; j < NTW; ++j) bfr[0][j] = read_b(0, j);
+  af[0] = read_a(0, 0);
+#pragma unroll
+  for (int p = 0; p < kPairs; ++p) {
+    const int s = p / MT, mt = p % MT;
+    const bool more_a = p + 1 < kPairs, more_b = s + 1 < kSteps && mt < NTW;
+    if (more_a) af[(p + 1) & 1] = read_a((p + 1) / MT, (p + 1) % MT);
+    if (more_b) bfr[(s + 1) & 1][mt] = read_b(s + 1, mt);
+#pragma unroll
+    for (int j = 0; j < NTW; ++j)
+      acc[mt][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[s & 1][j], af[p & 1], acc[mt][j], 0, 0, 0);
+    if (more_a) __builtin_amdgcn_sched_group_barrier(0x100, kARd, 0);
+    if (more_b) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+    __builtin_amdgcn_sched_group_barrier(0x008, NTW, 0);
+  }
+}
+
 // Row-major operand tile [128 rows][32 k] in the stripe layout for 64-byte rows (granule c of row r at
 // c ^ ((r >> 2) & 3)): thread t of the fill writes row t / 4, position t % 4.  `row` = that row's K extent, already
 // offset to the stage's first k and to this thread's granule (afill_granule).
@@ -111,24 +138,29 @@ __device__ __forceinline__ void afill(const bf16_t* row, bf16_t* tile) {
 
 // ---- input gradients: out[dst(r), n] = sum_k A[src(r), k] W[e][k, n] for the rows r of expert e ----------------
 // A row-major (K contiguous), W K-major as stored: [K, N] per expert.  src(r) = a_index[r] (GATHER) or r; dst(r) =
-// out_index[r] (SCATTER) or r.  Workgroup = 128 rows x 128 NTW columns, 2 x 4 waves, 32x32x16 MFMA, operands swapped
-// so that a lane owns one output row.  K is a multiple of 128.
-template <int NTW, bool GATHER, bool SCATTER>
+// out_index[r] (SCATTER) or r.  Workgroup = 64 MT rows x 128 NTW columns, 2 x 4 waves, 32x32x16 MFMA, operands swapped
+// so that a lane owns one output row.  K is a multiple of 128.  MT = 2: 128-row tiles, ring of four stages.  MT = 4:
+// 256-row tiles for experts with many rows - an expert's weights then pass through LDS once per 256 rows instead of
+// once per 128, which is what these kernels are bound by; 192 accumulator registers and 40 KB stages, ring of three.
+template <int MT, int NTW, bool GATHER, bool SCATTER>
 __global__ __launch_bounds__(512) void dgrad_kmajor_kernel(const bf16_t* __restrict__ A, const int32_t* __restrict__ a_index,
                                                            const bf16_t* __restrict__ W,
                                                            const int32_t* __restrict__ offsets,
                                                            const int32_t* __restrict__ out_index, int K, int N, int E,
                                                            int nblk_n, bf16_t* __restrict__ out) {
-  constexpr int MT = 2, BM = 128, BN = kSubW * NTW;
-  constexpr int kOps = 1 + NTW;                          // transfers per thread and stage
-  __shared__ __attribute__((aligned(16))) bf16_t a0[kATile];
-  __shared__ __attribute__((aligned(16))) bf16_t a1[kATile];
-  __shared__ __attribute__((aligned(16))) bf16_t a2[kATile];
-  __shared__ __attribute__((aligned(16))) bf16_t a3[kATile];
+  static_assert(MT == 2 || MT == 4, "128- or 256-row tiles");
+  constexpr int BM = 64 * MT, BN = kSubW * NTW;
+  constexpr int R = MT == 4 ? 3 : kRing;                 // stages that fit LDS
+  constexpr int kAOps = MT / 2;                          // 128-row blocks of the row operand
+  constexpr int kOps = kAOps + NTW;                      // transfers per thread and stage
+  __shared__ __attribute__((aligned(16))) bf16_t a0[kAOps * kATile];
+  __shared__ __attribute__((aligned(16))) bf16_t a1[kAOps * kATile];
+  __shared__ __attribute__((aligned(16))) bf16_t a2[kAOps * kATile];
+  __shared__ __attribute__((aligned(16))) bf16_t a3[R == 4 ? kAOps * kATile : 8];
   __shared__ __attribute__((aligned(16))) bf16_t b0[NTW * kSubElems];
   __shared__ __attribute__((aligned(16))) bf16_t b1[NTW * kSubElems];
   __shared__ __attribute__((aligned(16))) bf16_t b2[NTW * kSubElems];
-  __shared__ __attribute__((aligned(16))) bf16_t b3[NTW * kSubElems];
+  __shared__ __attribute__((aligned(16))) bf16_t b3[R == 4 ? NTW * kSubElems : 8];
   __shared__ int dst_s[BM];
 
   const TileMap tm = make_tile_map(offsets, E, BM);
@@ -146,8 +178,12 @@ __global__ __launch_bounds__(512) void dgrad_kmajor_kernel(const bf16_t* __restr
     dst_s[tid] = SCATTER ? out_index[r] : r;
   }
   // fill side
-  const int ar = row0 + min(tid >> 2, rows - 1);                   // rows past the end re-read the last one
-  const bf16_t* arow = A + (size_t)(GATHER ? a_index[ar] : ar) * K + afill_granule(tid) * 8;
+  const bf16_t* arow[kAOps];
+#pragma unroll
+  for (int hb = 0; hb < kAOps; ++hb) {
+    const int ar = row0 + min(hb * 128 + (tid >> 2), rows - 1);    // rows past the end re-read the last one
+    arow[hb] = A + (size_t)(GATHER ? a_index[ar] : ar) * K + afill_granule(tid) * 8;
+  }
   const int n0 = nb * BN;
   const bf16_t* wrow = W + (size_t)e * K * N + (size_t)(tid >> 4) * N + n0 + kfill_granule(tid) * 8;
   const int nstages = K / kKS;
@@ -161,7 +197,8 @@ __global__ __launch_bounds__(512) void dgrad_kmajor_kernel(const bf16_t* __restr
   };
   auto fill = [&](auto bc, int stage) {
     const int k0 = min(stage, nstages - 1) * kKS;
-    afill(arow + k0, abuf(bc));
+#pragma unroll
+    for (int hb = 0; hb < kAOps; ++hb) afill(arow[hb] + k0, abuf(bc) + hb * kATile);
     const bf16_t* w0 = wrow + (size_t)k0 * N;
 #pragma unroll
     for (int j = 0; j < NTW; ++j) kfill_subtile(w0 + j * kSubW, bbuf(bc) + j * kSubElems);
@@ -169,7 +206,7 @@ __global__ __launch_bounds__(512) void dgrad_kmajor_kernel(const bf16_t* __restr
   using std::integral_constant;
   fill(integral_constant<int, 0>{}, 0);
   fill(integral_constant<int, 1>{}, 1);
-  fill(integral_constant<int, 2>{}, 2);
+  if constexpr (R == 4) fill(integral_constant<int, 2>{}, 2);
 
   floatx16 acc[MT][NTW];
 #pragma unroll
@@ -191,21 +228,23 @@ __global__ __launch_bounds__(512) void dgrad_kmajor_kernel(const bf16_t* __restr
     const int t32 = wn * NTW + j;
     boff[j] = (t32 >> 2) * kSubElems + kfrag_offset(lane, (t32 & 3) * 32);
   }
-  auto step = [&](auto bc, auto nc, int stage) {
-    sync_keep_loads<2 * kOps>();
-    fill(nc, stage + 3);
+  // step `stage` reads buffer stage % R and requests stage + R - 1 into the buffer stage - 1 was read from
+  auto step = [&](auto bc, int stage) {
+    constexpr int b = decltype(bc)::value;
+    sync_keep_loads<(R - 2) * kOps>();
+    fill(integral_constant<int, (b + R - 1) % R>{}, stage + R - 1);
     const bf16_t* at = abuf(bc);
     const bf16_t* bt = bbuf(bc);
-    multiply_stage<MT, NTW>(
-        acc,
-        [&](int s, int mt) { return *reinterpret_cast<const bf16x8*>(at + aoff + mt * 32 * kKS + (apos0 ^ (s * 16))); },
-        [&](int s, int j) { return kfrag_read_s(bt, boff[j], s); });
+    auto read_a = [&](int s, int mt) { return *reinterpret_cast<const bf16x8*>(at + aoff + mt * 32 * kKS + (apos0 ^ (s * 16))); };
+    auto read_b = [&](int s, int j) { return kfrag_read_s(bt, boff[j], s); };
+    if constexpr (MT == 2) multiply_stage<MT, NTW>(acc, read_a, read_b);      // nstages is a multiple of 4
+    else if (stage < nstages) multiply_stage_tall<MT, NTW, 1>(acc, read_a, read_b);
   };
-  for (int i = 0; i < nstages; i += 4) {                           // nstages is a multiple of 4
-    step(integral_constant<int, 0>{}, integral_constant<int, 3>{}, i);
-    step(integral_constant<int, 1>{}, integral_constant<int, 0>{}, i + 1);
-    step(integral_constant<int, 2>{}, integral_constant<int, 1>{}, i + 2);
-    step(integral_constant<int, 3>{}, integral_constant<int, 2>{}, i + 3);
+  for (int i = 0; i < nstages; i += R) {
+    step(integral_constant<int, 0>{}, i);
+    step(integral_constant<int, 1>{}, i + 1);
+    step(integral_constant<int, 2>{}, i + 2);
+    if constexpr (R == 4) step(integral_constant<int, 3>{}, i + 3);
   }
   wait_loads_and_sync();                 // the repeated requests of the last steps have landed; every wave is done reading
 
@@ -214,10 +253,10 @@ __global__ __launch_bounds__(512) void dgrad_kmajor_kernel(const bf16_t* __restr
   const int hh = lane >> 5;
   constexpr int kOutCols = NTW * 32;
   constexpr int kOutStride = kOutCols + 8;          // +16 bytes staggers the rows over the banks
-  static_assert(2 * 32 * kOutStride <= NTW * kSubElems, "output staging does not fit a weight stage");
-  bf16_t* otile = bbuf(integral_constant<int, 0>{});
-  if (wave >= 6) otile = b3; else if (wave >= 4) otile = b2; else if (wave >= 2) otile = b1;
-  otile += (wave & 1) * (32 * kOutStride);
+  static_assert(3 * 32 * kOutStride <= NTW * kSubElems, "output staging does not fit a weight stage");
+  bf16_t* otile = b0;                    // three waves per stage buffer
+  if (wave >= 6) otile = b2; else if (wave >= 3) otile = b1;
+  otile += (wave % 3) * (32 * kOutStride);
   constexpr int kGranPerRow = kOutCols / 8;
   const int colbase = n0 + wn * kOutCols;
 #pragma unroll

@@ -36,7 +36,8 @@ def _run(T, H, E, k, I, norm="sum", act="radial", seed=0, theta="normal", scale=
 
 
 @pytest.mark.parametrize("T,H,E,k,I", [(300, 256, 16, 4, 128), (512, 512, 64, 6, 256), (64, 384, 8, 2, 384), (1000, 768, 64, 6, 384),
-                                       (200, 1024, 16, 4, 512)])     # the widest rows the backward pass takes
+                                       (200, 1024, 16, 4, 512),      # the widest rows the backward pass takes
+                                       (600, 256, 4, 2, 128), (700, 768, 5, 3, 384)])   # 300 / 420 rows per expert: 256-row tiles
 def test_backward_matches_oracle(T, H, E, k, I):
     got, ref, _ = _run(T, H, E, k, I, seed=T)
     for name in ("w", "x", "w_down", "w_gate_up", "w_router", "theta"):
