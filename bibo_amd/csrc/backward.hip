@@ -129,15 +129,23 @@ hipError_t launch_ggemm(const bf16_t* A, const int32_t* a_index, const bf16_t* W
   return launch_ggemm_t<1, GATHER, SCATTER>(A, a_index, W, offsets, out_index, S_rows, K, N, E, out, s);
 }
 
-// 256-row tiles once the experts hold 192 rows on average (a 256-row tile then is at least half full where it matters)
-inline bool tall_tiles(int S_rows, int E) { return (long long)S_rows >= 192ll * E; }
+// 256-row tiles stream an expert's weights through LDS half as often as 128-row tiles but take about 1.75 times as
+// long each, and the workgroups of a launch run in rounds of one per CU (256 on this chip): the tall tiles pay when
+// their rounds, weighted so, are fewer.  Only for experts that hold 192 rows on average (a 256-row tile is then at
+// least half full where it matters).
+inline bool tall_tiles(int S_rows, int E, long long tiles_short, long long tiles_tall) {
+  constexpr long long kCUs = 256;
+  const long long rs = (tiles_short + kCUs - 1) / kCUs, rt = (tiles_tall + kCUs - 1) / kCUs;
+  return (long long)S_rows >= 192ll * E && rt * 7 < rs * 4;
+}
 
 template <int NTW, bool GATHER, bool SCATTER>
 hipError_t launch_dgrad_t(const bf16_t* A, const int32_t* a_index, const bf16_t* W, const int32_t* offsets,
                           const int32_t* out_index, int S_rows, int K, int N, int E, bf16_t* out, hipStream_t s) {
   constexpr int BN = kSubW * NTW;
   const int nblk_n = N / BN;
-  const bool tall = tall_tiles(S_rows, E);
+  // an expert's last tile is ragged: about half a tile per expert on top of the full ones
+  const bool tall = tall_tiles(S_rows, E, (long long)(S_rows / 128 + E / 2) * nblk_n, (long long)(S_rows / 256 + E / 2) * nblk_n);
   const int tiles = (S_rows / (tall ? 256 : 128) + E) * nblk_n;
   const int grid = ((tiles + 7) & ~7) + 8;
   if (tall)
@@ -159,21 +167,31 @@ hipError_t launch_dgrad(const bf16_t* A, const int32_t* a_index, const bf16_t* W
 }
 
 // dW[e] = P(rows of e)^T Q(rows of e), P [.., N] and Q [.., M] row-major (kmajor.h)
+template <int MT, bool GATHER_P, bool GATHER_Q>
+hipError_t launch_wgrad_t(const bf16_t* P, const bf16_t* Q, const int32_t* index, const int32_t* offsets, const bf16_t* zrow,
+                          int N, int M, int E, bf16_t* dW, hipStream_t s) {
+  const dim3 block(512);
+  auto grid = [&](int bn) { return dim3((unsigned)((E * (N / (64 * MT)) * (M / bn) + 7) & ~7)); };
+  if (M % 384 == 0)
+    hipLaunchKernelGGL((wgrad_kmajor_kernel<MT, 3, GATHER_P, GATHER_Q>), grid(384), block, 0, s, P, Q, index, offsets, zrow, N,
+                       M, E, dW);
+  else if (M % 256 == 0)
+    hipLaunchKernelGGL((wgrad_kmajor_kernel<MT, 2, GATHER_P, GATHER_Q>), grid(256), block, 0, s, P, Q, index, offsets, zrow, N,
+                       M, E, dW);
+  else
+    hipLaunchKernelGGL((wgrad_kmajor_kernel<MT, 1, GATHER_P, GATHER_Q>), grid(128), block, 0, s, P, Q, index, offsets, zrow, N,
+                       M, E, dW);
+  return hipGetLastError();
+}
+
+// 256 rows of dW per workgroup where N allows and the experts have rows enough for the streams to matter
 template <bool GATHER_P, bool GATHER_Q>
 hipError_t launch_wgrad(const bf16_t* P, const bf16_t* Q, const int32_t* index, const int32_t* offsets, const bf16_t* zrow,
                         int N, int M, int S_rows, int E, bf16_t* dW, hipStream_t s) {
-  const dim3 block(512);
-  auto grid = [&](int bn) { return dim3((unsigned)((E * (N / 128) * (M / bn) + 7) & ~7)); };
-  if (M % 384 == 0)
-    hipLaunchKernelGGL((wgrad_kmajor_kernel<3, GATHER_P, GATHER_Q>), grid(384), block, 0, s, P, Q, index, offsets, zrow, N, M, E,
-                       dW);
-  else if (M % 256 == 0)
-    hipLaunchKernelGGL((wgrad_kmajor_kernel<2, GATHER_P, GATHER_Q>), grid(256), block, 0, s, P, Q, index, offsets, zrow, N, M, E,
-                       dW);
-  else
-    hipLaunchKernelGGL((wgrad_kmajor_kernel<1, GATHER_P, GATHER_Q>), grid(128), block, 0, s, P, Q, index, offsets, zrow, N, M, E,
-                       dW);
-  return hipGetLastError();
+  const int bn = M % 384 == 0 ? 384 : (M % 256 == 0 ? 256 : 128);
+  if (N % 256 == 0 && tall_tiles(S_rows, E, (long long)E * (N / 128) * (M / bn), (long long)E * (N / 256) * (M / bn)))
+    return launch_wgrad_t<4, GATHER_P, GATHER_Q>(P, Q, index, offsets, zrow, N, M, E, dW, s);
+  return launch_wgrad_t<2, GATHER_P, GATHER_Q>(P, Q, index, offsets, zrow, N, M, E, dW, s);
 }
 
 // ---- Radial NormSiLU backward (moe.py:87-92), one wave per permuted row ----------------------------------------

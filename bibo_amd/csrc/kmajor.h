@@ -288,23 +288,27 @@ __global__ __launch_bounds__(512) void dgrad_kmajor_kernel(const bf16_t* __restr
 // Both operands row-major activations, contracted over their rows: K-major both.  srcP(r) = index[r] (GATHER_P) or r,
 // likewise Q.  A K stage is 32 rows; rows past the expert's end read `zrow` (zeros, at least 128 elements) on the P
 // side and the expert's last row on the Q side (memory that is certainly finite, whatever the rows behind the
-// expert's hold).  One workgroup per (expert, 128 rows of dW, 128 NTW columns of dW).
-template <int NTW, bool GATHER_P, bool GATHER_Q>
+// expert's hold).  One workgroup per (expert, 64 MT rows of dW, 128 NTW columns of dW); MT = 4 (256 rows) halves what
+// a workgroup streams of Q per row of dW, at 192 accumulator registers and a ring of three 40 KB stages.
+template <int MT, int NTW, bool GATHER_P, bool GATHER_Q>
 __global__ __launch_bounds__(512) void wgrad_kmajor_kernel(const bf16_t* __restrict__ P, const bf16_t* __restrict__ Q,
                                                            const int32_t* __restrict__ index,
                                                            const int32_t* __restrict__ offsets,
                                                            const bf16_t* __restrict__ zrow, int N, int M, int E,
                                                            bf16_t* __restrict__ dW) {
-  constexpr int MT = 2, BM = 128, BN = kSubW * NTW;
-  constexpr int kOps = 1 + NTW;
-  __shared__ __attribute__((aligned(16))) bf16_t p0[kSubElems];
-  __shared__ __attribute__((aligned(16))) bf16_t p1[kSubElems];
-  __shared__ __attribute__((aligned(16))) bf16_t p2[kSubElems];
-  __shared__ __attribute__((aligned(16))) bf16_t p3[kSubElems];
+  static_assert(MT == 2 || MT == 4, "128 or 256 rows of dW per workgroup");
+  constexpr int BM = 64 * MT, BN = kSubW * NTW;
+  constexpr int R = MT == 4 ? 3 : kRing;                 // stages that fit LDS (MT = 4: 40 KB each)
+  constexpr int kPOps = MT / 2;                          // 128-column sub-tiles of P
+  constexpr int kOps = kPOps + NTW;
+  __shared__ __attribute__((aligned(16))) bf16_t p0[kPOps * kSubElems];
+  __shared__ __attribute__((aligned(16))) bf16_t p1[kPOps * kSubElems];
+  __shared__ __attribute__((aligned(16))) bf16_t p2[kPOps * kSubElems];
+  __shared__ __attribute__((aligned(16))) bf16_t p3[R == 4 ? kPOps * kSubElems : 8];
   __shared__ __attribute__((aligned(16))) bf16_t q0[NTW * kSubElems];
   __shared__ __attribute__((aligned(16))) bf16_t q1[NTW * kSubElems];
   __shared__ __attribute__((aligned(16))) bf16_t q2[NTW * kSubElems];
-  __shared__ __attribute__((aligned(16))) bf16_t q3[NTW * kSubElems];
+  __shared__ __attribute__((aligned(16))) bf16_t q3[R == 4 ? NTW * kSubElems : 8];
   // Workgroup ids congruent mod 8 run on one XCD: they walk a contiguous range of (expert, m block, n block) triples,
   // so the workgroups that read the same rows of Q (and of P) share that XCD's L2.
   const int nblk_n = N / BM, nblk_m = M / BN;
@@ -344,13 +348,17 @@ __global__ __launch_bounds__(512) void wgrad_kmajor_kernel(const bf16_t* __restr
     const int rc = live ? r : hi - 1;
     const bf16_t* prow = live ? P + (size_t)(GATHER_P ? ix : rc) * N + n0 : zrow;
     const bf16_t* qrow = Q + (size_t)(GATHER_Q ? ix : rc) * M + m0;
-    kfill_subtile(prow + gofs, pbuf(bc));
+#pragma unroll
+    for (int j = 0; j < kPOps; ++j) kfill_subtile(prow + j * kSubW + gofs, pbuf(bc) + j * kSubElems);
 #pragma unroll
     for (int j = 0; j < NTW; ++j) kfill_subtile(qrow + j * kSubW + gofs, qbuf(bc) + j * kSubElems);
   };
   int poff[MT], qoff[NTW];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) poff[mt] = kfrag_offset(lane, (wm * MT + mt) * 32);
+  for (int mt = 0; mt < MT; ++mt) {
+    const int t32 = wm * MT + mt;
+    poff[mt] = (t32 >> 2) * kSubElems + kfrag_offset(lane, (t32 & 3) * 32);
+  }
 #pragma unroll
   for (int j = 0; j < NTW; ++j) {
     const int t32 = wn * NTW + j;
@@ -358,37 +366,42 @@ __global__ __launch_bounds__(512) void wgrad_kmajor_kernel(const bf16_t* __restr
   }
   using std::integral_constant;
   if (nstages > 0) {                                               // an idle expert's gradient is zero
-    // The row index of a gathered operand is loaded three steps before the transfers that use it (four values
-    // rotate through ix[]): step s requests stage s + 3 with the index loaded at step s - 3 and loads the one of
-    // stage s + 6.  That load is one more vector-memory operation per step, so the ring's wait counts it.
+    // The row index of a gathered operand is loaded R - 1 steps before the transfers that use it (R values rotate
+    // through ix[], the index of stage s in ix[s % R]): step s requests stage s + R - 1 with the index loaded at step
+    // s - R + 1 and loads the one of stage s + 2 (R - 1).  That load is one more vector-memory operation per step, so
+    // the ring's wait counts it.
     constexpr int kVm = kOps + ((GATHER_P || GATHER_Q) ? 1 : 0);
-    int ix[4];
-    ix[0] = lookup(0); ix[1] = lookup(1); ix[2] = lookup(2);
-    fill(integral_constant<int, 0>{}, 0, ix[0]);
-    ix[3] = lookup(3);
-    fill(integral_constant<int, 1>{}, 1, ix[1]);
-    ix[0] = lookup(4);
-    fill(integral_constant<int, 2>{}, 2, ix[2]);
-    ix[1] = lookup(5);
-    // now in flight, oldest first: stage 0, index 3, stage 1, index 4, stage 2, index 5
-    auto step = [&](auto bc, auto nc, int stage) {
+    int ix[R];
+    // prologue, oldest request first: stage 0, index R - 1, stage 1, index R, ... stage R - 2, index 2 R - 3
+#pragma unroll
+    for (int i = 0; i < R - 1; ++i) ix[i] = lookup(i);
+    auto prologue = [&](auto ic) {
+      constexpr int i = decltype(ic)::value;
+      fill(integral_constant<int, i>{}, i, ix[i]);
+      ix[(i + R - 1) % R] = lookup(i + R - 1);
+    };
+    prologue(integral_constant<int, 0>{});
+    prologue(integral_constant<int, 1>{});
+    if constexpr (R == 4) prologue(integral_constant<int, 2>{});
+    auto step = [&](auto bc, int stage) {
       constexpr int b = decltype(bc)::value;
-      sync_keep_loads<2 * kVm>();
-      fill(nc, stage + 3, ix[(b + 3) & 3]);
-      ix[(b + 2) & 3] = lookup(stage + 6);
+      sync_keep_loads<(R - 2) * kVm>();
+      fill(integral_constant<int, (b + R - 1) % R>{}, stage + R - 1, ix[(b + R - 1) % R]);
+      ix[(b + R - 2) % R] = lookup(stage + 2 * (R - 1));
       if (stage < nstages) {
         const bf16_t* pt = pbuf(bc);
         const bf16_t* qt = qbuf(bc);
-        multiply_stage<MT, NTW>(
-            acc, [&](int s, int mt) { return kfrag_read_s(pt, poff[mt], s); },
-            [&](int s, int j) { return kfrag_read_s(qt, qoff[j], s); });
+        auto read_p = [&](int s, int mt) { return kfrag_read_s(pt, poff[mt], s); };
+        auto read_q = [&](int s, int j) { return kfrag_read_s(qt, qoff[j], s); };
+        if constexpr (MT == 2) multiply_stage<MT, NTW>(acc, read_p, read_q);
+        else multiply_stage_tall<MT, NTW, 2>(acc, read_p, read_q);
       }
     };
-    for (int i = 0; i < nstages; i += 4) {
-      step(integral_constant<int, 0>{}, integral_constant<int, 3>{}, i);
-      step(integral_constant<int, 1>{}, integral_constant<int, 0>{}, i + 1);
-      step(integral_constant<int, 2>{}, integral_constant<int, 1>{}, i + 2);
-      step(integral_constant<int, 3>{}, integral_constant<int, 2>{}, i + 3);
+    for (int i = 0; i < nstages; i += R) {
+      step(integral_constant<int, 0>{}, i);
+      step(integral_constant<int, 1>{}, i + 1);
+      step(integral_constant<int, 2>{}, i + 2);
+      if constexpr (R == 4) step(integral_constant<int, 3>{}, i + 3);
     }
     __builtin_amdgcn_s_waitcnt(0);       // the repeated requests of the last steps land before the workgroup ends
   }
