@@ -214,18 +214,8 @@ __global__ __launch_bounds__(256) void act_bwd_kernel(const bf16_t* __restrict__
     for (int i = threadIdx.x; i < n_zero_words; i += 256) zero_words[i] = 0u;
   const int lane = threadIdx.x & 63;
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (row >= S || row >= offsets[E]) return;                   // E = GLU experts: rows behind theirs have no activation
-  int e = 0;
-  {                                                            // expert of the row: offsets[e] <= row < offsets[e + 1]
-    int lo = 0, hi = E;
-    while (hi - lo > 1) {
-      const int mid = (lo + hi) >> 1;
-      if (offsets[mid] <= row) lo = mid; else hi = mid;
-    }
-    e = lo;
-  }
-  const int slot = perm_slot[row];
-  const float ws = w[slot];
+  if (row >= S) return;
+  // the row's values are requested first: nothing below that decides about the row depends on them
   const bool live = lane * 8 < I;
   bf16x8 gv, uv, dv;
 #pragma unroll
@@ -235,6 +225,13 @@ __global__ __launch_bounds__(256) void act_bwd_kernel(const bf16_t* __restrict__
     uv = *reinterpret_cast<const bf16x8*>(gu + (size_t)row * 2 * I + I + lane * 8);
     dv = *reinterpret_cast<const bf16x8*>(dhp + (size_t)row * I + lane * 8);
   }
+  const int slot = perm_slot[row];
+  // expert of the row: offsets[e] <= row < offsets[e + 1], one offset per lane (E <= 64) and a ballot
+  const int my_off = offsets[min(lane, E)];
+  const int end = E < kWave ? __shfl(my_off, E, kWave) : offsets[E];
+  if (row >= end) return;                                      // E = GLU experts: rows behind theirs have no activation
+  const int e = __popcll(__ballot(lane < E && my_off <= row)) - 1;
+  const float ws = w[slot];
   float g[8], u[8], d[8];
   float ss = 0.f;
 #pragma unroll
