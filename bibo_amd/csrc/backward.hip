@@ -490,8 +490,12 @@ hipError_t launch_backward(const void* x, const void* d_out, const void* w_route
     zero_bytes(d_wd, (size_t)E * H * I * sizeof(bf16_t), s);
     return hipGetLastError();
   }
-  // pre-activations again (moe.py:84): x W_gate_up^T, both contiguous along H
-  err = launch_ggemm<true, false>(xp, perm_token, wgup, offsets, nullptr, S, H, 2 * I, E, gu, s);
+  // pre-activations again (moe.py:84): x W_gate_up^T, both contiguous along H - by the first phase of the forward
+  // pass's fused kernel where it takes the shape (its ring of weight stages is the faster main loop)
+  if (fused_supported(H, I, BIBO_DTYPE_BF16) && (long long)T * H < (1LL << 31))
+    err = launch_gateup_raw(xp, wgup, offsets, perm_token, T, H, E, k, I, gu, s);
+  else
+    err = launch_ggemm<true, false>(xp, perm_token, wgup, offsets, nullptr, S, H, 2 * I, E, gu, s);
   if (err != hipSuccess) return err;
   // dh' = d W_down: contracts over H, the middle dimension of w_down [E, H, I]
   err = launch_dgrad<true, false>(dop, perm_token, wdp, offsets, nullptr, S, H, I, E, dhp, s);

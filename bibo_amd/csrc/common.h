@@ -202,6 +202,8 @@ hipError_t launch_down_mfma(const void* hidden, const void* wd, const float* w, 
                             const int32_t* perm_slot, int T, int H, int E, int k, int I, void* yw, hipStream_t s);
 
 bool fused_supported(int H, int I, int dtype);
+hipError_t launch_gateup_raw(const void* x, const void* wgu, const int32_t* offsets, const int32_t* perm_token, int T, int H,
+                             int E, int k, int I, void* gu, hipStream_t s);
 hipError_t launch_experts_fused(const void* x, const void* wgu, const void* wd, const float* theta, const float* w,
                                 const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token, int T,
                                 int H, int E, int k, int I, int act, void* yw, hipStream_t s);

@@ -123,7 +123,9 @@ __device__ __forceinline__ bf16x8 to_operand_lanes(bf16x8 v, int sel) {
   return __builtin_bit_cast(bf16x8, u);
 }
 
-template <int NT, int CT>
+// RAW: the backward pass's recomputation.  The kernel stops after phase 1 and writes the pre-activations themselves,
+// rounded to bf16, to rows row0 .. of `yw`, which then is [S, 2I] in permuted row order (gate columns, then up columns).
+template <int NT, int CT, bool RAW = false>
 __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wgu,
                                                             const bf16_t* __restrict__ wd,
                                                             const float* __restrict__ theta,
@@ -261,6 +263,46 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
     else kloop(integral_constant<int, 0>{});
   }
   wait_loads_and_sync();                   // every transfer has landed and every wave is done with the stages
+
+  if constexpr (RAW) {
+    // gate half, then up half: accumulators -> the stages in the activation layout (stage t = columns [128 t, 128 t + 128)
+    // of the half, granule c of row m at c ^ (m & 15)) -> whole 256-byte row segments to memory
+    const int hh = lane >> 5;
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        if (mt >= my_blocks) continue;
+        const int m = mbase + mt * 32 + n;
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+          const int tile32 = wn * NT + j;
+          bf16_t* hrow = ((tile32 >> 2) == 0 ? S0 : ((tile32 >> 2) == 1 ? S1 : S2)) + m * 128 + 4 * hh;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            bf16x4 hv;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) hv[r] = (bf16_t)acc[mt][half * NT + j][4 * q + r];
+            const int c = (tile32 & 3) * 4 + q;
+            *reinterpret_cast<bf16x4*>(hrow + (c ^ (m & 15)) * 8) = hv;
+          }
+        }
+      }
+      __syncthreads();
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        const bf16_t* slice = t == 0 ? S0 : (t == 1 ? S1 : S2);
+        for (int g = tid; g < BM * 16; g += 512) {
+          const int m = g >> 4, pos = g & 15;
+          if (m < rows)
+            *reinterpret_cast<u32x4*>(yw + (size_t)(row0 + m) * (2 * I) + half * I + t * 128 + ((pos ^ (m & 15)) * 8)) =
+                *reinterpret_cast<const u32x4*>(slice + m * 128 + pos * 8);
+        }
+      }
+      __syncthreads();                     // the stages are free for the other half
+    }
+    return;
+  }
 
   // ---- phase 2: Radial NormSiLU (moe.py:87-92), activations to LDS ----
   // The accumulators are transposed (lane = row mbase + 32*mt + n, register i = column acc_row(i, lane) of
@@ -461,7 +503,35 @@ void launch_fused_nt(const bf16_t* x, const bf16_t* wgu, const bf16_t* wd, const
   else launch_fused_t<NT, 1>(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, S, H, E, act, x_bytes, yw, s);
 }
 
+template <int NT>
+void launch_raw_nt(const bf16_t* x, const bf16_t* wgu, const int32_t* offsets, const int32_t* perm_token, int S, int H, int E,
+                   unsigned x_bytes, bf16_t* gu, hipStream_t s) {
+  const int grid = ((S / 128 + E + 7) & ~7) + 8;
+  hipLaunchKernelGGL((experts_fused_kernel<NT, 1, true>), dim3(grid), dim3(512), 0, s, x, wgu, nullptr, nullptr, nullptr,
+                     offsets, nullptr, perm_token, H, E, 0, x_bytes, gu);
+}
+
 }  // namespace
+
+// Phase 1 of the fused kernel alone: gu[row] = [x W_gate^T, x W_up^T] in bf16 for every permuted row (what the backward
+// pass recomputes, moe.py:84).  Same shapes as launch_experts_fused.
+hipError_t launch_gateup_raw(const void* x, const void* wgu, const int32_t* offsets, const int32_t* perm_token, int T, int H,
+                             int E, int k, int I, void* gu, hipStream_t s) {
+  const int S = T * k;
+  if (S == 0) return hipSuccess;
+  if ((unsigned long long)T * H * sizeof(bf16_t) >= (1ull << 32)) return hipErrorInvalidValue;
+  const unsigned xb = (unsigned)((size_t)T * H * sizeof(bf16_t));
+  const bf16_t* xp = static_cast<const bf16_t*>(x);
+  const bf16_t* gp = static_cast<const bf16_t*>(wgu);
+  bf16_t* out = static_cast<bf16_t*>(gu);
+  switch (I) {
+    case 128: launch_raw_nt<1>(xp, gp, offsets, perm_token, S, H, E, xb, out, s); break;
+    case 256: launch_raw_nt<2>(xp, gp, offsets, perm_token, S, H, E, xb, out, s); break;
+    case 384: launch_raw_nt<3>(xp, gp, offsets, perm_token, S, H, E, xb, out, s); break;
+    default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
 
 bool fused_supported(int H, int I, int dtype) {
   // the activation tile plus two weight stages have to fit 160 KB of LDS: I <= 384
