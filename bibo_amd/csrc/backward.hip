@@ -333,24 +333,36 @@ __global__ __launch_bounds__(256) void dtheta_reduce_kernel(const float* __restr
 }
 
 // ---- router backward (router.py:31,41-47) --------------------------------------------------------------------
-// One thread per token: dlogit of the k selected experts from the gradients of the combine weights.
-__global__ void router_bwd_kernel(const float* __restrict__ logits, const int32_t* __restrict__ idx,
-                                  const float* __restrict__ w, const float* __restrict__ dw, int T, int E, int k,
-                                  int norm_mode, float* __restrict__ dl) {
-  const int t = blockIdx.x * blockDim.x + threadIdx.x;
-  if (t >= T) return;
-  float s[kMaxK], sum = 0.f, dot = 0.f;
-  for (int j = 0; j < k; ++j) {
-    s[j] = 1.f / (1.f + __expf(-logits[(size_t)t * E + idx[t * k + j]]));
-    sum += s[j];
-    dot = fmaf(dw[t * k + j], w[t * k + j], dot);
+// Eight lanes per token, lane j < k for slot j: dlogit of the k selected experts from the gradients of the combine
+// weights.  The sums over a token's slots are taken in ascending j by every lane, so they are the same bits in all.
+__global__ __launch_bounds__(256) void router_bwd_kernel(const float* __restrict__ logits, const int32_t* __restrict__ idx,
+                                                         const float* __restrict__ w, const float* __restrict__ dw, int T,
+                                                         int E, int k, int norm_mode, float* __restrict__ dl) {
+  static_assert(kMaxK <= 8, "eight lanes per token");
+  const int gid = blockIdx.x * blockDim.x + threadIdx.x;
+  const int t = gid >> 3, j = gid & 7;
+  const bool live = t < T && j < k;
+  float sj = 0.f, dwj = 0.f, wj = 0.f;
+  if (live) {
+    sj = 1.f / (1.f + __expf(-logits[(size_t)t * E + idx[t * k + j]]));
+    dwj = dw[t * k + j];
+    wj = w[t * k + j];
   }
-  for (int j = 0; j < k; ++j) {
-    float ds = dw[t * k + j];
-    if (k > 1 && norm_mode == BIBO_NORM_SUM) ds = (ds - dot) / (sum + 1e-20f);
-    else if (k > 1 && norm_mode == BIBO_NORM_SOFTMAX) ds = w[t * k + j] * (ds - dot);
-    dl[t * k + j] = ds * s[j] * (1.f - s[j]);
+  const int base = (threadIdx.x & 63) & ~7;
+  float sum = 0.f, dot = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float si = __shfl(sj, base + i, kWave), di = __shfl(dwj, base + i, kWave), wi = __shfl(wj, base + i, kWave);
+    if (i < k) {
+      sum += si;
+      dot = fmaf(di, wi, dot);
+    }
   }
+  if (!live) return;
+  float ds = dwj;
+  if (k > 1 && norm_mode == BIBO_NORM_SUM) ds = (ds - dot) / (sum + 1e-20f);
+  else if (k > 1 && norm_mode == BIBO_NORM_SOFTMAX) ds = wj * (ds - dot);
+  dl[t * k + j] = ds * sj * (1.f - sj);
 }
 
 // dx[t, c] = sum_j dxs[t k + j, c] + sum_j dl[t, j] W_router[idx[t, j], c]; one thread per 8 columns.  dl == NULL: the
@@ -512,7 +524,7 @@ hipError_t launch_backward(const void* x, const void* d_out, const void* w_route
                        n_pos, n_neg, H, b.dw_slot, dxs);
   const bool with_router = w_router != nullptr;      // else: the experts alone, the caller owns the routing
   if (with_router)
-    hipLaunchKernelGGL(router_bwd_kernel, dim3((T + 255) / 256), dim3(256), 0, s, logits, idx, w, b.dw_slot, T, Et, k, norm_mode,
+    hipLaunchKernelGGL(router_bwd_kernel, dim3((T + 31) / 32), dim3(256), 0, s, logits, idx, w, b.dw_slot, T, Et, k, norm_mode,
                        b.dl);
   hipLaunchKernelGGL(dx_combine_kernel, dim3((unsigned)(((long long)T * (H / 8) + 255) / 256)), dim3(256), 0, s, dxs,
                      with_router ? b.dl : nullptr, idx, wrp, T, H, k, Et, b.dw_slot, static_cast<bf16_t*>(dx));
