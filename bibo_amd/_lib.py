@@ -23,6 +23,7 @@ SYMBOLS = (
     "bibo_moe_permute", "bibo_moe_gateup_fwd", "bibo_moe_down_combine_fwd", "bibo_moe_gateup_down_fwd",
     "bibo_moe_combine_fwd", "bibo_moe_combine_ex_fwd", "bibo_moe_experts_fwd", "bibo_moe_forward", "bibo_moe_rmsnorm_fwd",
     "bibo_moe_ffn_workspace_bytes", "bibo_moe_ffn_forward", "bibo_moe_forward_static", "bibo_moe_backward_workspace_bytes", "bibo_moe_backward", "bibo_moe_experts_backward",
+    "bibo_moe_train_state_bytes", "bibo_moe_forward_train", "bibo_moe_backward_saved",
     "bibo_moe_exp_attn_res_fwd",
 )
 STATIC_SCRATCH_BYTES = 16 << 20
@@ -78,6 +79,13 @@ def _declare(l):
     l.bibo_moe_backward.argtypes = [vp, vp, vp, vp, vp, vp, vp, ctypes.POINTER(Shape), ci, vp, vp, vp, vp, vp, vp, vp, sz, vp]
     l.bibo_moe_experts_backward.restype = ci
     l.bibo_moe_experts_backward.argtypes = [vp, vp, vp, vp, vp, vp, vp, ctypes.POINTER(Shape), vp, vp, vp, vp, vp, vp, sz, vp]
+    l.bibo_moe_train_state_bytes.restype = ci
+    l.bibo_moe_train_state_bytes.argtypes = [ctypes.POINTER(Shape), ctypes.POINTER(sz)]
+    l.bibo_moe_forward_train.restype = ci
+    l.bibo_moe_forward_train.argtypes = [vp, vp, vp, vp, vp, vp, ctypes.POINTER(Shape), ci, vp, vp, vp, sz, vp, sz, vp]
+    l.bibo_moe_backward_saved.restype = ci
+    l.bibo_moe_backward_saved.argtypes = [vp, vp, vp, vp, vp, vp, ctypes.POINTER(Shape), ci, vp, sz, vp, vp, vp, vp, vp, vp, vp,
+                                          sz, vp]
     l.bibo_moe_exp_attn_res_fwd.restype = ci
     l.bibo_moe_exp_attn_res_fwd.argtypes = [vp, ci, vp, ctypes.c_float, ci, ci, ci, vp, vp]
     l.bibo_moe_forward_static.argtypes = [vp, vp, vp, vp, vp, vp, ctypes.POINTER(Shape), ci, ci, vp, vp, vp, vp, vp, vp]

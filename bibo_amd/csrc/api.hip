@@ -168,7 +168,8 @@ int down_dispatch(const void* hidden, const void* wd, const float* w, const int3
 int experts_dispatch(const void* x, const void* wgu, const void* wd, const float* theta, const int32_t* idx,
                      const float* w, const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token,
                      const void* residual, bool idx_trusted, int T, int H, int Eg, int np, int nn, int k, int I, int dtype,
-                     int algo, int act, int flags, void* out, char* base, const Workspace& ws, hipStream_t s) {
+                     int algo, int act, int flags, void* out, char* base, const Workspace& ws, hipStream_t s,
+                     void* preact = nullptr) {
   float* yw = reinterpret_cast<float*>(base + ws.yw);
   CombineArgs ca;
   ca.residual = residual;
@@ -188,13 +189,34 @@ int experts_dispatch(const void* x, const void* wgu, const void* wd, const float
   }
   if (algo == BIBO_ALGO_FUSED) {
     if (!aligned16(x) || !aligned16(wgu) || !aligned16(wd)) return BIBO_ERR_MISALIGNED;
-    hipError_t e = launch_experts_fused(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, T, H, Eg, k, I, act, yw, s);
+    hipError_t e = launch_experts_fused(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, T, H, Eg, k, I, act, yw, preact, s);
     if (e != hipSuccess) return (int)e;
     return hip_rc(launch_combine(yw, 1, ca, T, H, k, dtype, out, s));
   }
   const int rc = gateup_dispatch(x, wgu, theta, offsets, perm_token, T, H, Eg, k, I, dtype, algo, act, base + ws.hidden, s);
   if (rc != BIBO_OK) return rc;
   return down_dispatch(base + ws.hidden, wd, w, offsets, perm_slot, ca, T, H, Eg, k, I, dtype, algo, out, yw, s);
+}
+
+// What a training forward leaves for its backward pass in a caller-owned buffer: the routing (selection, combine
+// weights, fp32 logits), the permutation and the bf16 gate/up pre-activations of every routed row.
+struct TrainState {
+  size_t idx, w, logits, offsets, perm_slot, perm_token, gu, total;
+};
+
+TrainState carve_state(int T, int E, int k, int I) {
+  const size_t S = (size_t)T * k;
+  TrainState st;
+  size_t o = 0;
+  st.idx = o;        o += align_up(S * sizeof(int32_t));
+  st.w = o;          o += align_up(S * sizeof(float));
+  st.logits = o;     o += align_up((size_t)T * E * sizeof(float));
+  st.offsets = o;    o += align_up((kMaxE + 1) * sizeof(int32_t));
+  st.perm_slot = o;  o += align_up(S * sizeof(int32_t));
+  st.perm_token = o; o += align_up(S * sizeof(int32_t));
+  st.gu = o;         o += align_up(S * 2 * (size_t)I * sizeof(bf16_t));
+  st.total = o;
+  return st;
 }
 
 // The whole layer on `x`; `residual` (or NULL) is added in the combine.  With `norm_src` given, `x` is a buffer the
@@ -204,7 +226,7 @@ int forward_impl(const void* x, const void* w_router, const float* bias, const v
                  const float* theta, const bibo_moe_shape* sh, int norm_mode, int algo, const void* residual, void* out,
                  int32_t* idx_out, float* w_out, int32_t* counts_out, float* logits_out, void* workspace,
                  size_t workspace_bytes, void* stream, const void* norm_src = nullptr, const float* norm_weight = nullptr,
-                 float eps = 0.f) {
+                 float eps = 0.f, char* state = nullptr) {
   if (sh == nullptr) return BIBO_ERR_NULL_POINTER;
   const int T = sh->T, H = sh->H, E = sh->E, k = sh->k, I = sh->I, dtype = sh->dtype;
   int rc = check_dims(T, H, E, k, I, dtype, sh->n_pos, sh->n_neg);
@@ -227,6 +249,17 @@ int forward_impl(const void* x, const void* w_router, const float* bias, const v
   int32_t* offsets = reinterpret_cast<int32_t*>(base + ws.offsets);
   int32_t* perm_slot = reinterpret_cast<int32_t*>(base + ws.perm_slot);
   int32_t* perm_token = reinterpret_cast<int32_t*>(base + ws.perm_token);
+  void* preact = nullptr;
+  if (state != nullptr) {                // a training forward: what the backward pass needs lands in the caller's state buffer
+    const TrainState st = carve_state(T, E, k, I);
+    idx = reinterpret_cast<int32_t*>(state + st.idx);
+    w = reinterpret_cast<float*>(state + st.w);
+    logits_out = reinterpret_cast<float*>(state + st.logits);
+    offsets = reinterpret_cast<int32_t*>(state + st.offsets);
+    perm_slot = reinterpret_cast<int32_t*>(state + st.perm_slot);
+    perm_token = reinterpret_cast<int32_t*>(state + st.perm_token);
+    preact = state + st.gu;
+  }
   // the streaming kernels find their rows themselves; the permutation then only serves the counts
   const bool need_permute = a != BIBO_ALGO_STREAM || counts_out != nullptr || T == 0;
   // the router kernel can leave per-workgroup histograms of its selections, which save the permutation its
@@ -250,7 +283,7 @@ int forward_impl(const void* x, const void* w_router, const float* bias, const v
   }
   if (T == 0) return BIBO_OK;
   return experts_dispatch(x, w_gate_up, w_down, theta, idx, w, offsets, perm_slot, perm_token, residual, true, T, H, Eg,
-                          sh->n_pos, sh->n_neg, k, I, dtype, a, sh->act, sh->flags, out, base, ws, s);
+                          sh->n_pos, sh->n_neg, k, I, dtype, a, sh->act, sh->flags, out, base, ws, s, preact);
 }
 
 
@@ -327,6 +360,71 @@ int backward_check(const bibo_moe_shape* sh, int norm_mode) {
   return BIBO_OK;
 }
 
+
+// The MFMA backward family behind bibo_moe_backward and bibo_moe_backward_saved.  `state` (or NULL): what a training
+// forward kept (routing, permutation, pre-activations); without it the routing and the permutation are computed again
+// from x - same kernels, same inputs, hence the same selection and weights - and so are the pre-activations.
+int backward_mfma(const void* x, const void* d_out, const void* w_router, const float* bias, const void* w_gate_up,
+                  const void* w_down, const float* theta, const bibo_moe_shape* sh, int norm_mode, const char* state, void* d_x,
+                  void* d_w_router, void* d_w_gate_up, void* d_w_down, float* d_theta, float* d_w_out, void* workspace,
+                  size_t workspace_bytes, void* stream) {
+  const int T = sh->T, H = sh->H, E = sh->E, k = sh->k, I = sh->I;
+  int rc;
+  if (!aligned16(x) || !aligned16(d_out) || !aligned16(w_router) || !aligned16(w_gate_up) || !aligned16(w_down) ||
+      !aligned16(d_x) || !aligned16(d_w_gate_up) || !aligned16(d_w_down))
+    return BIBO_ERR_MISALIGNED;
+  const BackwardWorkspace ws = carve_backward(T, H, E, k, I);
+  if (workspace_bytes < ws.total) return BIBO_ERR_WORKSPACE_TOO_SMALL;
+  char* base = static_cast<char*>(workspace);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int32_t* idx; const float* w; const float* logits; const int32_t* offsets; const int32_t* perm_slot;
+  const int32_t* perm_token; const void* gu_saved = nullptr;
+  if (state != nullptr) {
+    const TrainState st = carve_state(T, E, k, I);
+    idx = reinterpret_cast<const int32_t*>(state + st.idx);
+    w = reinterpret_cast<const float*>(state + st.w);
+    logits = reinterpret_cast<const float*>(state + st.logits);
+    offsets = reinterpret_cast<const int32_t*>(state + st.offsets);
+    perm_slot = reinterpret_cast<const int32_t*>(state + st.perm_slot);
+    perm_token = reinterpret_cast<const int32_t*>(state + st.perm_token);
+    gu_saved = state + st.gu;
+  } else {
+    int32_t* idx_w = reinterpret_cast<int32_t*>(base + ws.idx);
+    float* w_w = reinterpret_cast<float*>(base + ws.w);
+    float* logits_w = reinterpret_cast<float*>(base + ws.logits);
+    int32_t* counts = reinterpret_cast<int32_t*>(base + ws.counts);
+    int32_t* offsets_w = reinterpret_cast<int32_t*>(base + ws.offsets);
+    int32_t* slot_w = reinterpret_cast<int32_t*>(base + ws.perm_slot);
+    int32_t* token_w = reinterpret_cast<int32_t*>(base + ws.perm_token);
+    // (the router kernel leaves per-workgroup histograms of its selections for the permutation, as in the forward pass)
+    int32_t* hist = reinterpret_cast<int32_t*>(base + ws.hist);
+    int hist_tokens = 0;
+    const bool want_hist = T > 0 && permute_takes_router_hist(T, k);
+    if (T > 0 && (rc = hip_rc(launch_router(x, w_router, bias, T, H, E, k, sh->dtype, norm_mode, logits_w, idx_w, w_w, nullptr,
+                                            want_hist ? hist : nullptr, &hist_tokens, s))) != BIBO_OK)
+      return rc;
+    rc = hip_rc((want_hist && hist_tokens > 0)
+                    ? launch_permute_from_hist(idx_w, T, E, k, hist, hist_tokens, counts, offsets_w, slot_w, token_w, s)
+                    : launch_permute(idx_w, T, E, k, counts, offsets_w, slot_w, token_w, hist, s));
+    if (rc != BIBO_OK) return rc;
+    idx = idx_w; w = w_w; logits = logits_w; offsets = offsets_w; perm_slot = slot_w; perm_token = token_w;
+  }
+  BackwardBuffers b;
+  b.gu = base + ws.gu; b.dhp = base + ws.dhp; b.dgu = base + ws.dgu;
+  b.hidden = base + ws.hidden; b.dxs = base + ws.dxs; b.zrow = base + ws.zrow;
+  b.dw_slot = d_w_out ? d_w_out : reinterpret_cast<float*>(base + ws.dw_slot);
+  b.dl = reinterpret_cast<float*>(base + ws.dl);
+  b.dtheta_row = reinterpret_cast<float*>(base + ws.dtheta_row);
+  b.dwr_part = reinterpret_cast<float*>(base + ws.dwr_part);
+  return hip_rc(launch_backward(x, d_out, w_router, w_gate_up, w_down, theta, logits, idx, w, offsets, perm_slot, perm_token,
+                                T, H, E - sh->n_pos - sh->n_neg, sh->n_pos, sh->n_neg, k, I, norm_mode, sh->act, b, d_x,
+                                d_w_router, d_w_gate_up, d_w_down, d_theta, s, gu_saved));
+}
+
+// whether a shape has the training forward that keeps its state: the fused forward kernel and the MFMA backward both take it
+inline bool train_state_supported(const bibo_moe_shape* sh) {
+  return backward_fast(sh) && fused_supported(sh->H, sh->I, sh->dtype) && fused_fits(sh->T, sh->H);
+}
 
 }  // namespace
 
@@ -431,7 +529,7 @@ int bibo_moe_gateup_down_fwd(const void* x, const void* w_gate_up, const void* w
     return BIBO_ERR_NULL_POINTER;
   if (!aligned16(x) || !aligned16(w_gate_up) || !aligned16(w_down) || !aligned16(yw)) return BIBO_ERR_MISALIGNED;
   return hip_rc(launch_experts_fused(x, w_gate_up, w_down, theta, w, offsets, perm_slot, perm_token, T, H, E, k, I, act,
-                                     yw, static_cast<hipStream_t>(stream)));
+                                     yw, nullptr, static_cast<hipStream_t>(stream)));
 }
 
 int bibo_moe_combine_fwd(const void* yw, int yw_is_bf16, int T, int H, int k, int dtype, void* out, void* stream) {
@@ -605,42 +703,49 @@ int bibo_moe_backward(const void* x, const void* d_out, const void* w_router, co
                                           g_token, T, H, E - sh->n_pos - sh->n_neg, sh->n_pos, sh->n_neg, k, I, sh->dtype,
                                           norm_mode, sh->act, g, d_x, d_w_router, d_w_gate_up, d_w_down, d_theta, gs));
   }
-  if (!aligned16(x) || !aligned16(d_out) || !aligned16(w_router) || !aligned16(w_gate_up) || !aligned16(w_down) ||
-      !aligned16(d_x) || !aligned16(d_w_gate_up) || !aligned16(d_w_down))
-    return BIBO_ERR_MISALIGNED;
-  const BackwardWorkspace ws = carve_backward(T, H, E, k, I);
-  if (workspace_bytes < ws.total) return BIBO_ERR_WORKSPACE_TOO_SMALL;
-  char* base = static_cast<char*>(workspace);
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  int32_t* idx = reinterpret_cast<int32_t*>(base + ws.idx);
-  float* w = reinterpret_cast<float*>(base + ws.w);
-  float* logits = reinterpret_cast<float*>(base + ws.logits);
-  int32_t* counts = reinterpret_cast<int32_t*>(base + ws.counts);
-  int32_t* offsets = reinterpret_cast<int32_t*>(base + ws.offsets);
-  int32_t* perm_slot = reinterpret_cast<int32_t*>(base + ws.perm_slot);
-  int32_t* perm_token = reinterpret_cast<int32_t*>(base + ws.perm_token);
-  // the routing of the forward pass again: same kernel, same inputs, hence the same selection and weights
-  // (the router kernel leaves per-workgroup histograms of its selections for the permutation, as in the forward pass)
-  int32_t* hist = reinterpret_cast<int32_t*>(base + ws.hist);
-  int hist_tokens = 0;
-  const bool want_hist = T > 0 && permute_takes_router_hist(T, k);
-  if (T > 0 && (rc = hip_rc(launch_router(x, w_router, bias, T, H, E, k, sh->dtype, norm_mode, logits, idx, w, nullptr,
-                                          want_hist ? hist : nullptr, &hist_tokens, s))) != BIBO_OK)
-    return rc;
-  rc = hip_rc((want_hist && hist_tokens > 0)
-                  ? launch_permute_from_hist(idx, T, E, k, hist, hist_tokens, counts, offsets, perm_slot, perm_token, s)
-                  : launch_permute(idx, T, E, k, counts, offsets, perm_slot, perm_token, hist, s));
+  return backward_mfma(x, d_out, w_router, bias, w_gate_up, w_down, theta, sh, norm_mode, nullptr, d_x, d_w_router,
+                       d_w_gate_up, d_w_down, d_theta, d_w_out, workspace, workspace_bytes, stream);
+}
+
+int bibo_moe_train_state_bytes(const bibo_moe_shape* sh, size_t* bytes) {
+  if (bytes == nullptr) return BIBO_ERR_NULL_POINTER;
+  const int rc = backward_check(sh, BIBO_NORM_SUM);
   if (rc != BIBO_OK) return rc;
-  BackwardBuffers b;
-  b.gu = base + ws.gu; b.dhp = base + ws.dhp; b.dgu = base + ws.dgu;
-  b.hidden = base + ws.hidden; b.dxs = base + ws.dxs; b.zrow = base + ws.zrow;
-  b.dw_slot = d_w_out ? d_w_out : reinterpret_cast<float*>(base + ws.dw_slot);
-  b.dl = reinterpret_cast<float*>(base + ws.dl);
-  b.dtheta_row = reinterpret_cast<float*>(base + ws.dtheta_row);
-  b.dwr_part = reinterpret_cast<float*>(base + ws.dwr_part);
-  return hip_rc(launch_backward(x, d_out, w_router, w_gate_up, w_down, theta, logits, idx, w, offsets, perm_slot, perm_token,
-                                T, H, E - sh->n_pos - sh->n_neg, sh->n_pos, sh->n_neg, k, I, norm_mode, sh->act, b, d_x,
-                                d_w_router, d_w_gate_up, d_w_down, d_theta, s));
+  if (!train_state_supported(sh)) return BIBO_ERR_UNSUPPORTED;
+  *bytes = carve_state(sh->T, sh->E, sh->k, sh->I).total;
+  return BIBO_OK;
+}
+
+int bibo_moe_forward_train(const void* x, const void* w_router, const float* bias, const void* w_gate_up, const void* w_down,
+                           const float* theta, const bibo_moe_shape* sh, int norm_mode, void* out, int32_t* counts_out,
+                           void* state, size_t state_bytes, void* workspace, size_t workspace_bytes, void* stream) {
+  const int rc = backward_check(sh, norm_mode);
+  if (rc != BIBO_OK) return rc;
+  if (!train_state_supported(sh)) return BIBO_ERR_UNSUPPORTED;
+  if (state == nullptr) return BIBO_ERR_NULL_POINTER;
+  if (!aligned_ws(state)) return BIBO_ERR_MISALIGNED;
+  if (state_bytes < carve_state(sh->T, sh->E, sh->k, sh->I).total) return BIBO_ERR_WORKSPACE_TOO_SMALL;
+  return forward_impl(x, w_router, bias, w_gate_up, w_down, theta, sh, norm_mode, BIBO_ALGO_FUSED, nullptr, out, nullptr,
+                      nullptr, counts_out, nullptr, workspace, workspace_bytes, stream, nullptr, nullptr, 0.f,
+                      static_cast<char*>(state));
+}
+
+int bibo_moe_backward_saved(const void* x, const void* d_out, const void* w_router, const void* w_gate_up, const void* w_down,
+                            const float* theta, const bibo_moe_shape* sh, int norm_mode, const void* state,
+                            size_t state_bytes, void* d_x, void* d_w_router, void* d_w_gate_up, void* d_w_down,
+                            float* d_theta, float* d_w_out, void* workspace, size_t workspace_bytes, void* stream) {
+  const int rc = backward_check(sh, norm_mode);
+  if (rc != BIBO_OK) return rc;
+  if (!train_state_supported(sh)) return BIBO_ERR_UNSUPPORTED;
+  const int T = sh->T;
+  if (!workspace || !state) return BIBO_ERR_NULL_POINTER;
+  if (!aligned_ws(workspace) || !aligned_ws(state)) return BIBO_ERR_MISALIGNED;
+  if (state_bytes < carve_state(T, sh->E, sh->k, sh->I).total) return BIBO_ERR_WORKSPACE_TOO_SMALL;
+  if (!d_w_router || !d_w_gate_up || !d_w_down || !d_theta) return BIBO_ERR_NULL_POINTER;
+  if (T > 0 && (!x || !d_out || !w_router || !w_gate_up || !w_down || !d_x)) return BIBO_ERR_NULL_POINTER;
+  if (T > 0 && !theta && sh->act != BIBO_ACT_SILU) return BIBO_ERR_NULL_POINTER;
+  return backward_mfma(x, d_out, w_router, nullptr, w_gate_up, w_down, theta, sh, norm_mode, static_cast<const char*>(state),
+                       d_x, d_w_router, d_w_gate_up, d_w_down, d_theta, d_w_out, workspace, workspace_bytes, stream);
 }
 
 int bibo_moe_experts_backward(const void* x, const void* d_out, const int32_t* idx, const float* w, const void* w_gate_up,

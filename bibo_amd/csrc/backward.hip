@@ -479,7 +479,7 @@ hipError_t launch_backward(const void* x, const void* d_out, const void* w_route
                            const float* theta, const float* logits, const int32_t* idx, const float* w,
                            const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token, int T, int H, int E,
                            int n_pos, int n_neg, int k, int I, int norm_mode, int act, const BackwardBuffers& b, void* dx,
-                           void* d_w_router, void* d_wgu, void* d_wd, float* d_theta, hipStream_t s) {
+                           void* d_w_router, void* d_wgu, void* d_wd, float* d_theta, hipStream_t s, const void* gu_saved) {
   // E = GLU experts (with weights); the router and the permutation know Et experts, the +/-Identity ones last
   const int Et = E + n_pos + n_neg;
   const int S = T * k;
@@ -488,7 +488,8 @@ hipError_t launch_backward(const void* x, const void* d_out, const void* w_route
   const bf16_t* wrp = static_cast<const bf16_t*>(w_router);
   const bf16_t* wgup = static_cast<const bf16_t*>(wgu);
   const bf16_t* wdp = static_cast<const bf16_t*>(wd);
-  bf16_t* gu = static_cast<bf16_t*>(b.gu);
+  // the pre-activations: a training forward's, or recomputed below into the workspace
+  const bf16_t* gu = gu_saved != nullptr ? static_cast<const bf16_t*>(gu_saved) : static_cast<const bf16_t*>(b.gu);
   bf16_t* dhp = static_cast<bf16_t*>(b.dhp);
   bf16_t* dgu = static_cast<bf16_t*>(b.dgu);
   bf16_t* hidden = static_cast<bf16_t*>(b.hidden);
@@ -504,10 +505,12 @@ hipError_t launch_backward(const void* x, const void* d_out, const void* w_route
   }
   // pre-activations again (moe.py:84): x W_gate_up^T, both contiguous along H - by the first phase of the forward
   // pass's fused kernel where it takes the shape (its ring of weight stages is the faster main loop)
-  if (fused_supported(H, I, BIBO_DTYPE_BF16) && (long long)T * H < (1LL << 31))
-    err = launch_gateup_raw(xp, wgup, offsets, perm_token, T, H, E, k, I, gu, s);
+  if (gu_saved != nullptr)
+    err = hipSuccess;
+  else if (fused_supported(H, I, BIBO_DTYPE_BF16) && (long long)T * H < (1LL << 31))
+    err = launch_gateup_raw(xp, wgup, offsets, perm_token, T, H, E, k, I, b.gu, s);
   else
-    err = launch_ggemm<true, false>(xp, perm_token, wgup, offsets, nullptr, S, H, 2 * I, E, gu, s);
+    err = launch_ggemm<true, false>(xp, perm_token, wgup, offsets, nullptr, S, H, 2 * I, E, static_cast<bf16_t*>(b.gu), s);
   if (err != hipSuccess) return err;
   // dh' = d W_down: contracts over H, the middle dimension of w_down [E, H, I]
   err = launch_dgrad<true, false>(dop, perm_token, wdp, offsets, nullptr, S, H, I, E, dhp, s);

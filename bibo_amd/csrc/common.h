@@ -206,7 +206,7 @@ hipError_t launch_gateup_raw(const void* x, const void* wgu, const int32_t* offs
                              int E, int k, int I, void* gu, hipStream_t s);
 hipError_t launch_experts_fused(const void* x, const void* wgu, const void* wd, const float* theta, const float* w,
                                 const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token, int T,
-                                int H, int E, int k, int I, int act, void* yw, hipStream_t s);
+                                int H, int E, int k, int I, int act, void* yw, void* preact, hipStream_t s);
 bool stream_supported(int H, int I, int dtype);
 hipError_t launch_gateup_stream(const void* x, const void* wgu, const int32_t* idx, int T, int H, int E, int k, int I,
                                 void* gu, hipStream_t s);
@@ -242,6 +242,6 @@ hipError_t launch_backward(const void* x, const void* d_out, const void* w_route
                            const float* theta, const float* logits, const int32_t* idx, const float* w,
                            const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token, int T, int H, int E,
                            int n_pos, int n_neg, int k, int I, int norm_mode, int act, const BackwardBuffers& b, void* dx,
-                           void* d_w_router, void* d_wgu, void* d_wd, float* d_theta, hipStream_t s);
+                           void* d_w_router, void* d_wgu, void* d_wd, float* d_theta, hipStream_t s, const void* gu_saved = nullptr);
 
 }  // namespace bibo

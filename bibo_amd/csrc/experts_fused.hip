@@ -123,9 +123,12 @@ __device__ __forceinline__ bf16x8 to_operand_lanes(bf16x8 v, int sel) {
   return __builtin_bit_cast(bf16x8, u);
 }
 
-// RAW: the backward pass's recomputation.  The kernel stops after phase 1 and writes the pre-activations themselves,
-// rounded to bf16, to rows row0 .. of `yw`, which then is [S, 2I] in permuted row order (gate columns, then up columns).
-template <int NT, int CT, bool RAW = false>
+// MODE 0: the forward pass.  MODE 1: the backward pass's recomputation - the kernel stops after phase 1 and writes the
+// pre-activations themselves, rounded to bf16, to `preact` [S, 2I] in permuted row order (gate columns, then up
+// columns), staged through the LDS stages into whole row segments.  MODE 2: the training forward - the forward pass that
+// also leaves those pre-activations for its backward, in the same way (8-byte stores straight from the accumulator
+// registers during phase 2 were slower: 140 against 133 us at T = 8192).
+template <int NT, int CT, int MODE = 0>
 __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wgu,
                                                             const bf16_t* __restrict__ wd,
                                                             const float* __restrict__ theta,
@@ -133,7 +136,8 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
                                                             const int32_t* __restrict__ offsets,
                                                             const int32_t* __restrict__ perm_slot,
                                                             const int32_t* __restrict__ perm_token, int H, int E,
-                                                            int act, unsigned x_bytes, bf16_t* __restrict__ yw) {
+                                                            int act, unsigned x_bytes, bf16_t* __restrict__ yw,
+                                                            bf16_t* __restrict__ preact) {
   using F = FusedShape<NT, CT>;
   constexpr int MT = F::MT, BM = F::BM, I = F::I, BK = F::BK;
   // Every buffer that is read while LDS-DMA fills another is a variable of its own: the compiler orders a DMA
@@ -264,7 +268,7 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
   }
   wait_loads_and_sync();                   // every transfer has landed and every wave is done with the stages
 
-  if constexpr (RAW) {
+  if constexpr (MODE != 0) {
     // gate half, then up half: accumulators -> the stages in the activation layout (stage t = columns [128 t, 128 t + 128)
     // of the half, granule c of row m at c ^ (m & 15)) -> whole 256-byte row segments to memory
     const int hh = lane >> 5;
@@ -295,13 +299,13 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
         for (int g = tid; g < BM * 16; g += 512) {
           const int m = g >> 4, pos = g & 15;
           if (m < rows)
-            *reinterpret_cast<u32x4*>(yw + (size_t)(row0 + m) * (2 * I) + half * I + t * 128 + ((pos ^ (m & 15)) * 8)) =
+            *reinterpret_cast<u32x4*>(preact + (size_t)(row0 + m) * (2 * I) + half * I + t * 128 + ((pos ^ (m & 15)) * 8)) =
                 *reinterpret_cast<const u32x4*>(slice + m * 128 + pos * 8);
         }
       }
       __syncthreads();                     // the stages are free for the other half
     }
-    return;
+    if constexpr (MODE == 1) return;
   }
 
   // ---- phase 2: Radial NormSiLU (moe.py:87-92), activations to LDS ----
@@ -488,27 +492,31 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
 template <int NT, int CT>
 void launch_fused_t(const bf16_t* x, const bf16_t* wgu, const bf16_t* wd, const float* theta, const float* w,
                     const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token, int S, int H, int E,
-                    int act, unsigned x_bytes, bf16_t* yw, hipStream_t s) {
+                    int act, unsigned x_bytes, bf16_t* yw, bf16_t* preact, hipStream_t s) {
   const int grid = ((S / 128 + E + 7) & ~7) + 8;
-  hipLaunchKernelGGL((experts_fused_kernel<NT, CT>), dim3(grid), dim3(512), 0, s, x, wgu, wd, theta, w, offsets,
-                     perm_slot, perm_token, H, E, act, x_bytes, yw);
+  if (preact != nullptr)
+    hipLaunchKernelGGL((experts_fused_kernel<NT, CT, 2>), dim3(grid), dim3(512), 0, s, x, wgu, wd, theta, w, offsets,
+                       perm_slot, perm_token, H, E, act, x_bytes, yw, preact);
+  else
+    hipLaunchKernelGGL((experts_fused_kernel<NT, CT, 0>), dim3(grid), dim3(512), 0, s, x, wgu, wd, theta, w, offsets,
+                       perm_slot, perm_token, H, E, act, x_bytes, yw, preact);
 }
 
 template <int NT>
 void launch_fused_nt(const bf16_t* x, const bf16_t* wgu, const bf16_t* wd, const float* theta, const float* w,
                      const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token, int S, int H, int E,
-                     int act, unsigned x_bytes, bf16_t* yw, hipStream_t s) {
-  if (H % 384 == 0) launch_fused_t<NT, 3>(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, S, H, E, act, x_bytes, yw, s);
-  else if (H % 256 == 0) launch_fused_t<NT, 2>(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, S, H, E, act, x_bytes, yw, s);
-  else launch_fused_t<NT, 1>(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, S, H, E, act, x_bytes, yw, s);
+                     int act, unsigned x_bytes, bf16_t* yw, bf16_t* preact, hipStream_t s) {
+  if (H % 384 == 0) launch_fused_t<NT, 3>(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, S, H, E, act, x_bytes, yw, preact, s);
+  else if (H % 256 == 0) launch_fused_t<NT, 2>(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, S, H, E, act, x_bytes, yw, preact, s);
+  else launch_fused_t<NT, 1>(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, S, H, E, act, x_bytes, yw, preact, s);
 }
 
 template <int NT>
 void launch_raw_nt(const bf16_t* x, const bf16_t* wgu, const int32_t* offsets, const int32_t* perm_token, int S, int H, int E,
                    unsigned x_bytes, bf16_t* gu, hipStream_t s) {
   const int grid = ((S / 128 + E + 7) & ~7) + 8;
-  hipLaunchKernelGGL((experts_fused_kernel<NT, 1, true>), dim3(grid), dim3(512), 0, s, x, wgu, nullptr, nullptr, nullptr,
-                     offsets, nullptr, perm_token, H, E, 0, x_bytes, gu);
+  hipLaunchKernelGGL((experts_fused_kernel<NT, 1, 1>), dim3(grid), dim3(512), 0, s, x, wgu, nullptr, nullptr, nullptr,
+                     offsets, nullptr, perm_token, H, E, 0, x_bytes, nullptr, gu);
 }
 
 }  // namespace
@@ -540,7 +548,7 @@ bool fused_supported(int H, int I, int dtype) {
 
 hipError_t launch_experts_fused(const void* x, const void* wgu, const void* wd, const float* theta, const float* w,
                                 const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token, int T,
-                                int H, int E, int k, int I, int act, void* yw, hipStream_t s) {
+                                int H, int E, int k, int I, int act, void* yw, void* preact, hipStream_t s) {
   const int S = T * k;
   if (S == 0) return hipSuccess;
   if ((unsigned long long)T * H * sizeof(bf16_t) >= (1ull << 32)) return hipErrorInvalidValue;   // 32-bit byte offsets into x
@@ -549,10 +557,11 @@ hipError_t launch_experts_fused(const void* x, const void* wgu, const void* wd, 
   const bf16_t* gp = static_cast<const bf16_t*>(wgu);
   const bf16_t* dp = static_cast<const bf16_t*>(wd);
   bf16_t* yp = static_cast<bf16_t*>(yw);
+  bf16_t* pp = static_cast<bf16_t*>(preact);
   switch (I) {
-    case 128: launch_fused_nt<1>(xp, gp, dp, theta, w, offsets, perm_slot, perm_token, S, H, E, act, xb, yp, s); break;
-    case 256: launch_fused_nt<2>(xp, gp, dp, theta, w, offsets, perm_slot, perm_token, S, H, E, act, xb, yp, s); break;
-    case 384: launch_fused_nt<3>(xp, gp, dp, theta, w, offsets, perm_slot, perm_token, S, H, E, act, xb, yp, s); break;
+    case 128: launch_fused_nt<1>(xp, gp, dp, theta, w, offsets, perm_slot, perm_token, S, H, E, act, xb, yp, pp, s); break;
+    case 256: launch_fused_nt<2>(xp, gp, dp, theta, w, offsets, perm_slot, perm_token, S, H, E, act, xb, yp, pp, s); break;
+    case 384: launch_fused_nt<3>(xp, gp, dp, theta, w, offsets, perm_slot, perm_token, S, H, E, act, xb, yp, pp, s); break;
     default: return hipErrorInvalidValue;
   }
   return hipGetLastError();

@@ -28,15 +28,18 @@ def _wants_grad(*tensors) -> bool:
 
 
 class _MoELayerFn(torch.autograd.Function):
-    """The whole layer as one autograd node: forward = bibo_moe_forward, backward = bibo_moe_backward, which recomputes
-    the routing and the activations from the saved input, so nothing but the input rows is kept.  Gradients are what
-    autograd gives the reference's eager layer with the selection held fixed (moe.py:157-183); the balancing bias
-    gets none (router.py:38).  The per-expert row counts come out as a second, non-differentiable result.  `cd` is the
-    compute dtype: bf16 runs the MFMA backward where its tiles divide the sizes, anything else the generic kernels."""
+    """The whole layer as one autograd node.  Gradients are what autograd gives the reference's eager layer with the
+    selection held fixed (moe.py:157-183); the balancing bias gets none (router.py:38).  The per-expert row counts come
+    out as a second, non-differentiable result.  `cd` is the compute dtype: bf16 runs the MFMA backward where its tiles
+    divide the sizes, anything else the generic kernels.  Two ways through the library: with `keep` and a shape that
+    has the pair, forward = bibo_moe_forward_train, which leaves routing, permutation and pre-activations in a state
+    tensor (about 4 I bytes per routed slot), and backward = bibo_moe_backward_saved; otherwise forward =
+    bibo_moe_forward and backward = bibo_moe_backward, which computes all of that again from the saved input rows.
+    The gradients are the same bits either way."""
 
     @staticmethod
     def forward(ctx, x, w_router, w_gate_up, w_down, theta, bias, k, norm, act, algo, want_counts, n_pos=0, n_neg=0,
-                casts=None, cd=torch.bfloat16):
+                casts=None, cd=torch.bfloat16, keep=True):
         cast = lambda t, d: (t if t.dtype == d else t.to(d)).contiguous()
         xb = cast(x.detach(), cd)
         # `casts`: kernel-dtype copies of the three weight tensors the caller already holds (the layer's cast cache), so
@@ -47,9 +50,17 @@ class _MoELayerFn(torch.autograd.Function):
         # A private copy of the E selection biases: the layer's balancing step writes gate.bias in place later in the
         # same forward (update_bias), and the backward pass has to route with the values the forward saw.
         b = bias.detach().to(torch.float32).clone()
-        out, _, _, counts, _ = ops.moe_forward(xb, wr, b, gu, dn, th, k, norm=norm, algo=algo, want_counts=want_counts, act=act,
-                                               n_pos=n_pos, n_neg=n_neg)
-        ctx.save_for_backward(xb, wr, gu, dn, th, b)
+        T, H = xb.shape
+        state = None
+        if keep and algo in ("auto", "fused") and ops.train_state_bytes(T, H, wr.shape[0], k, gu.shape[1] // 2, cd, n_pos,
+                                                                        n_neg, act) is not None:
+            out, counts, state = ops.moe_forward_train(xb, wr, b, gu, dn, th, k, norm=norm, want_counts=want_counts, act=act,
+                                                       n_pos=n_pos, n_neg=n_neg)
+        else:
+            out, _, _, counts, _ = ops.moe_forward(xb, wr, b, gu, dn, th, k, norm=norm, algo=algo, want_counts=want_counts,
+                                                   act=act, n_pos=n_pos, n_neg=n_neg)
+        ctx.has_state = state is not None
+        ctx.save_for_backward(xb, wr, gu, dn, th, b, *((state,) if state is not None else ()))
         ctx.conf = (k, norm, act, n_pos, n_neg)
         ctx.in_dtypes = (x.dtype, w_router.dtype, w_gate_up.dtype, w_down.dtype, theta.dtype)
         if counts is None:
@@ -59,11 +70,16 @@ class _MoELayerFn(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, d_out, _d_counts):
-        xb, wr, gu, dn, th, b = ctx.saved_tensors
+        saved = ctx.saved_tensors                        # read once: activation checkpointing unpacks on access
+        xb, wr, gu, dn, th, b = saved[:6]
         k, norm, act, n_pos, n_neg = ctx.conf
         d = d_out.to(xb.dtype).contiguous()
-        grads = ops.moe_backward(xb, d, wr, b, gu, dn, th, k, norm=norm, act=act, n_pos=n_pos, n_neg=n_neg)[:5]
-        return tuple(g.to(dt) for g, dt in zip(grads, ctx.in_dtypes)) + (None,) * 10
+        if ctx.has_state:
+            grads = ops.moe_backward_saved(xb, d, wr, gu, dn, th, k, saved[6], norm=norm, act=act, n_pos=n_pos,
+                                           n_neg=n_neg)[:5]
+        else:
+            grads = ops.moe_backward(xb, d, wr, b, gu, dn, th, k, norm=norm, act=act, n_pos=n_pos, n_neg=n_neg)[:5]
+        return tuple(g.to(dt) for g, dt in zip(grads, ctx.in_dtypes)) + (None,) * 11
 
 
 class _ExpertsFn(torch.autograd.Function):
@@ -344,6 +360,10 @@ class BiBoMoELayer(nn.Module):
         self.register_buffer("accumulated_tpe", torch.zeros(config.num_routed_experts, dtype=torch.float))
         self._fwd_step = 0
         self._update_every = None
+        # Training forwards keep routing, permutation and gate/up pre-activations for their backward pass (about
+        # 4 * moe_intermediate_size bytes per routed slot until that backward has run), as autograd keeps the reference
+        # layer's activations; False makes the backward pass compute them again from the input rows instead.
+        self.keep_activations = True
         self.experts = BiBoFusedExperts(config)
         self.use_shared_expert = getattr(config, "use_shared_expert", False)
         self.shared_experts_list = nn.ModuleList()
@@ -445,7 +465,7 @@ class BiBoMoELayer(nn.Module):
         casts = (self.gate._cache.get("w", self.gate.gate_proj.weight, cd), gu, dn)
         out, counts = _MoELayerFn.apply(x, self.gate.gate_proj.weight, e.gate_up_proj, e.down_proj, e.radial_theta,
                                         self.gate.bias, self.num_experts_per_tok, self.gate.norm_topk_prob, e.act, e.algo,
-                                        want_counts, e.num_pos, e.num_neg, casts, cd)
+                                        want_counts, e.num_pos, e.num_neg, casts, cd, self.keep_activations)
         return out, (counts if want_counts else None)
 
     @_no_compile

@@ -328,6 +328,72 @@ def moe_backward(x, d_out, w_router, bias, w_gate_up, w_down, theta, k, norm="su
     return d_x, d_wr, d_gu, d_dn, d_theta, d_w
 
 
+def train_state_bytes(T, H, E, k, I, dtype, n_pos=0, n_neg=0, act="radial"):
+    """Size of the buffer a training forward keeps for its backward pass (bibo_moe_train_state_bytes), or None where the
+    shape has no such pair (anything but bf16 with H a multiple of 128 and I in {128, 256, 384})."""
+    sh = L.Shape(T, H, E, k, I, L.DTYPE_BF16 if dtype == torch.bfloat16 else L.DTYPE_F32, n_pos, n_neg, act_code(act), 0)
+    n = ctypes.c_size_t(0)
+    rc = L.lib().bibo_moe_train_state_bytes(ctypes.byref(sh), ctypes.byref(n))
+    return n.value if rc == 0 else None
+
+
+def moe_forward_train(x, w_router, bias, w_gate_up, w_down, theta, k, norm="sum", want_counts=False, n_pos=0, n_neg=0,
+                      act="radial"):
+    """bibo_moe_forward_train: the layer's forward that keeps routing, permutation and gate/up pre-activations in a
+    state tensor for moe_backward_saved.  -> out [T,H], counts int32 [E]|None, state (uint8)."""
+    T, H = x.shape
+    Eg, two_i, _ = w_gate_up.shape
+    E = Eg + n_pos + n_neg
+    I = two_i // 2
+    dc = _dtype_code(x)
+    _chk(x, "x"); _chk(w_router, "w_router", x.dtype, (E, H)); _chk(bias, "bias", torch.float32, (E,))
+    _chk(w_gate_up, "w_gate_up", x.dtype, (Eg, 2 * I, H)); _chk(w_down, "w_down", x.dtype, (Eg, H, I))
+    _chk(theta, "theta", torch.float32, (Eg,))
+    dev = x.device
+    nbytes = train_state_bytes(T, H, E, k, I, x.dtype, n_pos, n_neg, act)
+    if nbytes is None:
+        raise NotImplementedError("no state-keeping training forward for this shape; use moe_forward and moe_backward")
+    out = torch.empty(T, H, dtype=x.dtype, device=dev)
+    counts = torch.empty(E, dtype=torch.int32, device=dev) if want_counts else None
+    state = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=dev)
+    ws = workspace(dev, workspace_bytes(T, H, E, k, I, dc))
+    sh = L.Shape(T, H, E, k, I, dc, n_pos, n_neg, act_code(act), 0)
+    with torch.cuda.device(dev):
+        L.check(L.lib().bibo_moe_forward_train(_ptr(x), _ptr(w_router), _ptr(bias), _ptr(w_gate_up), _ptr(w_down), _ptr(theta),
+                                               ctypes.byref(sh), norm_mode(norm), _ptr(out), _ptr(counts), _ptr(state),
+                                               state.numel(), _ptr(ws), ws.numel(), _stream(dev)), "bibo_moe_forward_train")
+    return out, counts, state
+
+
+def moe_backward_saved(x, d_out, w_router, w_gate_up, w_down, theta, k, state, norm="sum", act="radial", want_dw=False,
+                       n_pos=0, n_neg=0):
+    """bibo_moe_backward_saved: moe_backward with the routing, the permutation and the pre-activations taken from the
+    state tensor of moe_forward_train on the same x and weights (same results, bit for bit)."""
+    T, H = x.shape
+    Eg, two_i, _ = w_gate_up.shape
+    E = Eg + n_pos + n_neg
+    I = two_i // 2
+    dc = _dtype_code(x)
+    _chk(x, "x"); _chk(d_out, "d_out", x.dtype, (T, H)); _chk(w_router, "w_router", x.dtype, (E, H))
+    _chk(w_gate_up, "w_gate_up", x.dtype, (Eg, 2 * I, H)); _chk(w_down, "w_down", x.dtype, (Eg, H, I))
+    _chk(theta, "theta", torch.float32, (Eg,)); _chk(state, "state", torch.uint8)
+    dev = x.device
+    d_x = torch.empty_like(x)
+    d_wr, d_gu, d_dn = torch.empty_like(w_router), torch.empty_like(w_gate_up), torch.empty_like(w_down)
+    d_theta = torch.empty(Eg, dtype=torch.float32, device=dev)
+    d_w = torch.empty(T, k, dtype=torch.float32, device=dev) if want_dw else None
+    sh = L.Shape(T, H, E, k, I, dc, n_pos, n_neg, act_code(act), 0)
+    nbytes = ctypes.c_size_t(0)
+    L.check(L.lib().bibo_moe_backward_workspace_bytes(ctypes.byref(sh), ctypes.byref(nbytes)), "bibo_moe_backward_workspace_bytes")
+    ws = workspace(dev, nbytes.value)
+    with torch.cuda.device(dev):
+        L.check(L.lib().bibo_moe_backward_saved(_ptr(x), _ptr(d_out), _ptr(w_router), _ptr(w_gate_up), _ptr(w_down),
+                                                _ptr(theta), ctypes.byref(sh), norm_mode(norm), _ptr(state), state.numel(),
+                                                _ptr(d_x), _ptr(d_wr), _ptr(d_gu), _ptr(d_dn), _ptr(d_theta), _ptr(d_w),
+                                                _ptr(ws), ws.numel(), _stream(dev)), "bibo_moe_backward_saved")
+    return d_x, d_wr, d_gu, d_dn, d_theta, d_w
+
+
 def experts_backward(x, d_out, idx, w, w_gate_up, w_down, theta, act="radial", n_pos=0, n_neg=0):
     """bibo_moe_experts_backward: gradients of experts_fwd for a caller-owned routing (idx int32 [T,k], w fp32 [T,k];
     expert ids Eg .. Eg+n_pos-1 are +Identity, the next n_neg -Identity, as in experts_fwd).

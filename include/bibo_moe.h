@@ -290,6 +290,28 @@ int bibo_moe_backward(const void* x, const void* d_out, const void* w_router, co
                       void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * The training forward that keeps what bibo_moe_backward would compute again: the layer of bibo_moe_forward
+ * (BiBoMoELayer.forward in training, src/modeling/ffn/moe.py:157-183) whose routing, permutation and bf16 gate/up
+ * pre-activations (moe.py:84) land in a caller-owned `state` buffer, and the backward pass that reads them there instead
+ * of running the router, the permutation and the gate/up projection a second time (about a fifth of bibo_moe_backward's
+ * time; the forward call grows by the copy-out of the pre-activations).  `state`: 256-byte aligned device memory of
+ * bibo_moe_train_state_bytes (about 4 I bytes per routed slot), untouched between the two calls; it belongs to ONE
+ * forward call, x and the weights must be the same in both calls.  out / counts_out as in bibo_moe_forward (kernel family
+ * fixed: the fused kernel); gradients, d_w_out and the workspace (bibo_moe_backward_workspace_bytes) as in
+ * bibo_moe_backward, whose results bibo_moe_backward_saved reproduces bit for bit.  Shapes: bf16, H a multiple of 128,
+ * I in {128, 256, 384}; BIBO_ERR_UNSUPPORTED otherwise (use bibo_moe_forward + bibo_moe_backward).  The reference keeps
+ * its activations through torch.autograd; this pair is that choice made explicit.
+ */
+int bibo_moe_train_state_bytes(const bibo_moe_shape* shape, size_t* bytes);
+int bibo_moe_forward_train(const void* x, const void* w_router, const float* bias, const void* w_gate_up, const void* w_down,
+                           const float* theta, const bibo_moe_shape* shape, int norm_mode, void* out, int32_t* counts_out,
+                           void* state, size_t state_bytes, void* workspace, size_t workspace_bytes, void* stream);
+int bibo_moe_backward_saved(const void* x, const void* d_out, const void* w_router, const void* w_gate_up, const void* w_down,
+                            const float* theta, const bibo_moe_shape* shape, int norm_mode, const void* state,
+                            size_t state_bytes, void* d_x, void* d_w_router, void* d_w_gate_up, void* d_w_down,
+                            float* d_theta, float* d_w_out, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Backward pass of the experts alone (what autograd derives for BiBoFusedExperts.forward, src/modeling/ffn/moe.py:46-101)
  * for a caller that owns the routing: idx int32 [T,k] (every entry a valid expert id) and w fp32 [T,k] as handed to
  * bibo_moe_experts_fwd.  d_w fp32 [T,k] is the gradient with respect to w (moe.py:93), through which the caller's own

@@ -149,6 +149,56 @@ def test_backward_of_a_few_tokens_and_of_none(H, I, dtype):
         assert float(g.float().abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("T,H,Eg,n_pos,n_neg,k,I,norm,act", [(700, 768, 5, 0, 0, 3, 384, "sum", "radial"),
+                                                              (300, 256, 6, 1, 1, 3, 128, "softmax", "tanh"),
+                                                              (37, 256, 64, 0, 0, 2, 128, "sum", "radial"),
+                                                              (1, 384, 8, 0, 0, 2, 256, False, "silu")])
+def test_training_forward_keeps_what_the_backward_would_recompute(T, H, Eg, n_pos, n_neg, k, I, norm, act):
+    """bibo_moe_forward_train gives the output of bibo_moe_forward with the fused kernels bit for bit, and
+    bibo_moe_backward_saved, reading routing, permutation and pre-activations from its state buffer, the gradients of
+    bibo_moe_backward bit for bit (tall and short tiles, +/-Identity experts, idle experts, one token)."""
+    E = Eg + n_pos + n_neg
+    p = O.make_inputs(T=T, H=H, E=Eg, k=k, I=I, theta="normal", seed=T + 1)
+    g = torch.Generator().manual_seed(T)
+    p["w_router"] = (torch.randn(E, H, generator=g) * 0.05).bfloat16()
+    p["bias"] = torch.rand(E, generator=g) * 0.02 - 0.01
+    d_out = torch.randn(T, H, generator=g).to(torch.bfloat16).to(DEV)
+    dev = lambda t: t.to(DEV)
+    x, wr, b, gu, dn, th = (dev(p[n]) for n in ("x", "w_router", "bias", "w_gate_up", "w_down", "theta"))
+    kw = dict(norm=norm, act=act, n_pos=n_pos, n_neg=n_neg)
+    ref_out, _, _, ref_counts, _ = ops.moe_forward(x, wr, b, gu, dn, th, k, algo="fused", want_counts=True, **kw)
+    ref = ops.moe_backward(x, d_out, wr, b, gu, dn, th, k, want_dw=True, **kw)
+    out, counts, state = ops.moe_forward_train(x, wr, b, gu, dn, th, k, want_counts=True, **kw)
+    ops.workspace(DEV, 1 << 20).fill_(0x7f)                            # nothing may be left over in the workspace
+    got = ops.moe_backward_saved(x, d_out, wr, gu, dn, th, k, state, want_dw=True, **kw)
+    torch.cuda.synchronize()
+    assert torch.equal(out, ref_out) and torch.equal(counts, ref_counts)
+    for a, r, name in zip(got, ref, ("x", "w_router", "w_gate_up", "w_down", "theta", "w")):
+        assert torch.equal(a, r), name
+
+
+def test_layer_trains_the_same_with_and_without_kept_activations():
+    """The module's two ways through the library (keep_activations) give the same output and gradients, and what has
+    no state-keeping pair (fp32, odd sizes) is reported as such instead of failing."""
+    assert ops.train_state_bytes(64, 256, 8, 2, 128, torch.float32) is None
+    assert ops.train_state_bytes(64, 200, 8, 2, 128, torch.bfloat16) is None
+    assert ops.train_state_bytes(64, 256, 8, 2, 512, torch.bfloat16) is None      # I = 512: MFMA backward, no fused forward
+    assert ops.train_state_bytes(64, 256, 8, 2, 128, torch.bfloat16) > 64 * 2 * 2 * 128 * 2
+    res = []
+    for keep in (True, False):
+        torch.manual_seed(5)
+        layer = _layer()
+        layer.keep_activations = keep
+        x = torch.randn(2, 400, 256, device=DEV, dtype=torch.bfloat16, requires_grad=True)   # 200 rows per expert: the fused kernel either way
+        out = layer(x)
+        out.float().square().sum().backward()
+        res.append((out.detach(), x.grad, {n: p_.grad for n, p_ in layer.named_parameters() if p_.grad is not None}))
+    (o1, g1, p1), (o2, g2, p2) = res
+    assert torch.equal(o1, o2) and torch.equal(g1, g2) and sorted(p1) == sorted(p2)
+    for n in p1:
+        assert torch.equal(p1[n], p2[n]), n
+
+
 def test_backward_is_linear_in_the_upstream_gradient():
     """Size-independent property at the full c2 shape: the gradients of 2 d are twice those of d (every path is linear
     in d_out), to bf16 rounding; and nothing is accumulated between calls."""
