@@ -152,11 +152,12 @@ def test_backward_of_a_few_tokens_and_of_none(H, I, dtype):
 @pytest.mark.parametrize("T,H,Eg,n_pos,n_neg,k,I,norm,act", [(700, 768, 5, 0, 0, 3, 384, "sum", "radial"),
                                                               (300, 256, 6, 1, 1, 3, 128, "softmax", "tanh"),
                                                               (37, 256, 64, 0, 0, 2, 128, "sum", "radial"),
-                                                              (1, 384, 8, 0, 0, 2, 256, False, "silu")])
+                                                              (1, 384, 8, 0, 0, 2, 256, False, "silu"),
+                                                              (0, 256, 8, 0, 0, 2, 128, "sum", "radial")])
 def test_training_forward_keeps_what_the_backward_would_recompute(T, H, Eg, n_pos, n_neg, k, I, norm, act):
     """bibo_moe_forward_train gives the output of bibo_moe_forward with the fused kernels bit for bit, and
     bibo_moe_backward_saved, reading routing, permutation and pre-activations from its state buffer, the gradients of
-    bibo_moe_backward bit for bit (tall and short tiles, +/-Identity experts, idle experts, one token)."""
+    bibo_moe_backward bit for bit (tall and short tiles, +/-Identity experts, idle experts, one token, no token)."""
     E = Eg + n_pos + n_neg
     p = O.make_inputs(T=T, H=H, E=Eg, k=k, I=I, theta="normal", seed=T + 1)
     g = torch.Generator().manual_seed(T)
