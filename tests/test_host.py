@@ -82,6 +82,36 @@ def test_argument_errors_are_reported_without_a_gpu():
         L.check(-4, "x")
 
 
+def test_training_pair_checks_its_arguments_without_a_gpu():
+    """bibo_moe_train_state_bytes / bibo_moe_forward_train / bibo_moe_backward_saved: which shapes have the pair, and the
+    errors found on the host before any launch."""
+    lib = L.lib()
+    n = ctypes.c_size_t(0)
+    ok = L.Shape(8192, 768, 64, 6, 384, L.DTYPE_BF16)
+    assert lib.bibo_moe_train_state_bytes(ctypes.byref(ok), ctypes.byref(n)) == 0
+    assert n.value >= 8192 * 6 * (2 * 384 * 2 + 16) + 8192 * 64 * 4      # pre-activations, routing, permutation, logits
+    assert lib.bibo_moe_train_state_bytes(ctypes.byref(ok), None) == -1
+    assert lib.bibo_moe_train_state_bytes(None, ctypes.byref(n)) == -1
+    for other in (L.Shape(64, 768, 64, 6, 384, L.DTYPE_F32), L.Shape(64, 1024, 64, 6, 512, L.DTYPE_BF16),
+                  L.Shape(64, 200, 8, 2, 128, L.DTYPE_BF16)):
+        assert lib.bibo_moe_train_state_bytes(ctypes.byref(other), ctypes.byref(n)) == -6
+        assert lib.bibo_moe_forward_train(None, None, None, None, None, None, ctypes.byref(other), 1, None, None, None, 0, None, 0,
+                                          None) == -6
+    assert lib.bibo_moe_forward_train(None, None, None, None, None, None, ctypes.byref(ok), 1, None, None, None, 0, None, 0,
+                                      None) == -1                                       # no state buffer
+    assert lib.bibo_moe_forward_train(None, None, None, None, None, None, ctypes.byref(ok), 7, None, None, None, 0, None, 0,
+                                      None) == -6                                       # no such normalisation mode
+    fake = ctypes.c_void_p(4096)                                                        # aligned, never dereferenced here
+    assert lib.bibo_moe_forward_train(None, None, None, None, None, None, ctypes.byref(ok), 1, None, None, fake, 256, None, 0,
+                                      None) == -4                                       # state buffer too small
+    assert lib.bibo_moe_backward_saved(None, None, None, None, None, None, ctypes.byref(ok), 1, None, 0, None, None, None, None,
+                                       None, None, None, 0, None) == -1
+    assert lib.bibo_moe_backward_saved(None, None, None, None, None, None, ctypes.byref(ok), 1, fake, 256, None, None, None, None,
+                                       None, None, fake, 0, None) == -4
+    assert lib.bibo_moe_backward_saved(None, None, None, None, None, None, ctypes.byref(ok), 1, ctypes.c_void_p(4100), 1 << 40,
+                                       None, None, None, None, None, None, fake, 0, None) == -5   # misaligned state
+
+
 def test_kernel_family_selection_is_exported():
     """bibo_moe_select_algo: what the composite calls run per workload, and which requests cannot be met."""
     from bibo_amd import ops
@@ -144,7 +174,7 @@ def test_state_dict_layout_matches_the_reference_layer():
         "accumulated_tpe": (8,), "gate.bias": (8,), "gate.gate_proj.weight": (8, 64),
         "experts.gate_up_proj": (8, 192, 64), "experts.down_proj": (8, 64, 96), "experts.radial_theta": (8,)}
     assert layer.gate.bias.requires_grad is False and layer.experts.radial_theta.requires_grad
-    assert float(layer.experts.radial_theta.abs().max()) == 0.0
+    assert float(layer.experts.radial_theta.detach().abs().max()) == 0.0
     e = layer.experts
     assert (e.pos_start, e.pos_end, e.neg_start, e.neg_end) == (8, 8, 8, 8)
     assert layer.gate.top_k == 2 and layer.gate.norm_topk_prob == "sum" and layer.gate._probe_gap is False
