@@ -289,7 +289,7 @@ int forward_impl(const void* x, const void* w_router, const float* bias, const v
 
 struct BackwardWorkspace {
   size_t hist, idx, w, logits, counts, offsets, perm_slot, perm_token, dw_slot, dl, dtheta_row, dwr_part, zrow, gu, dhp, dgu,
-      hidden, dxs, total;
+      hidden, dxs, wgrad_part, wgrad_plan, total;
 };
 
 BackwardWorkspace carve_backward(int T, int H, int E, int k, int I) {
@@ -315,6 +315,8 @@ BackwardWorkspace carve_backward(int T, int H, int E, int k, int I) {
   ws.dgu = o;        o += align_up(S * 2 * I * b);
   ws.hidden = o;     o += align_up(S * I * b);
   ws.dxs = o;        o += align_up(S * H * b);
+  ws.wgrad_part = o; o += align_up(backward_wgrad_part_bytes((int)S, H, E, I));
+  ws.wgrad_plan = o; o += align_up(backward_wgrad_plan_bytes((int)S, E));
   ws.total = o;
   return ws;
 }
@@ -416,6 +418,8 @@ int backward_mfma(const void* x, const void* d_out, const void* w_router, const 
   b.dl = reinterpret_cast<float*>(base + ws.dl);
   b.dtheta_row = reinterpret_cast<float*>(base + ws.dtheta_row);
   b.dwr_part = reinterpret_cast<float*>(base + ws.dwr_part);
+  b.wgrad_part = reinterpret_cast<float*>(base + ws.wgrad_part);
+  b.wgrad_plan = reinterpret_cast<int*>(base + ws.wgrad_plan);
   return hip_rc(launch_backward(x, d_out, w_router, w_gate_up, w_down, theta, logits, idx, w, offsets, perm_slot, perm_token,
                                 T, H, E - sh->n_pos - sh->n_neg, sh->n_pos, sh->n_neg, k, I, norm_mode, sh->act, b, d_x,
                                 d_w_router, d_w_gate_up, d_w_down, d_theta, s, gu_saved));
@@ -800,6 +804,8 @@ int bibo_moe_experts_backward(const void* x, const void* d_out, const int32_t* i
   b.dl = reinterpret_cast<float*>(base + ws.dl);
   b.dtheta_row = reinterpret_cast<float*>(base + ws.dtheta_row);
   b.dwr_part = reinterpret_cast<float*>(base + ws.dwr_part);
+  b.wgrad_part = reinterpret_cast<float*>(base + ws.wgrad_part);
+  b.wgrad_plan = reinterpret_cast<int*>(base + ws.wgrad_plan);
   return hip_rc(launch_backward(x, d_out, nullptr, w_gate_up, w_down, theta, nullptr, idx, w, offsets, perm_slot, perm_token,
                                 T, H, E - sh->n_pos - sh->n_neg, sh->n_pos, sh->n_neg, k, I, BIBO_NORM_SUM, sh->act, b, d_x,
                                 nullptr, d_w_gate_up, d_w_down, d_theta, s));

@@ -169,29 +169,30 @@ hipError_t launch_dgrad(const bf16_t* A, const int32_t* a_index, const bf16_t* W
 // dW[e] = P(rows of e)^T Q(rows of e), P [.., N] and Q [.., M] row-major (kmajor.h)
 template <int MT, bool GATHER_P, bool GATHER_Q>
 hipError_t launch_wgrad_t(const bf16_t* P, const bf16_t* Q, const int32_t* index, const int32_t* offsets, const bf16_t* zrow,
-                          int N, int M, int E, bf16_t* dW, hipStream_t s) {
+                          int N, int M, int S_rows, int E, const int* plan, float* part, bf16_t* dW, hipStream_t s) {
   const dim3 block(512);
-  auto grid = [&](int bn) { return dim3((unsigned)((E * (N / (64 * MT)) * (M / bn) + 7) & ~7)); };
+  const int slots = backward_wgrad_part_slots(S_rows, E);      // (the partial tiles of cut experts are added up by wgrad_reduce_kernel)
+  auto grid = [&](int bn) { return dim3((unsigned)((slots * (N / (64 * MT)) * (M / bn) + 7) & ~7)); };
   if (M % 384 == 0)
     hipLaunchKernelGGL((wgrad_kmajor_kernel<MT, 3, GATHER_P, GATHER_Q>), grid(384), block, 0, s, P, Q, index, offsets, zrow, N,
-                       M, E, dW);
+                       M, plan, part, dW);
   else if (M % 256 == 0)
     hipLaunchKernelGGL((wgrad_kmajor_kernel<MT, 2, GATHER_P, GATHER_Q>), grid(256), block, 0, s, P, Q, index, offsets, zrow, N,
-                       M, E, dW);
+                       M, plan, part, dW);
   else
     hipLaunchKernelGGL((wgrad_kmajor_kernel<MT, 1, GATHER_P, GATHER_Q>), grid(128), block, 0, s, P, Q, index, offsets, zrow, N,
-                       M, E, dW);
+                       M, plan, part, dW);
   return hipGetLastError();
 }
 
 // 256 rows of dW per workgroup where N allows and the experts have rows enough for the streams to matter
 template <bool GATHER_P, bool GATHER_Q>
 hipError_t launch_wgrad(const bf16_t* P, const bf16_t* Q, const int32_t* index, const int32_t* offsets, const bf16_t* zrow,
-                        int N, int M, int S_rows, int E, bf16_t* dW, hipStream_t s) {
+                        int N, int M, int S_rows, int E, const int* plan, float* part, bf16_t* dW, hipStream_t s) {
   const int bn = M % 384 == 0 ? 384 : (M % 256 == 0 ? 256 : 128);
   if (N % 256 == 0 && tall_tiles(S_rows, E, (long long)E * (N / 128) * (M / bn), (long long)E * (N / 256) * (M / bn)))
-    return launch_wgrad_t<4, GATHER_P, GATHER_Q>(P, Q, index, offsets, zrow, N, M, E, dW, s);
-  return launch_wgrad_t<2, GATHER_P, GATHER_Q>(P, Q, index, offsets, zrow, N, M, E, dW, s);
+    return launch_wgrad_t<4, GATHER_P, GATHER_Q>(P, Q, index, offsets, zrow, N, M, S_rows, E, plan, part, dW, s);
+  return launch_wgrad_t<2, GATHER_P, GATHER_Q>(P, Q, index, offsets, zrow, N, M, S_rows, E, plan, part, dW, s);
 }
 
 // ---- Radial NormSiLU backward (moe.py:87-92), one wave per permuted row ----------------------------------------
@@ -208,10 +209,14 @@ __global__ __launch_bounds__(256) void act_bwd_kernel(const bf16_t* __restrict__
                                                       const int32_t* __restrict__ perm_slot, int S, int E, int I, int act,
                                                       bf16_t* __restrict__ dgu, bf16_t* __restrict__ hidden,
                                                       float* __restrict__ dw_slot, float* __restrict__ dtheta_row,
-                                                      uint32_t* __restrict__ zero_words, int n_zero_words) {
-  // (the first workgroup also clears the row of zeros the weight-gradient kernels read past an expert's last row)
-  if (blockIdx.x == 0)
+                                                      uint32_t* __restrict__ zero_words, int n_zero_words,
+                                                      int* __restrict__ plan, int chunk, int slots) {
+  // (the first workgroup also clears the row of zeros the weight-gradient kernels read past an expert's last row and,
+  // with its first wave, lists the row chunks those kernels work through)
+  if (blockIdx.x == 0) {
     for (int i = threadIdx.x; i < n_zero_words; i += 256) zero_words[i] = 0u;
+    if (threadIdx.x < kWave) wgrad_plan(offsets, E, chunk, slots, plan);
+  }
   const int lane = threadIdx.x & 63;
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= S) return;
@@ -470,6 +475,20 @@ bool backward_supported(int H, int I, int k, int dtype) {
 int backward_dwr_split() { return kDwrSplit; }
 
 // a row of zeros as wide as the widest weight-gradient operand: what a K stage reads past an expert's last row
+// The weight-gradient GEMMs cut an expert with more rows than this into chunks (kmajor.h): one and a half times the
+// average, so that evenly routed tokens leave every expert in one piece, and at least 512.
+int backward_wgrad_chunk_rows(int S_rows, int E) {
+  const long long c = (3ll * S_rows / (2ll * E) + 31) & ~31ll;
+  return (int)(c < 512 ? 512 : c);
+}
+// chunks over all experts, at most: the fp32 partial tiles of the cut experts are numbered so
+int backward_wgrad_part_slots(int S_rows, int E) { return S_rows / backward_wgrad_chunk_rows(S_rows, E) + E; }
+size_t backward_wgrad_part_bytes(int S_rows, int H, int E, int I) {
+  return (size_t)backward_wgrad_part_slots(S_rows, E) * 3 * I * H * sizeof(float);      // dW_down's and dW_gate_up's
+}
+// the list of chunks (kmajor.h: WgradPlan): a header, a 16-byte entry per chunk and one per expert
+size_t backward_wgrad_plan_bytes(int S_rows, int E) { return 16 + (size_t)(backward_wgrad_part_slots(S_rows, E) + E) * 16; }
+
 size_t backward_zero_row_bytes(int H, int I) { return (size_t)(H > 2 * I ? H : 2 * I) * sizeof(bf16_t); }
 
 // The launches after routing and permutation.  Buffers (bf16 unless noted): gu [S,2I], dhp [S,I], dgu [S,2I],
@@ -517,7 +536,8 @@ hipError_t launch_backward(const void* x, const void* d_out, const void* w_route
   if (err != hipSuccess) return err;
   hipLaunchKernelGGL(act_bwd_kernel, dim3((S + 3) / 4), dim3(256), 0, s, gu, dhp, w, theta, offsets, perm_slot, S, E, I, act,
                      dgu, hidden, b.dw_slot, b.dtheta_row, reinterpret_cast<uint32_t*>(zrow),
-                     (int)(backward_zero_row_bytes(H, I) / 4));
+                     (int)(backward_zero_row_bytes(H, I) / 4), b.wgrad_plan, backward_wgrad_chunk_rows(S, E),
+                     backward_wgrad_part_slots(S, E));
   hipLaunchKernelGGL(dtheta_reduce_kernel, dim3(E), dim3(256), 0, s, b.dtheta_row, offsets, d_theta);
   // dx of every slot, in slot order: [dg, du] W_gate_up, contracts over the 2I rows of w_gate_up [E, 2I, H]
   err = launch_dgrad<false, true>(dgu, nullptr, wgup, offsets, perm_slot, S, 2 * I, H, E, dxs, s);
@@ -539,10 +559,15 @@ hipError_t launch_backward(const void* x, const void* d_out, const void* w_route
   }
   // weight gradients, contracted over each expert's rows: dW_down[e] = d^T (w h) (d gathered by token, `hidden`
   // already carries w), dW_gate_up[e] = [dg, du]^T x (x gathered by token)
-  err = launch_wgrad<true, false>(dop, hidden, perm_token, offsets, zrow, H, I, S, E, static_cast<bf16_t*>(d_wd), s);
+  err = launch_wgrad<true, false>(dop, hidden, perm_token, offsets, zrow, H, I, S, E, b.wgrad_plan, b.wgrad_part, static_cast<bf16_t*>(d_wd), s);
   if (err != hipSuccess) return err;
-  err = launch_wgrad<false, true>(dgu, xp, perm_token, offsets, zrow, 2 * I, H, S, E, static_cast<bf16_t*>(d_wgu), s);
+  float* part_gu = b.wgrad_part + (size_t)backward_wgrad_part_slots(S, E) * H * I;
+  err = launch_wgrad<false, true>(dgu, xp, perm_token, offsets, zrow, 2 * I, H, S, E, b.wgrad_plan, part_gu, static_cast<bf16_t*>(d_wgu), s);
   if (err != hipSuccess) return err;
+  // experts with so many rows that they were cut into chunks: their partial tiles added up in chunk order
+  hipLaunchKernelGGL(wgrad_reduce_kernel, dim3((unsigned)(((size_t)2 * I * H / 4 + 255) / 256)), dim3(256), 0, s, b.wgrad_part,
+                     part_gu, b.wgrad_plan, backward_wgrad_part_slots(S, E), H * I, 2 * I * H, static_cast<bf16_t*>(d_wd),
+                     static_cast<bf16_t*>(d_wgu));
   return hipGetLastError();
 }
 

@@ -290,11 +290,41 @@ __global__ __launch_bounds__(512) void dgrad_kmajor_kernel(const bf16_t* __restr
 // side and the expert's last row on the Q side (memory that is certainly finite, whatever the rows behind the
 // expert's hold).  One workgroup per (expert, 64 MT rows of dW, 128 NTW columns of dW); MT = 4 (256 rows) halves what
 // a workgroup streams of Q per row of dW, at 192 accumulator registers and a ring of three 40 KB stages.
+// An expert with more than `chunk` rows is cut into chunks of that many rows, each a workgroup of its own per tile of
+// dW, so that a few experts holding most of the rows do not leave a few workgroups with most of the work; such an
+// expert's chunks write fp32 partial tiles to `part` (one [N, M] slot per chunk, slots numbered over all experts'
+// chunks) and wgrad_reduce_kernel adds them in chunk order.  Experts of one chunk write dW directly.  The chunks are
+// listed once per backward pass by wgrad_plan (below), so that a workgroup finds its chunk with one load.
+struct WgradPlan {
+  int total;         // chunks over all experts
+  int n_cut;         // experts cut into more than one chunk
+  int pad[2];
+  // followed by int4 chunk[total] = {expert, first row, end row, chunks of that expert}
+  // and, from entry `slots` on, int4 cut[n_cut] = {expert, its first chunk, its chunks, 0}
+};
+
+// One wave: lane = expert.  `slots` = the capacity of the chunk list (backward_wgrad_part_slots).
+__device__ __forceinline__ void wgrad_plan(const int32_t* __restrict__ offsets, int E, int chunk, int slots, int* __restrict__ plan) {
+  const int lane = lane_id();
+  int lo = 0, hi = 0;
+  if (lane < E) { lo = offsets[lane]; hi = offsets[lane + 1]; }
+  const int mine = lane < E ? max(1, (hi - lo + chunk - 1) / chunk) : 0;   // an idle expert keeps one (empty) chunk: its zero gradient
+  const int incl = wave_inclusive_scan(mine);
+  const int first = incl - mine;
+  const unsigned long long cut = __ballot(mine > 1);
+  if (lane == kWave - 1) { plan[0] = incl; plan[1] = __popcll(cut); }
+  typedef int int4v __attribute__((ext_vector_type(4)));
+  int4v* list = reinterpret_cast<int4v*>(plan + 4);
+  for (int c = 0; c < mine; ++c) list[first + c] = int4v{lane, lo + c * chunk, min(lo + (c + 1) * chunk, hi), mine};
+  if (mine > 1) list[slots + __popcll(cut & ((1ull << lane) - 1))] = int4v{lane, first, mine, 0};
+}
+
 template <int MT, int NTW, bool GATHER_P, bool GATHER_Q>
 __global__ __launch_bounds__(512) void wgrad_kmajor_kernel(const bf16_t* __restrict__ P, const bf16_t* __restrict__ Q,
                                                            const int32_t* __restrict__ index,
                                                            const int32_t* __restrict__ offsets,
-                                                           const bf16_t* __restrict__ zrow, int N, int M, int E,
+                                                           const bf16_t* __restrict__ zrow, int N, int M,
+                                                           const int* __restrict__ plan, float* __restrict__ part,
                                                            bf16_t* __restrict__ dW) {
   static_assert(MT == 2 || MT == 4, "128 or 256 rows of dW per workgroup");
   constexpr int BM = 64 * MT, BN = kSubW * NTW;
@@ -312,12 +342,16 @@ __global__ __launch_bounds__(512) void wgrad_kmajor_kernel(const bf16_t* __restr
   // Workgroup ids congruent mod 8 run on one XCD: they walk a contiguous range of (expert, m block, n block) triples,
   // so the workgroups that read the same rows of Q (and of P) share that XCD's L2.
   const int nblk_n = N / BM, nblk_m = M / BN;
-  const int item = xcd_tile(blockIdx.x, E * nblk_n * nblk_m);
-  if (item >= E * nblk_n * nblk_m) return;
-  const int e = item / (nblk_n * nblk_m), rest = item - e * (nblk_n * nblk_m);
-  const int n0 = (rest % nblk_n) * BM, m0 = (rest / nblk_n) * BN;
-  const int lo = __builtin_amdgcn_readfirstlane(offsets[e]), hi = __builtin_amdgcn_readfirstlane(offsets[e + 1]);
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int total_chunks = __builtin_amdgcn_readfirstlane(plan[0]);
+  const int item = xcd_tile(blockIdx.x, total_chunks * nblk_n * nblk_m);
+  if (item >= total_chunks * nblk_n * nblk_m) return;
+  const int cg = item / (nblk_n * nblk_m), rest = item - cg * (nblk_n * nblk_m);      // chunk, numbered over all experts
+  const int* entry = plan + 4 + 4 * cg;
+  const int e = __builtin_amdgcn_readfirstlane(entry[0]);
+  const int lo = __builtin_amdgcn_readfirstlane(entry[1]), hi = __builtin_amdgcn_readfirstlane(entry[2]);
+  const int e_chunks = __builtin_amdgcn_readfirstlane(entry[3]);
+  const int n0 = (rest % nblk_n) * BM, m0 = (rest / nblk_n) * BN;
   const int wn = wave & 3, wm = wave >> 2;
   floatx16 acc[MT][NTW];
 #pragma unroll
@@ -408,18 +442,64 @@ __global__ __launch_bounds__(512) void wgrad_kmajor_kernel(const bf16_t* __restr
   // accumulators transposed: lane = row n0 + wm MT 32 + 32 mt + lane % 32, register 4 q + r = column
   // m0 + (wn NTW + j) 32 + 8 q + 4 (lane / 32) + r
   const int n = lane & 31, hh = lane >> 5;
-  bf16_t* orow = dW + ((size_t)e * N + n0 + wm * MT * 32 + n) * M + m0 + wn * NTW * 32 + 4 * hh;
+  const size_t oofs = ((size_t)n0 + wm * MT * 32 + n) * M + m0 + wn * NTW * 32 + 4 * hh;
+  if (e_chunks == 1) {
+    bf16_t* orow = dW + (size_t)e * N * M + oofs;
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
+    for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-    for (int j = 0; j < NTW; ++j)
+      for (int j = 0; j < NTW; ++j)
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        bf16x4 v;
+        for (int q = 0; q < 4; ++q) {
+          bf16x4 v;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) v[r] = (bf16_t)acc[mt][j][4 * q + r];
-        *reinterpret_cast<bf16x4*>(orow + (size_t)mt * 32 * M + j * 32 + 8 * q) = v;
-      }
+          for (int r = 0; r < 4; ++r) v[r] = (bf16_t)acc[mt][j][4 * q + r];
+          *reinterpret_cast<bf16x4*>(orow + (size_t)mt * 32 * M + j * 32 + 8 * q) = v;
+        }
+  } else {
+    float* prow = part + (size_t)cg * N * M + oofs;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int j = 0; j < NTW; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          floatx4 v;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) v[r] = acc[mt][j][4 * q + r];
+          *reinterpret_cast<floatx4*>(prow + (size_t)mt * 32 * M + j * 32 + 8 * q) = v;
+        }
+  }
+}
+
+// For the experts that were cut into chunks (none, when the tokens are spread evenly: then a workgroup reads one word
+// of the plan and is done): dW[e] = the sum of expert e's partial tiles, in chunk order, for both weight tensors in one
+// launch (partials of the first in `part_a`, [.., NMa] each, of the second in `part_b`).  A thread per four elements.
+__global__ __launch_bounds__(256) void wgrad_reduce_kernel(const float* __restrict__ part_a, const float* __restrict__ part_b,
+                                                           const int* __restrict__ plan, int slots, int NMa, int NMb,
+                                                           bf16_t* __restrict__ dWa, bf16_t* __restrict__ dWb) {
+  const int n_cut = plan[1];
+  if (n_cut == 0) return;
+  const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  const int* cut = plan + 4 + 4 * slots;
+  auto reduce = [&](const float* part, int NM, bf16_t* dW, int e, int first, int n) {
+    if (i >= (size_t)NM) return;
+    floatx4 acc = *reinterpret_cast<const floatx4*>(part + (size_t)first * NM + i);
+    for (int c = 1; c < n; ++c) {
+      const floatx4 v = *reinterpret_cast<const floatx4*>(part + (size_t)(first + c) * NM + i);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[r] += v[r];
+    }
+    bf16x4 o;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) o[r] = (bf16_t)acc[r];
+    *reinterpret_cast<bf16x4*>(dW + (size_t)e * NM + i) = o;
+  };
+  for (int q = 0; q < n_cut; ++q) {
+    const int e = cut[4 * q], first = cut[4 * q + 1], n = cut[4 * q + 2];
+    reduce(part_a, NMa, dWa, e, first, n);
+    reduce(part_b, NMb, dWb, e, first, n);
+  }
 }
 
 }  // namespace

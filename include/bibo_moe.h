@@ -281,7 +281,9 @@ int bibo_moe_ffn_forward(const void* h, const float* norm_weight, float eps, con
  * 2H + 5I floats of a row in LDS: BIBO_ERR_UNSUPPORTED when neither applies, i.e. off the MFMA sizes with
  * (2H + 5I) * 4 + 64 > 65536.  The intermediate activations are recomputed, nothing has to be kept from the forward
  * call.  All gradients are overwritten, not accumulated.  Workspace: bibo_moe_backward_workspace_bytes (MFMA family:
- * about 12 I + 2 H bytes per routed slot; generic family: 12 I + 4 H).
+ * about 12 I + 2 H bytes per routed slot plus 12 I H bytes for each of up to 1.7 E partial weight-gradient tiles, which
+ * are only written for experts that hold more than 1.5 times the average number of rows; generic family: 12 I + 4 H
+ * bytes per routed slot).
  */
 int bibo_moe_backward_workspace_bytes(const bibo_moe_shape* shape, size_t* bytes);
 int bibo_moe_backward(const void* x, const void* d_out, const void* w_router, const float* bias, const void* w_gate_up,

@@ -200,6 +200,26 @@ def test_layer_trains_the_same_with_and_without_kept_activations():
         assert torch.equal(p1[n], p2[n]), n
 
 
+def test_backward_with_a_few_experts_holding_most_rows():
+    """Four experts that every token selects (selection bias + 2): their rows are cut into chunks by the weight-gradient
+    GEMMs and the chunks' partial tiles are added up; every gradient against the oracle, and twice the same bits."""
+    T, H, E, k, I = 1500, 256, 16, 6, 128                  # 1500 rows on each hot expert, 250 on average elsewhere
+    p = O.make_inputs(T=T, H=H, E=E, k=k, I=I, bias="hot4", theta="normal", seed=44)
+    g = torch.Generator().manual_seed(45)
+    d_out = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    dev = lambda t: t.to(DEV)
+    args = [dev(p[n]) for n in ("w_router", "bias", "w_gate_up", "w_down", "theta")]
+    _, idx, _, counts, _ = ops.moe_forward(dev(p["x"]), *args, k, want_routing=True, want_counts=True)
+    assert int(counts.max()) == T and int(counts.max()) > 2 * (T * k // E)      # cut into chunks: above 1.5 x the average
+    got = ops.moe_backward(dev(p["x"]), dev(d_out), *args, k, want_dw=True)
+    again = ops.moe_backward(dev(p["x"]), dev(d_out), *args, k, want_dw=True)
+    torch.cuda.synchronize()
+    ref = O.moe_backward(p["x"], p["w_router"], p["w_gate_up"], p["w_down"], p["theta"], idx.cpu().numpy(), d_out)
+    for a, b_, name in zip(got, again, ("x", "w_router", "w_gate_up", "w_down", "theta", "w")):
+        assert torch.equal(a, b_), name
+        assert _rel(a, ref[name]) <= TOL, (name, _rel(a, ref[name]))
+
+
 def test_backward_is_linear_in_the_upstream_gradient():
     """Size-independent property at the full c2 shape: the gradients of 2 d are twice those of d (every path is linear
     in d_out), to bf16 rounding; and nothing is accumulated between calls."""
