@@ -169,30 +169,29 @@ hipError_t launch_dgrad(const bf16_t* A, const int32_t* a_index, const bf16_t* W
 // dW[e] = P(rows of e)^T Q(rows of e), P [.., N] and Q [.., M] row-major (kmajor.h)
 template <int MT, bool GATHER_P, bool GATHER_Q>
 hipError_t launch_wgrad_t(const bf16_t* P, const bf16_t* Q, const int32_t* index, const int32_t* offsets, const bf16_t* zrow,
-                          int N, int M, int S_rows, int E, const int* plan, float* part, bf16_t* dW, hipStream_t s) {
-  const dim3 block(512);
-  const int slots = backward_wgrad_part_slots(S_rows, E);      // (the partial tiles of cut experts are added up by wgrad_reduce_kernel)
+                          int N, int M, int E, int slots, const int* plan, float* part, bf16_t* dW, hipStream_t s) {
+  const dim3 block(512);               // (the partial tiles of cut experts are added up by wgrad_reduce_kernel)
   auto grid = [&](int bn) { return dim3((unsigned)((slots * (N / (64 * MT)) * (M / bn) + 7) & ~7)); };
   if (M % 384 == 0)
     hipLaunchKernelGGL((wgrad_kmajor_kernel<MT, 3, GATHER_P, GATHER_Q>), grid(384), block, 0, s, P, Q, index, offsets, zrow, N,
-                       M, plan, part, dW);
+                       M, E, plan, part, dW);
   else if (M % 256 == 0)
     hipLaunchKernelGGL((wgrad_kmajor_kernel<MT, 2, GATHER_P, GATHER_Q>), grid(256), block, 0, s, P, Q, index, offsets, zrow, N,
-                       M, plan, part, dW);
+                       M, E, plan, part, dW);
   else
     hipLaunchKernelGGL((wgrad_kmajor_kernel<MT, 1, GATHER_P, GATHER_Q>), grid(128), block, 0, s, P, Q, index, offsets, zrow, N,
-                       M, plan, part, dW);
+                       M, E, plan, part, dW);
   return hipGetLastError();
 }
 
 // 256 rows of dW per workgroup where N allows and the experts have rows enough for the streams to matter
 template <bool GATHER_P, bool GATHER_Q>
 hipError_t launch_wgrad(const bf16_t* P, const bf16_t* Q, const int32_t* index, const int32_t* offsets, const bf16_t* zrow,
-                        int N, int M, int S_rows, int E, const int* plan, float* part, bf16_t* dW, hipStream_t s) {
+                        int N, int M, int S_rows, int E, int slots, const int* plan, float* part, bf16_t* dW, hipStream_t s) {
   const int bn = M % 384 == 0 ? 384 : (M % 256 == 0 ? 256 : 128);
   if (N % 256 == 0 && tall_tiles(S_rows, E, (long long)E * (N / 128) * (M / bn), (long long)E * (N / 256) * (M / bn)))
-    return launch_wgrad_t<4, GATHER_P, GATHER_Q>(P, Q, index, offsets, zrow, N, M, S_rows, E, plan, part, dW, s);
-  return launch_wgrad_t<2, GATHER_P, GATHER_Q>(P, Q, index, offsets, zrow, N, M, S_rows, E, plan, part, dW, s);
+    return launch_wgrad_t<4, GATHER_P, GATHER_Q>(P, Q, index, offsets, zrow, N, M, E, slots, plan, part, dW, s);
+  return launch_wgrad_t<2, GATHER_P, GATHER_Q>(P, Q, index, offsets, zrow, N, M, E, slots, plan, part, dW, s);
 }
 
 // ---- Radial NormSiLU backward (moe.py:87-92), one wave per permuted row ----------------------------------------
@@ -210,12 +209,12 @@ __global__ __launch_bounds__(256) void act_bwd_kernel(const bf16_t* __restrict__
                                                       bf16_t* __restrict__ dgu, bf16_t* __restrict__ hidden,
                                                       float* __restrict__ dw_slot, float* __restrict__ dtheta_row,
                                                       uint32_t* __restrict__ zero_words, int n_zero_words,
-                                                      int* __restrict__ plan, int chunk, int slots) {
+                                                      int* __restrict__ plan, int n_routed, int chunk, int slots) {
   // (the first workgroup also clears the row of zeros the weight-gradient kernels read past an expert's last row and,
   // with its first wave, lists the row chunks those kernels work through)
   if (blockIdx.x == 0) {
     for (int i = threadIdx.x; i < n_zero_words; i += 256) zero_words[i] = 0u;
-    if (threadIdx.x < kWave) wgrad_plan(offsets, E, chunk, slots, plan);
+    if (threadIdx.x < kWave) wgrad_plan(offsets, n_routed, chunk, slots, plan);
   }
   const int lane = threadIdx.x & 63;
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -323,18 +322,22 @@ __global__ __launch_bounds__(256) void special_bwd_kernel(const bf16_t* __restri
   if (lane == 0) dw_slot[slot] = sign * dot;
 }
 
-// dtheta[e] = sum of its rows' contributions, in a fixed order (no atomics: the same bits on every call).
-__global__ __launch_bounds__(256) void dtheta_reduce_kernel(const float* __restrict__ dtheta_row,
-                                                            const int32_t* __restrict__ offsets,
-                                                            float* __restrict__ dtheta) {
+// The theta gradient's sum over an expert's rows, in a fixed order (no atomics: the same bits on every call): one
+// workgroup per row chunk of the plan (kmajor.h) -> theta_part[chunk]; wgrad_reduce_kernel adds an expert's chunks.
+__global__ __launch_bounds__(256) void dtheta_reduce_kernel(const float* __restrict__ dtheta_row, const int* __restrict__ plan,
+                                                            int E, float* __restrict__ theta_part) {
   __shared__ float red[4];
-  const int e = blockIdx.x, lo = offsets[e], hi = offsets[e + 1];
+  const int cg = blockIdx.x;
+  if (cg >= plan[0]) return;
+  const int* entry = plan + 4 + 4 * cg;
+  const int e = entry[0], lo = entry[1], hi = entry[2];
+  if (e >= E) return;
   float acc = 0.f;
   for (int r = lo + threadIdx.x; r < hi; r += 256) acc += dtheta_row[r];
   acc = wave_sum(acc);
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;
   __syncthreads();
-  if (threadIdx.x == 0) dtheta[e] = (red[0] + red[1]) + (red[2] + red[3]);
+  if (threadIdx.x == 0) theta_part[cg] = (red[0] + red[1]) + (red[2] + red[3]);
 }
 
 // ---- router backward (router.py:31,41-47) --------------------------------------------------------------------
@@ -408,20 +411,22 @@ __global__ __launch_bounds__(256) void dx_combine_kernel(const bf16_t* __restric
 }
 
 // dW_router[e, c] = sum over the rows r of expert e of dl[slot(r)] x[token(r), c], in two steps.  Step 1, grid =
-// (H / 256, E, kDwrSplit): block z takes the z-th of kDwrSplit equal row ranges of the expert; thread (rl = t / 32,
-// cg = t % 32) adds up rows rl, rl + 8, .. of the range for columns 8 cg .. + 8 of the block's 256, the eight partial
-// sums meet in LDS in a fixed order -> part[e][z][c] fp32.  Step 2 adds the kDwrSplit ranges in order.
+// (H / 256, chunks, kDwrSplit): block (., g, z) takes the z-th of kDwrSplit equal row ranges of row chunk g of the plan
+// (kmajor.h: an expert's rows, cut where an expert holds many); thread (rl = t / 32, cg = t % 32) adds up rows rl,
+// rl + 8, .. of the range for columns 8 cg .. + 8 of the block's 256, the eight partial sums meet in LDS in a fixed
+// order -> part[g][z][c] fp32.  Step 2 adds the ranges of an expert's chunks in order.
 constexpr int kDwrSplit = 8;
 
 __global__ __launch_bounds__(256) void dwr_partial_kernel(const bf16_t* __restrict__ x, const float* __restrict__ dl,
-                                                          const int32_t* __restrict__ offsets,
+                                                          const int* __restrict__ plan,
                                                           const int32_t* __restrict__ perm_slot,
                                                           const int32_t* __restrict__ perm_token, int H,
                                                           float* __restrict__ part) {
   __shared__ float red[8][256];
-  const int e = blockIdx.y, z = blockIdx.z, cg = threadIdx.x & 31, rl = threadIdx.x >> 5;
+  const int g = blockIdx.y, z = blockIdx.z, cg = threadIdx.x & 31, rl = threadIdx.x >> 5;
+  if (g >= plan[0]) return;
   const int c = blockIdx.x * 256 + cg * 8;
-  const int lo_e = offsets[e], n = offsets[e + 1] - lo_e;
+  const int lo_e = plan[4 + 4 * g + 1], n = plan[4 + 4 * g + 2] - lo_e;
   const int per = (n + kDwrSplit - 1) / kDwrSplit;
   const int lo = lo_e + min(z * per, n), hi = lo_e + min((z + 1) * per, n);
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -438,18 +443,20 @@ __global__ __launch_bounds__(256) void dwr_partial_kernel(const bf16_t* __restri
   const int col = blockIdx.x * 256 + threadIdx.x;
   if (col < H) {
     const int t = threadIdx.x;
-    part[((size_t)e * kDwrSplit + z) * H + col] =
+    part[((size_t)g * kDwrSplit + z) * H + col] =
         ((red[0][t] + red[1][t]) + (red[2][t] + red[3][t])) + ((red[4][t] + red[5][t]) + (red[6][t] + red[7][t]));
   }
 }
 
-__global__ __launch_bounds__(256) void dwr_sum_kernel(const float* __restrict__ part, int H, int n, bf16_t* __restrict__ dwr) {
+// n = E H elements; `experts` = the plan's per-expert entries {first chunk, chunks, ., .}
+__global__ __launch_bounds__(256) void dwr_sum_kernel(const float* __restrict__ part, const int* __restrict__ experts, int H,
+                                                      int n, bf16_t* __restrict__ dwr) {
   const int i = blockIdx.x * 256 + threadIdx.x;                 // element of [E, H]
   if (i >= n) return;
   const int e = i / H, c = i - e * H;
+  const int first = experts[4 * e], chunks = experts[4 * e + 1];
   float acc = 0.f;
-#pragma unroll
-  for (int z = 0; z < kDwrSplit; ++z) acc += part[((size_t)e * kDwrSplit + z) * H + c];
+  for (int j = 0; j < chunks * kDwrSplit; ++j) acc += part[((size_t)first * kDwrSplit + j) * H + c];
   dwr[i] = (bf16_t)acc;
 }
 
@@ -475,25 +482,27 @@ bool backward_supported(int H, int I, int k, int dtype) {
 int backward_dwr_split() { return kDwrSplit; }
 
 // a row of zeros as wide as the widest weight-gradient operand: what a K stage reads past an expert's last row
-// The weight-gradient GEMMs cut an expert with more rows than this into chunks (kmajor.h): one and a half times the
-// average, so that evenly routed tokens leave every expert in one piece, and at least 512.
-int backward_wgrad_chunk_rows(int S_rows, int E) {
+// The sums over an expert's rows (weight-gradient GEMMs, router weight gradient, theta gradient) cut an expert with more
+// rows than this into chunks (kmajor.h): one and a half times the average over all E routed experts, so that evenly
+// routed tokens leave every expert in one piece, and at least 512.
+int backward_chunk_rows(int S_rows, int E) {
   const long long c = (3ll * S_rows / (2ll * E) + 31) & ~31ll;
   return (int)(c < 512 ? 512 : c);
 }
-// chunks over all experts, at most: the fp32 partial tiles of the cut experts are numbered so
-int backward_wgrad_part_slots(int S_rows, int E) { return S_rows / backward_wgrad_chunk_rows(S_rows, E) + E; }
+// chunks over all experts, at most
+int backward_chunk_slots(int S_rows, int E) { return S_rows / backward_chunk_rows(S_rows, E) + E; }
+// fp32 partial tiles of the cut experts, dW_down's and dW_gate_up's, one slot per chunk each
 size_t backward_wgrad_part_bytes(int S_rows, int H, int E, int I) {
-  return (size_t)backward_wgrad_part_slots(S_rows, E) * 3 * I * H * sizeof(float);      // dW_down's and dW_gate_up's
+  return (size_t)backward_chunk_slots(S_rows, E) * 3 * I * H * sizeof(float);
 }
-// the list of chunks (kmajor.h: WgradPlan): a header, a 16-byte entry per chunk and one per expert
-size_t backward_wgrad_plan_bytes(int S_rows, int E) { return 16 + (size_t)(backward_wgrad_part_slots(S_rows, E) + E) * 16; }
+// the list of chunks (kmajor.h: WgradPlan): a header, a 16-byte entry per chunk and two per expert
+size_t backward_plan_bytes(int S_rows, int E) { return 16 + (size_t)(backward_chunk_slots(S_rows, E) + 2 * E) * 16; }
 
 size_t backward_zero_row_bytes(int H, int I) { return (size_t)(H > 2 * I ? H : 2 * I) * sizeof(bf16_t); }
 
 // The launches after routing and permutation.  Buffers (bf16 unless noted): gu [S,2I], dhp [S,I], dgu [S,2I],
 // hidden [S,I], dxs [S,H], zrow [max(H, 2I)] (cleared by act_bwd_kernel), dw_slot [S] f32, dl [S] f32, dtheta_row [S] f32,
-// dwr_part [E, backward_dwr_split(), H] f32.
+// dwr_part [backward_chunk_slots(), backward_dwr_split(), H] f32, theta_part [backward_chunk_slots()] f32.
 hipError_t launch_backward(const void* x, const void* d_out, const void* w_router, const void* wgu, const void* wd,
                            const float* theta, const float* logits, const int32_t* idx, const float* w,
                            const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token, int T, int H, int E,
@@ -502,6 +511,7 @@ hipError_t launch_backward(const void* x, const void* d_out, const void* w_route
   // E = GLU experts (with weights); the router and the permutation know Et experts, the +/-Identity ones last
   const int Et = E + n_pos + n_neg;
   const int S = T * k;
+  const int slots = backward_chunk_slots(S, Et);      // row chunks of the plan, at most
   const bf16_t* xp = static_cast<const bf16_t*>(x);
   const bf16_t* dop = static_cast<const bf16_t*>(d_out);
   const bf16_t* wrp = static_cast<const bf16_t*>(w_router);
@@ -536,9 +546,8 @@ hipError_t launch_backward(const void* x, const void* d_out, const void* w_route
   if (err != hipSuccess) return err;
   hipLaunchKernelGGL(act_bwd_kernel, dim3((S + 3) / 4), dim3(256), 0, s, gu, dhp, w, theta, offsets, perm_slot, S, E, I, act,
                      dgu, hidden, b.dw_slot, b.dtheta_row, reinterpret_cast<uint32_t*>(zrow),
-                     (int)(backward_zero_row_bytes(H, I) / 4), b.wgrad_plan, backward_wgrad_chunk_rows(S, E),
-                     backward_wgrad_part_slots(S, E));
-  hipLaunchKernelGGL(dtheta_reduce_kernel, dim3(E), dim3(256), 0, s, b.dtheta_row, offsets, d_theta);
+                     (int)(backward_zero_row_bytes(H, I) / 4), b.wgrad_plan, Et, backward_chunk_rows(S, Et), slots);
+  hipLaunchKernelGGL(dtheta_reduce_kernel, dim3(slots), dim3(256), 0, s, b.dtheta_row, b.wgrad_plan, E, b.theta_part);
   // dx of every slot, in slot order: [dg, du] W_gate_up, contracts over the 2I rows of w_gate_up [E, 2I, H]
   err = launch_dgrad<false, true>(dgu, nullptr, wgup, offsets, perm_slot, S, 2 * I, H, E, dxs, s);
   if (err != hipSuccess) return err;
@@ -552,22 +561,22 @@ hipError_t launch_backward(const void* x, const void* d_out, const void* w_route
   hipLaunchKernelGGL(dx_combine_kernel, dim3((unsigned)(((long long)T * (H / 8) + 255) / 256)), dim3(256), 0, s, dxs,
                      with_router ? b.dl : nullptr, idx, wrp, T, H, k, Et, b.dw_slot, static_cast<bf16_t*>(dx));
   if (with_router) {
-    hipLaunchKernelGGL(dwr_partial_kernel, dim3((H + 255) / 256, Et, kDwrSplit), dim3(256), 0, s, xp, b.dl, offsets, perm_slot,
-                       perm_token, H, b.dwr_part);
-    hipLaunchKernelGGL(dwr_sum_kernel, dim3((Et * H + 255) / 256), dim3(256), 0, s, b.dwr_part, H, Et * H,
-                       static_cast<bf16_t*>(d_w_router));
+    hipLaunchKernelGGL(dwr_partial_kernel, dim3((H + 255) / 256, slots, kDwrSplit), dim3(256), 0, s, xp, b.dl, b.wgrad_plan,
+                       perm_slot, perm_token, H, b.dwr_part);
+    hipLaunchKernelGGL(dwr_sum_kernel, dim3((Et * H + 255) / 256), dim3(256), 0, s, b.dwr_part,
+                       b.wgrad_plan + 4 + 4 * (slots + Et), H, Et * H, static_cast<bf16_t*>(d_w_router));
   }
   // weight gradients, contracted over each expert's rows: dW_down[e] = d^T (w h) (d gathered by token, `hidden`
   // already carries w), dW_gate_up[e] = [dg, du]^T x (x gathered by token)
-  err = launch_wgrad<true, false>(dop, hidden, perm_token, offsets, zrow, H, I, S, E, b.wgrad_plan, b.wgrad_part, static_cast<bf16_t*>(d_wd), s);
+  err = launch_wgrad<true, false>(dop, hidden, perm_token, offsets, zrow, H, I, S, E, slots, b.wgrad_plan, b.wgrad_part, static_cast<bf16_t*>(d_wd), s);
   if (err != hipSuccess) return err;
-  float* part_gu = b.wgrad_part + (size_t)backward_wgrad_part_slots(S, E) * H * I;
-  err = launch_wgrad<false, true>(dgu, xp, perm_token, offsets, zrow, 2 * I, H, S, E, b.wgrad_plan, part_gu, static_cast<bf16_t*>(d_wgu), s);
+  float* part_gu = b.wgrad_part + (size_t)slots * H * I;
+  err = launch_wgrad<false, true>(dgu, xp, perm_token, offsets, zrow, 2 * I, H, S, E, slots, b.wgrad_plan, part_gu, static_cast<bf16_t*>(d_wgu), s);
   if (err != hipSuccess) return err;
   // experts with so many rows that they were cut into chunks: their partial tiles added up in chunk order
   hipLaunchKernelGGL(wgrad_reduce_kernel, dim3((unsigned)(((size_t)2 * I * H / 4 + 255) / 256)), dim3(256), 0, s, b.wgrad_part,
-                     part_gu, b.wgrad_plan, backward_wgrad_part_slots(S, E), H * I, 2 * I * H, static_cast<bf16_t*>(d_wd),
-                     static_cast<bf16_t*>(d_wgu));
+                     part_gu, b.wgrad_plan, slots, H * I, 2 * I * H, E, Et, b.theta_part, static_cast<bf16_t*>(d_wd),
+                     static_cast<bf16_t*>(d_wgu), d_theta);
   return hipGetLastError();
 }
 

@@ -221,16 +221,17 @@ hipError_t launch_attn_res(const void* const* cands, int n_cand, const float* sc
 struct BackwardBuffers {
   void *gu, *dhp, *dgu, *hidden, *dxs, *zrow;                       // bf16 device buffers, sizes in launch_backward's comment
   float *dw_slot, *dl, *dtheta_row;                                 // [T*k] each
-  float* dwr_part;                                                  // [E, backward_dwr_split(), H]
+  float* dwr_part;                                                  // [backward_chunk_slots(), backward_dwr_split(), H]
+  float* theta_part;                                                // [backward_chunk_slots()]
   float* wgrad_part;                                                // backward_wgrad_part_bytes(): partial dW tiles of experts cut into chunks
-  int* wgrad_plan;                                                  // backward_wgrad_plan_bytes(): the list of chunks, written by act_bwd_kernel
+  int* wgrad_plan;                                                  // backward_plan_bytes(): the list of row chunks, written by act_bwd_kernel
 };
 bool backward_supported(int H, int I, int k, int dtype);
 size_t backward_zero_row_bytes(int H, int I);
-int backward_wgrad_chunk_rows(int S_rows, int E);
-int backward_wgrad_part_slots(int S_rows, int E);
+int backward_chunk_rows(int S_rows, int E);
+int backward_chunk_slots(int S_rows, int E);
 size_t backward_wgrad_part_bytes(int S_rows, int H, int E, int I);
-size_t backward_wgrad_plan_bytes(int S_rows, int E);
+size_t backward_plan_bytes(int S_rows, int E);
 int backward_dwr_split();
 // the generic family (backward_generic.hip): any sizes, bf16 or fp32 operands; every buffer fp32
 struct GenericBackwardBuffers {

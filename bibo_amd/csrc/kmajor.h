@@ -299,11 +299,13 @@ struct WgradPlan {
   int total;         // chunks over all experts
   int n_cut;         // experts cut into more than one chunk
   int pad[2];
-  // followed by int4 chunk[total] = {expert, first row, end row, chunks of that expert}
-  // and, from entry `slots` on, int4 cut[n_cut] = {expert, its first chunk, its chunks, 0}
+  // followed by int4 chunk[total] = {expert, first row, end row, chunks of that expert},
+  // from entry `slots` on int4 cut[n_cut] = {expert, its first chunk, its chunks, 0},
+  // and from entry `slots + E` on int4 expert[E] = {first chunk, chunks, 0, 0}
 };
 
-// One wave: lane = expert.  `slots` = the capacity of the chunk list (backward_wgrad_part_slots).
+// One wave: lane = expert, over ALL routed experts (the +/-Identity ones have rows for the router's weight gradient).
+// `slots` = the capacity of the chunk list (backward_chunk_slots).
 __device__ __forceinline__ void wgrad_plan(const int32_t* __restrict__ offsets, int E, int chunk, int slots, int* __restrict__ plan) {
   const int lane = lane_id();
   int lo = 0, hi = 0;
@@ -317,13 +319,14 @@ __device__ __forceinline__ void wgrad_plan(const int32_t* __restrict__ offsets, 
   int4v* list = reinterpret_cast<int4v*>(plan + 4);
   for (int c = 0; c < mine; ++c) list[first + c] = int4v{lane, lo + c * chunk, min(lo + (c + 1) * chunk, hi), mine};
   if (mine > 1) list[slots + __popcll(cut & ((1ull << lane) - 1))] = int4v{lane, first, mine, 0};
+  if (lane < E) list[slots + E + lane] = int4v{first, mine, 0, 0};
 }
 
 template <int MT, int NTW, bool GATHER_P, bool GATHER_Q>
 __global__ __launch_bounds__(512) void wgrad_kmajor_kernel(const bf16_t* __restrict__ P, const bf16_t* __restrict__ Q,
                                                            const int32_t* __restrict__ index,
                                                            const int32_t* __restrict__ offsets,
-                                                           const bf16_t* __restrict__ zrow, int N, int M,
+                                                           const bf16_t* __restrict__ zrow, int N, int M, int E,
                                                            const int* __restrict__ plan, float* __restrict__ part,
                                                            bf16_t* __restrict__ dW) {
   static_assert(MT == 2 || MT == 4, "128 or 256 rows of dW per workgroup");
@@ -344,11 +347,15 @@ __global__ __launch_bounds__(512) void wgrad_kmajor_kernel(const bf16_t* __restr
   const int nblk_n = N / BM, nblk_m = M / BN;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int total_chunks = __builtin_amdgcn_readfirstlane(plan[0]);
-  const int item = xcd_tile(blockIdx.x, total_chunks * nblk_n * nblk_m);
+  // With experts cut into chunks the work per chunk is uneven (a cut expert's chunks are several times a small
+  // expert's rows) and contiguous ranges of chunks per XCD would leave some XCDs with most of it: round robin then.
+  const bool uneven = __builtin_amdgcn_readfirstlane(plan[1]) > 0;
+  const int item = uneven ? (int)blockIdx.x : xcd_tile(blockIdx.x, total_chunks * nblk_n * nblk_m);
   if (item >= total_chunks * nblk_n * nblk_m) return;
   const int cg = item / (nblk_n * nblk_m), rest = item - cg * (nblk_n * nblk_m);      // chunk, numbered over all experts
   const int* entry = plan + 4 + 4 * cg;
   const int e = __builtin_amdgcn_readfirstlane(entry[0]);
+  if (e >= E) return;                    // E = experts with weights; the chunks behind them belong to +/-Identity experts
   const int lo = __builtin_amdgcn_readfirstlane(entry[1]), hi = __builtin_amdgcn_readfirstlane(entry[2]);
   const int e_chunks = __builtin_amdgcn_readfirstlane(entry[3]);
   const int n0 = (rest % nblk_n) * BM, m0 = (rest / nblk_n) * BN;
@@ -472,12 +479,21 @@ __global__ __launch_bounds__(512) void wgrad_kmajor_kernel(const bf16_t* __restr
   }
 }
 
-// For the experts that were cut into chunks (none, when the tokens are spread evenly: then a workgroup reads one word
-// of the plan and is done): dW[e] = the sum of expert e's partial tiles, in chunk order, for both weight tensors in one
-// launch (partials of the first in `part_a`, [.., NMa] each, of the second in `part_b`).  A thread per four elements.
+// The last launch of the backward pass.  For the experts that were cut into chunks (none, when the tokens are spread
+// evenly): dW[e] = the sum of expert e's partial tiles, in chunk order, for both weight tensors (partials of the first
+// in `part_a`, [.., NMa] each, of the second in `part_b`).  A thread per four elements.  And dtheta[e] = the sum of
+// expert e's per-chunk sums, in chunk order (workgroup 0, thread e).  E = experts with weights, Et = all.
 __global__ __launch_bounds__(256) void wgrad_reduce_kernel(const float* __restrict__ part_a, const float* __restrict__ part_b,
-                                                           const int* __restrict__ plan, int slots, int NMa, int NMb,
-                                                           bf16_t* __restrict__ dWa, bf16_t* __restrict__ dWb) {
+                                                           const int* __restrict__ plan, int slots, int NMa, int NMb, int E,
+                                                           int Et, const float* __restrict__ theta_part,
+                                                           bf16_t* __restrict__ dWa, bf16_t* __restrict__ dWb,
+                                                           float* __restrict__ dtheta) {
+  if (blockIdx.x == 0 && (int)threadIdx.x < E) {
+    const int* ex = plan + 4 + 4 * (slots + Et + threadIdx.x);
+    float acc = 0.f;
+    for (int c = 0; c < ex[1]; ++c) acc += theta_part[ex[0] + c];
+    dtheta[threadIdx.x] = acc;
+  }
   const int n_cut = plan[1];
   if (n_cut == 0) return;
   const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
@@ -497,6 +513,7 @@ __global__ __launch_bounds__(256) void wgrad_reduce_kernel(const float* __restri
   };
   for (int q = 0; q < n_cut; ++q) {
     const int e = cut[4 * q], first = cut[4 * q + 1], n = cut[4 * q + 2];
+    if (e >= E) continue;
     reduce(part_a, NMa, dWa, e, first, n);
     reduce(part_b, NMb, dWb, e, first, n);
   }
