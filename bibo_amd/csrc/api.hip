@@ -288,7 +288,7 @@ int forward_impl(const void* x, const void* w_router, const float* bias, const v
 
 
 struct BackwardWorkspace {
-  size_t hist, idx, w, logits, counts, offsets, perm_slot, perm_token, dw_slot, dl, dtheta_row, dwr_part, theta_part, zrow, gu, dhp, dgu,
+  size_t hist, idx, w, logits, counts, offsets, perm_slot, perm_token, dw_slot, dl, dtheta_row, dwr_part, zrow, gu, dhp, dgu,
       hidden, dxs, wgrad_part, wgrad_plan, total;
 };
 
@@ -309,7 +309,6 @@ BackwardWorkspace carve_backward(int T, int H, int E, int k, int I) {
   ws.dl = o;         o += align_up(S * sizeof(float));
   ws.dtheta_row = o; o += align_up(S * sizeof(float));
   ws.dwr_part = o;   o += align_up((size_t)backward_chunk_slots((int)S, E) * backward_dwr_split() * H * sizeof(float));
-  ws.theta_part = o; o += align_up((size_t)backward_chunk_slots((int)S, E) * sizeof(float));
   ws.zrow = o;       o += align_up(backward_zero_row_bytes(H, I));
   ws.gu = o;         o += align_up(S * 2 * I * b);
   ws.dhp = o;        o += align_up(S * I * b);
@@ -419,7 +418,6 @@ int backward_mfma(const void* x, const void* d_out, const void* w_router, const 
   b.dl = reinterpret_cast<float*>(base + ws.dl);
   b.dtheta_row = reinterpret_cast<float*>(base + ws.dtheta_row);
   b.dwr_part = reinterpret_cast<float*>(base + ws.dwr_part);
-  b.theta_part = reinterpret_cast<float*>(base + ws.theta_part);
   b.wgrad_part = reinterpret_cast<float*>(base + ws.wgrad_part);
   b.wgrad_plan = reinterpret_cast<int*>(base + ws.wgrad_plan);
   return hip_rc(launch_backward(x, d_out, w_router, w_gate_up, w_down, theta, logits, idx, w, offsets, perm_slot, perm_token,
@@ -806,7 +804,6 @@ int bibo_moe_experts_backward(const void* x, const void* d_out, const int32_t* i
   b.dl = reinterpret_cast<float*>(base + ws.dl);
   b.dtheta_row = reinterpret_cast<float*>(base + ws.dtheta_row);
   b.dwr_part = reinterpret_cast<float*>(base + ws.dwr_part);
-  b.theta_part = reinterpret_cast<float*>(base + ws.theta_part);
   b.wgrad_part = reinterpret_cast<float*>(base + ws.wgrad_part);
   b.wgrad_plan = reinterpret_cast<int*>(base + ws.wgrad_plan);
   return hip_rc(launch_backward(x, d_out, nullptr, w_gate_up, w_down, theta, nullptr, idx, w, offsets, perm_slot, perm_token,

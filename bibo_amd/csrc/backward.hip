@@ -170,7 +170,7 @@ hipError_t launch_dgrad(const bf16_t* A, const int32_t* a_index, const bf16_t* W
 template <int MT, bool GATHER_P, bool GATHER_Q>
 hipError_t launch_wgrad_t(const bf16_t* P, const bf16_t* Q, const int32_t* index, const int32_t* offsets, const bf16_t* zrow,
                           int N, int M, int E, int slots, const int* plan, float* part, bf16_t* dW, hipStream_t s) {
-  const dim3 block(512);               // (the partial tiles of cut experts are added up by wgrad_reduce_kernel)
+  const dim3 block(512);               // (the partial tiles of cut experts are added up by backward_sums_kernel)
   auto grid = [&](int bn) { return dim3((unsigned)((slots * (N / (64 * MT)) * (M / bn) + 7) & ~7)); };
   if (M % 384 == 0)
     hipLaunchKernelGGL((wgrad_kmajor_kernel<MT, 3, GATHER_P, GATHER_Q>), grid(384), block, 0, s, P, Q, index, offsets, zrow, N,
@@ -322,24 +322,6 @@ __global__ __launch_bounds__(256) void special_bwd_kernel(const bf16_t* __restri
   if (lane == 0) dw_slot[slot] = sign * dot;
 }
 
-// The theta gradient's sum over an expert's rows, in a fixed order (no atomics: the same bits on every call): one
-// workgroup per row chunk of the plan (kmajor.h) -> theta_part[chunk]; wgrad_reduce_kernel adds an expert's chunks.
-__global__ __launch_bounds__(256) void dtheta_reduce_kernel(const float* __restrict__ dtheta_row, const int* __restrict__ plan,
-                                                            int E, float* __restrict__ theta_part) {
-  __shared__ float red[4];
-  const int cg = blockIdx.x;
-  if (cg >= plan[0]) return;
-  const int* entry = plan + 4 + 4 * cg;
-  const int e = entry[0], lo = entry[1], hi = entry[2];
-  if (e >= E) return;
-  float acc = 0.f;
-  for (int r = lo + threadIdx.x; r < hi; r += 256) acc += dtheta_row[r];
-  acc = wave_sum(acc);
-  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;
-  __syncthreads();
-  if (threadIdx.x == 0) theta_part[cg] = (red[0] + red[1]) + (red[2] + red[3]);
-}
-
 // ---- router backward (router.py:31,41-47) --------------------------------------------------------------------
 // Eight lanes per token, lane j < k for slot j: dlogit of the k selected experts from the gradients of the combine
 // weights.  The sums over a token's slots are taken in ascending j by every lane, so they are the same bits in all.
@@ -448,15 +430,50 @@ __global__ __launch_bounds__(256) void dwr_partial_kernel(const bf16_t* __restri
   }
 }
 
-// n = E H elements; `experts` = the plan's per-expert entries {first chunk, chunks, ., .}
-__global__ __launch_bounds__(256) void dwr_sum_kernel(const float* __restrict__ part, const int* __restrict__ experts, int H,
-                                                      int n, bf16_t* __restrict__ dwr) {
-  const int i = blockIdx.x * 256 + threadIdx.x;                 // element of [E, H]
-  if (i >= n) return;
+// The last launch of the backward pass: every sum that ends one, by ranges of workgroups.
+//   [0, nb_w): the partial tiles of the experts that were cut into chunks (kmajor.h) -> dW_down, dW_gate_up;
+//   [nb_w, nb_w + E): dtheta[e] = the sum of the theta shares of expert e's rows, chunk by chunk of the plan and the
+//     chunks in order (no atomics: the same bits on every call);
+//   from nb_w + E on (when dwr != nullptr): the router's weight gradient [Et, H] = the sum over an expert's chunks
+//     of dwr_partial_kernel's partial rows.
+__global__ __launch_bounds__(256) void backward_sums_kernel(int nb_w, const float* __restrict__ part_a,
+                                                            const float* __restrict__ part_b, const int* __restrict__ plan,
+                                                            int slots, int NMa, int NMb, int E, int Et,
+                                                            bf16_t* __restrict__ dWa, bf16_t* __restrict__ dWb,
+                                                            const float* __restrict__ dtheta_row, float* __restrict__ dtheta,
+                                                            const float* __restrict__ dwr_part, int H,
+                                                            bf16_t* __restrict__ dwr) {
+  const int block = blockIdx.x;
+  if (block < nb_w) {
+    wgrad_reduce_block(block, part_a, part_b, plan, slots, NMa, NMb, E, dWa, dWb);
+    return;
+  }
+  const int* experts = plan + 4 + 4 * (slots + Et);            // {first chunk, chunks, ., .} per expert
+  if (block < nb_w + E) {
+    __shared__ float red[4];
+    const int e = block - nb_w;
+    const int first = experts[4 * e], chunks = experts[4 * e + 1];
+    float total = 0.f;
+    for (int c = 0; c < chunks; ++c) {
+      const int* entry = plan + 4 + 4 * (first + c);
+      float acc = 0.f;
+      for (int r = entry[1] + threadIdx.x; r < entry[2]; r += 256) acc += dtheta_row[r];
+      acc = wave_sum(acc);
+      __syncthreads();
+      if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;
+      __syncthreads();
+      total += (red[0] + red[1]) + (red[2] + red[3]);
+    }
+    if (threadIdx.x == 0) dtheta[e] = total;
+    return;
+  }
+  if (dwr == nullptr) return;
+  const int i = (block - nb_w - E) * 256 + threadIdx.x;         // element of [Et, H]
+  if (i >= Et * H) return;
   const int e = i / H, c = i - e * H;
   const int first = experts[4 * e], chunks = experts[4 * e + 1];
   float acc = 0.f;
-  for (int j = 0; j < chunks * kDwrSplit; ++j) acc += part[((size_t)first * kDwrSplit + j) * H + c];
+  for (int j = 0; j < chunks * kDwrSplit; ++j) acc += dwr_part[((size_t)first * kDwrSplit + j) * H + c];
   dwr[i] = (bf16_t)acc;
 }
 
@@ -502,7 +519,7 @@ size_t backward_zero_row_bytes(int H, int I) { return (size_t)(H > 2 * I ? H : 2
 
 // The launches after routing and permutation.  Buffers (bf16 unless noted): gu [S,2I], dhp [S,I], dgu [S,2I],
 // hidden [S,I], dxs [S,H], zrow [max(H, 2I)] (cleared by act_bwd_kernel), dw_slot [S] f32, dl [S] f32, dtheta_row [S] f32,
-// dwr_part [backward_chunk_slots(), backward_dwr_split(), H] f32, theta_part [backward_chunk_slots()] f32.
+// dwr_part [backward_chunk_slots(), backward_dwr_split(), H] f32.
 hipError_t launch_backward(const void* x, const void* d_out, const void* w_router, const void* wgu, const void* wd,
                            const float* theta, const float* logits, const int32_t* idx, const float* w,
                            const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token, int T, int H, int E,
@@ -547,7 +564,6 @@ hipError_t launch_backward(const void* x, const void* d_out, const void* w_route
   hipLaunchKernelGGL(act_bwd_kernel, dim3((S + 3) / 4), dim3(256), 0, s, gu, dhp, w, theta, offsets, perm_slot, S, E, I, act,
                      dgu, hidden, b.dw_slot, b.dtheta_row, reinterpret_cast<uint32_t*>(zrow),
                      (int)(backward_zero_row_bytes(H, I) / 4), b.wgrad_plan, Et, backward_chunk_rows(S, Et), slots);
-  hipLaunchKernelGGL(dtheta_reduce_kernel, dim3(slots), dim3(256), 0, s, b.dtheta_row, b.wgrad_plan, E, b.theta_part);
   // dx of every slot, in slot order: [dg, du] W_gate_up, contracts over the 2I rows of w_gate_up [E, 2I, H]
   err = launch_dgrad<false, true>(dgu, nullptr, wgup, offsets, perm_slot, S, 2 * I, H, E, dxs, s);
   if (err != hipSuccess) return err;
@@ -560,12 +576,9 @@ hipError_t launch_backward(const void* x, const void* d_out, const void* w_route
                        b.dl);
   hipLaunchKernelGGL(dx_combine_kernel, dim3((unsigned)(((long long)T * (H / 8) + 255) / 256)), dim3(256), 0, s, dxs,
                      with_router ? b.dl : nullptr, idx, wrp, T, H, k, Et, b.dw_slot, static_cast<bf16_t*>(dx));
-  if (with_router) {
+  if (with_router)
     hipLaunchKernelGGL(dwr_partial_kernel, dim3((H + 255) / 256, slots, kDwrSplit), dim3(256), 0, s, xp, b.dl, b.wgrad_plan,
                        perm_slot, perm_token, H, b.dwr_part);
-    hipLaunchKernelGGL(dwr_sum_kernel, dim3((Et * H + 255) / 256), dim3(256), 0, s, b.dwr_part,
-                       b.wgrad_plan + 4 + 4 * (slots + Et), H, Et * H, static_cast<bf16_t*>(d_w_router));
-  }
   // weight gradients, contracted over each expert's rows: dW_down[e] = d^T (w h) (d gathered by token, `hidden`
   // already carries w), dW_gate_up[e] = [dg, du]^T x (x gathered by token)
   err = launch_wgrad<true, false>(dop, hidden, perm_token, offsets, zrow, H, I, S, E, slots, b.wgrad_plan, b.wgrad_part, static_cast<bf16_t*>(d_wd), s);
@@ -573,10 +586,12 @@ hipError_t launch_backward(const void* x, const void* d_out, const void* w_route
   float* part_gu = b.wgrad_part + (size_t)slots * H * I;
   err = launch_wgrad<false, true>(dgu, xp, perm_token, offsets, zrow, 2 * I, H, S, E, slots, b.wgrad_plan, part_gu, static_cast<bf16_t*>(d_wgu), s);
   if (err != hipSuccess) return err;
-  // experts with so many rows that they were cut into chunks: their partial tiles added up in chunk order
-  hipLaunchKernelGGL(wgrad_reduce_kernel, dim3((unsigned)(((size_t)2 * I * H / 4 + 255) / 256)), dim3(256), 0, s, b.wgrad_part,
-                     part_gu, b.wgrad_plan, slots, H * I, 2 * I * H, E, Et, b.theta_part, static_cast<bf16_t*>(d_wd),
-                     static_cast<bf16_t*>(d_wgu), d_theta);
+  // the sums that end the pass: cut experts' partial tiles, dtheta, the router's weight gradient
+  const int nb_w = (int)(((size_t)2 * I * H / 4 + 255) / 256);
+  const int nb_r = with_router ? (Et * H + 255) / 256 : 0;
+  hipLaunchKernelGGL(backward_sums_kernel, dim3(nb_w + E + nb_r), dim3(256), 0, s, nb_w, b.wgrad_part, part_gu, b.wgrad_plan,
+                     slots, H * I, 2 * I * H, E, Et, static_cast<bf16_t*>(d_wd), static_cast<bf16_t*>(d_wgu), b.dtheta_row,
+                     d_theta, b.dwr_part, H, with_router ? static_cast<bf16_t*>(d_w_router) : nullptr);
   return hipGetLastError();
 }
 

@@ -222,7 +222,6 @@ struct BackwardBuffers {
   void *gu, *dhp, *dgu, *hidden, *dxs, *zrow;                       // bf16 device buffers, sizes in launch_backward's comment
   float *dw_slot, *dl, *dtheta_row;                                 // [T*k] each
   float* dwr_part;                                                  // [backward_chunk_slots(), backward_dwr_split(), H]
-  float* theta_part;                                                // [backward_chunk_slots()]
   float* wgrad_part;                                                // backward_wgrad_part_bytes(): partial dW tiles of experts cut into chunks
   int* wgrad_plan;                                                  // backward_plan_bytes(): the list of row chunks, written by act_bwd_kernel
 };

@@ -293,7 +293,7 @@ __global__ __launch_bounds__(512) void dgrad_kmajor_kernel(const bf16_t* __restr
 // An expert with more than `chunk` rows is cut into chunks of that many rows, each a workgroup of its own per tile of
 // dW, so that a few experts holding most of the rows do not leave a few workgroups with most of the work; such an
 // expert's chunks write fp32 partial tiles to `part` (one [N, M] slot per chunk, slots numbered over all experts'
-// chunks) and wgrad_reduce_kernel adds them in chunk order.  Experts of one chunk write dW directly.  The chunks are
+// chunks) and wgrad_reduce_block adds them in chunk order.  Experts of one chunk write dW directly.  The chunks are
 // listed once per backward pass by wgrad_plan (below), so that a workgroup finds its chunk with one load.
 struct WgradPlan {
   int total;         // chunks over all experts
@@ -479,24 +479,15 @@ __global__ __launch_bounds__(512) void wgrad_kmajor_kernel(const bf16_t* __restr
   }
 }
 
-// The last launch of the backward pass.  For the experts that were cut into chunks (none, when the tokens are spread
-// evenly): dW[e] = the sum of expert e's partial tiles, in chunk order, for both weight tensors (partials of the first
-// in `part_a`, [.., NMa] each, of the second in `part_b`).  A thread per four elements.  And dtheta[e] = the sum of
-// expert e's per-chunk sums, in chunk order (workgroup 0, thread e).  E = experts with weights, Et = all.
-__global__ __launch_bounds__(256) void wgrad_reduce_kernel(const float* __restrict__ part_a, const float* __restrict__ part_b,
-                                                           const int* __restrict__ plan, int slots, int NMa, int NMb, int E,
-                                                           int Et, const float* __restrict__ theta_part,
-                                                           bf16_t* __restrict__ dWa, bf16_t* __restrict__ dWb,
-                                                           float* __restrict__ dtheta) {
-  if (blockIdx.x == 0 && (int)threadIdx.x < E) {
-    const int* ex = plan + 4 + 4 * (slots + Et + threadIdx.x);
-    float acc = 0.f;
-    for (int c = 0; c < ex[1]; ++c) acc += theta_part[ex[0] + c];
-    dtheta[threadIdx.x] = acc;
-  }
+// For the experts that were cut into chunks (none, when the tokens are spread evenly): dW[e] = the sum of expert e's
+// partial tiles, in chunk order, for both weight tensors (partials of the first in `part_a`, [.., NMa] each, of the
+// second in `part_b`).  Workgroup `block` of 256 threads, a thread per four elements.  E = experts with weights.
+__device__ __forceinline__ void wgrad_reduce_block(int block, const float* __restrict__ part_a, const float* __restrict__ part_b,
+                                                   const int* __restrict__ plan, int slots, int NMa, int NMb, int E,
+                                                   bf16_t* __restrict__ dWa, bf16_t* __restrict__ dWb) {
   const int n_cut = plan[1];
   if (n_cut == 0) return;
-  const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  const size_t i = ((size_t)block * 256 + threadIdx.x) * 4;
   const int* cut = plan + 4 + 4 * slots;
   auto reduce = [&](const float* part, int NM, bf16_t* dW, int e, int first, int n) {
     if (i >= (size_t)NM) return;
