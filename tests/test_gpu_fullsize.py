@@ -141,3 +141,45 @@ def test_streaming_kernels_take_repeats_that_fit_their_row_list():
     torch.cuda.synchronize()
     ref = O.experts_forward(p["x"], idx, w, p["w_gate_up"], p["w_down"], p["theta"])
     assert rel_err(out.cpu(), ref) <= BF16_TOL
+
+
+def test_half_a_million_tokens_cross_the_4_gib_offsets():
+    """T = 524288 at the prefill shape: 3.1 M routed rows, so the slot rows, the pre-activations and the per-slot input
+    gradients each hold more than 2^31 elements (4.8 GB) and every row offset near the end needs 64 bits.  A token's
+    output and input gradient depend on its own row, its routing and the weights alone, so chunks of the big call equal
+    the same tokens run by themselves bit for bit (first, middle and last chunk); the weight gradients of the big call
+    equal the sum over all 64 chunks' to bf16 rounding."""
+    T, H, E, k, I, CH = 524288, 768, 64, 6, 384, 8192
+    p = O.make_inputs(T=64, H=H, E=E, k=k, I=I, bias="uniform", theta="normal", seed=77)
+    wts = [p[n].to(DEV) for n in ("w_router", "bias", "w_gate_up", "w_down", "theta")]
+    g = torch.Generator(device=DEV).manual_seed(78)
+    x = torch.randn(T, H, generator=g, device=DEV, dtype=torch.float32).to(torch.bfloat16)
+    d = torch.randn(T, H, generator=g, device=DEV, dtype=torch.float32).to(torch.bfloat16)
+    assert T * k * H > 2 ** 31
+    try:
+        out, idx, w, _, _ = ops.moe_forward(x, *wts, k, want_routing=True)
+        grads = ops.moe_backward(x, d, *wts, k)
+        torch.cuda.synchronize()
+        assert all(bool(torch.isfinite(t.float()).all()) for t in (out,) + tuple(grads[:5]))
+        sums = [torch.zeros_like(t, dtype=torch.float64) for t in grads[1:5]]
+        for a in range(0, T, CH):
+            gc = ops.moe_backward(x[a:a + CH], d[a:a + CH], *wts, k)
+            for s_, t_ in zip(sums, gc[1:5]):
+                s_ += t_.double()
+            if a in (0, T // 2, T - CH):
+                oc, ic, wc, _, _ = ops.moe_forward(x[a:a + CH], *wts, k, want_routing=True)
+                assert torch.equal(ic, idx[a:a + CH]) and torch.equal(wc, w[a:a + CH]), f"routing of chunk {a}"
+                assert torch.equal(oc, out[a:a + CH]), f"output of chunk {a}"
+                assert torch.equal(gc[0], grads[0][a:a + CH]), f"input gradient of chunk {a}"
+        for name, s_, t_ in zip(("d_w_router", "d_w_gate_up", "d_w_down", "d_theta"), sums, grads[1:5]):
+            err = ((t_.double() - s_).abs().max() / s_.abs().max()).item()
+            assert err <= BF16_TOL, f"{name}: big call against the sum over chunks, rel err {err:.3e}"
+        # the last tokens against the fp32 oracle
+        tail = slice(T - 64, T)
+        oi, ow = idx[tail].cpu().numpy(), w[tail].cpu().numpy()
+        ref = O.experts_forward(x[tail].cpu(), oi, ow, p["w_gate_up"], p["w_down"], p["theta"])
+        assert rel_err(out[tail].cpu(), ref) <= BF16_TOL
+    finally:
+        ops._workspaces.clear()                      # 20 GB of workspace: not kept for the tests that follow
+        del x, d
+        torch.cuda.empty_cache()
