@@ -30,6 +30,7 @@ def test_forward_and_backward_replay_like_eager_calls(shape):
     wts = [p0[n].to(DEV) for n in NAMES]
     x_s, d_s = p0["x"].to(DEV), d0.to(DEV)
 
+    norm_w = (1.0 + 0.1 * torch.randn(shape["H"], generator=torch.Generator().manual_seed(9))).to(DEV)
     keeps = ops.train_state_bytes(shape["T"], shape["H"], shape["E"], k, shape["I"], torch.bfloat16) is not None
 
     def call(x, d):
@@ -40,6 +41,10 @@ def test_forward_and_backward_replay_like_eager_calls(shape):
             w_router, _, w_gate_up, w_down, theta = wts
             res += (out_t, counts_t) + tuple(ops.moe_backward_saved(x, d, w_router, w_gate_up, w_down, theta, k, state,
                                                                     want_dw=True))
+        # the caller's seam (norm + block + residual) and the experts alone with the routing handed over
+        res += tuple(ops.ffn_forward(x, norm_w, 1e-6, *wts, k, want_routing=True, want_counts=True))
+        res += (ops.experts_fwd(x, idx, w, wts[2], wts[3], wts[4])[0],)
+        res += tuple(ops.experts_backward(x, d, idx, w, wts[2], wts[3], wts[4]))
         return res
 
     side = torch.cuda.Stream(device=DEV)
@@ -60,8 +65,12 @@ def test_forward_and_backward_replay_like_eager_calls(shape):
         graph.replay()
         torch.cuda.synchronize()
         grads = ("d_x", "d_w_router", "d_w_gate_up", "d_w_down", "d_theta", "d_w")
-        names = ("out", "idx", "w", "counts") + grads + ("out (train)", "counts (train)") + tuple(g + " (saved)" for g in grads)
-        assert len(captured) == len(eager) == (18 if keeps else 10)
+        names = ("out", "idx", "w", "counts") + grads
+        if keeps:
+            names += ("out (train)", "counts (train)") + tuple(g + " (saved)" for g in grads)
+        names += ("out (seam)", "idx (seam)", "w (seam)", "counts (seam)", "out (experts)", "d_x (experts)", "d_w (experts)",
+                  "d_w_gate_up (experts)", "d_w_down (experts)", "d_theta (experts)")
+        assert len(captured) == len(eager) == len(names)
         for name, a, b in zip(names, captured, eager):
             assert torch.equal(a, b), f"{name} of the replay differs from the eager call (seed {seed}, {shape})"
 
