@@ -6,11 +6,12 @@
 // 128-byte line: the L2 -> LDS path moves almost twice the bytes per second for whole lines than for the
 // half lines of a 32-element step.  All 2I weight rows of a step would not fit LDS more than once, so a step
 // is cut into I/128 sub-steps of 256 rows: sub-step t holds, for each of the four N waves, its t-th 32-column
-// gate tile and the up tile of the same columns (16 MFMAs per wave).  The 32 KB stages form a ring (three
-// for I = 384, two otherwise): the rows of sub-step n + ring - 1 are requested while sub-step n is multiplied,
-// and a wave waits only until the loads older than the latest sub-step's have landed (loads complete in order),
-// so the L2 -> LDS path always has a stage or two in flight instead of draining at every barrier.  The x rows of
-// step s+1 arrive during step s in a double buffer of their own.
+// gate tile and the up tile of the same columns (16 MFMAs per wave).  The 32 KB stages form a ring of three (two
+// where I < 384 meets blocks of 384 output columns, whose staging buffers leave no room): the rows of sub-step
+// n + ring - 1 are requested while sub-step n is multiplied, and a wave waits only until the loads older than the
+// latest sub-step's have landed (loads complete in order), so the L2 -> LDS path always has a stage or two in flight
+// instead of draining at every barrier.  The x rows of step s+1 arrive during step s in a double buffer of their own
+// (I = 384), or those of step s+2 in a ring of three (I < 384).
 // Phase 2 turns the accumulators into bf16 activations and parks them in the stages, whose contents are dead by
 // then, as an operand of the second GEMM: stage t holds columns [128t, 128t+128) of all 128 rows; row r keeps
 // 16-byte granule c at position c ^ (r & 15), which spreads the 16 lanes of a fragment read over all banks
@@ -42,7 +43,11 @@ struct FusedShape {
   static constexpr int MT = 2, BM = 128, BK = 64;
   static constexpr int I = 128 * NT;
   static constexpr int BN2 = 128 * CT;                             // output columns per block: 8 waves x CT x 16
-  static constexpr int kRing = NT == 3 ? 3 : 2;                    // weight stages in LDS
+  // I = 384: the three stages are the three sub-steps of a K step and the x rows alternate between two buffers.
+  // I < 384 with at most 256 output columns per block (kDeep): three stages all the same, walked round by the running
+  // sub-step, and a third x buffer, so that x rows are requested two K steps ahead.  Otherwise two stages.
+  static constexpr bool kDeep = NT < 3 && CT < 3;
+  static constexpr int kRing = (NT == 3 || kDeep) ? 3 : 2;         // weight stages in LDS
   static constexpr int kDist = kRing - 1;                          // sub-steps between a stage's request and its use
   static constexpr int kStageRows = 256;                           // 4 N waves x (gate tile + up tile) x 32 rows
   static constexpr int kStageElems = kStageRows * BK;              // 32 KB = one [128][128] slice of the activations
@@ -147,6 +152,7 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
   __shared__ __attribute__((aligned(16))) bf16_t S2[F::kRing == 3 ? F::kStageElems : 8];
   __shared__ __attribute__((aligned(16))) bf16_t A0[F::kXElems];      // x rows of even K steps; then output staging,
   __shared__ __attribute__((aligned(16))) bf16_t A1[F::kXElems];      // x rows of odd K steps;  alternating per 32 rows
+  __shared__ __attribute__((aligned(16))) bf16_t A2[F::kDeep ? F::kAElems : 8];   // kDeep: x rows of every third K step
   __shared__ float ssq[4 * BM];
   __shared__ float rinv_s[BM], gain_s[BM], w_s[BM];
   __shared__ int slot_s[BM];
@@ -199,6 +205,72 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
       const int m = min(a * 64 + drow, rows - 1);                                // rows past the end re-read the last valid row
       ld.a_voff[a] = (unsigned)perm_token[row0 + m] * hb + chunk * 16;          // gather, moe.py:81
     }
+    const int pos0 = ((lane >> 5) ^ ((n >> 1) & 7)) * 8;    // fragment side: lane (n, h) reads logical granule 2*ss + h of rows congruent to n mod 32
+    auto frag_row = [&](int j) { return (wn * 2 + j) * 32; };
+    using std::integral_constant;
+    auto zero_acc = [&]() {                      // (after the prologue's requests, which do not wait for it)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int j = 0; j < 2 * NT; ++j)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) acc[mt][j][i] = 0.f;
+    };
+    if constexpr (F::kDeep) {
+      // Sub-step g = s NT + t reads stage g % 3 and x buffer s % 3, and requests the weight rows of sub-step g + 2
+      // and, at t = 0, the x rows of step s + 2 (K steps clamped to the last one: requests past the end fetch valid
+      // rows into buffers nobody reads again).  The K loop is unrolled by three steps (ph = s % 3), so every buffer is
+      // chosen at compile time.  What a sub-step may leave in flight are the loads of the sub-step before it.
+      auto abuf = [&](auto ic) -> bf16_t* {
+        constexpr int i = decltype(ic)::value;
+        if constexpr (i == 0) return A0; else if constexpr (i == 1) return A1; else return A2;
+      };
+      constexpr unsigned kb = BK * sizeof(bf16_t);
+      // prologue, oldest first: sub-step 0, x rows of steps 0 and 1, sub-step 1
+#pragma unroll
+      for (int q = 0; q < F::kBInstr; ++q) dma16_buf(ld.w_rsrc, ld.b_voff, q * ld.bstep, S0 + q * 512 * 8 + ld.wave_elems);
+#pragma unroll
+      for (int a = 0; a < 2; ++a) dma16_buf(ld.x_rsrc, ld.a_voff[a], 0, A0 + a * 512 * 8 + ld.wave_elems);
+#pragma unroll
+      for (int a = 0; a < 2; ++a) dma16_buf(ld.x_rsrc, ld.a_voff[a], kb, A1 + a * 512 * 8 + ld.wave_elems);
+#pragma unroll
+      for (int q = 0; q < F::kBInstr; ++q)
+        dma16_buf(ld.w_rsrc, ld.b_voff, (NT == 1 ? kb : 32 * hb) + q * ld.bstep, S1 + q * 512 * 8 + ld.wave_elems);
+      zero_acc();
+      auto substep = [&](auto mc, auto phc, auto tc, int s) {
+        constexpr int nmt = decltype(mc)::value;
+        constexpr int ph = decltype(phc)::value, t = decltype(tc)::value;
+        constexpr int cur = (ph * NT + t) % 3, target = (ph * NT + t + 2) % 3;
+        constexpr int tn = (t + 2) % NT, ds = (t + 2) / NT;
+        constexpr bool after_t0 = NT == 1 || t == 1;                   // the sub-step before also requested x rows
+        sync_keep_loads<F::kBInstr + (after_t0 ? 2 : 0)>();
+        const bf16_t* a0 = abuf(integral_constant<int, ph>{}) + (mbase + n) * BK + pos0;
+        const bf16_t* b0 = stage(integral_constant<int, cur>{}) + n * BK;
+        ld.b_soff = (unsigned)tn * 32 * hb + (unsigned)min(s + ds, nsteps - 1) * kb;
+        ld.b_dst = stage(integral_constant<int, target>{});
+        ld.a_soff = (unsigned)min(s + 2, nsteps - 1) * kb;
+        ld.a_dst = abuf(integral_constant<int, (ph + 2) % 3>{});
+        const SubIssuer<F, t == 0> issuer{ld};
+        if constexpr (nmt > 0)
+          stripe_step<nmt, 2, BK, true, 2 * NT, t, NT>(acc, a0, 32 * BK, b0, pos0, frag_row, issuer, true, 0, nullptr);
+        else
+          issue_some<0, SubIssuer<F, t == 0>::kInstr>(issuer, 0, nullptr);
+      };
+      auto kstep = [&](auto mc, auto phc, int s) {
+        substep(mc, phc, integral_constant<int, 0>{}, s);
+        if constexpr (NT > 1) substep(mc, phc, integral_constant<int, 1>{}, s);
+      };
+      auto kloop = [&](auto mc) {
+        for (int s = 0; s < nsteps; s += 3) {
+          kstep(mc, integral_constant<int, 0>{}, s);
+          if (s + 1 < nsteps) kstep(mc, integral_constant<int, 1>{}, s + 1);
+          if (s + 2 < nsteps) kstep(mc, integral_constant<int, 2>{}, s + 2);
+        }
+      };
+      if (my_blocks == 2) kloop(integral_constant<int, 2>{});
+      else if (my_blocks == 1) kloop(integral_constant<int, 1>{});
+      else kloop(integral_constant<int, 0>{});
+    } else {
     // what sub-step (s, t) requests: the weight rows of sub-step (s, t) + kDist (its K step clamped to the last
     // one: requests past the end fetch valid rows into a stage nobody reads again), and at t = 0 the x rows of
     // step s + 1.  Every sub-step issues the same number of loads, so the wait counts below are constants.
@@ -222,15 +294,7 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
       for (int q = 0; q < F::kBInstr; ++q)
         dma16_buf(ld.w_rsrc, ld.b_voff, 32 * hb + q * ld.bstep, S1 + q * 512 * 8 + ld.wave_elems);   // sub-step (0, 1)
     }
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-      for (int j = 0; j < 2 * NT; ++j)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) acc[mt][j][i] = 0.f;
-    // fragment side: lane (n, h) reads logical granule 2*ss + h of rows congruent to n mod 32
-    const int pos0 = ((lane >> 5) ^ ((n >> 1) & 7)) * 8;
-    auto frag_row = [&](int j) { return (wn * 2 + j) * 32; };
+    zero_acc();
     auto substep = [&](auto mc, auto tc, auto pc, int s) {
       constexpr int nmt = decltype(mc)::value;           // M tiles of this wave that hold rows
       constexpr int t = decltype(tc)::value, par = decltype(pc)::value;
@@ -248,7 +312,6 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
       else
         issue_some<0, SubIssuer<F, t == 0>::kInstr>(issuer, 0, nullptr);   // its share of the requests all the same
     };
-    using std::integral_constant;
     // one copy of the K loop per number of M tiles with rows, chosen once: a choice inside the loop would meet at
     // every sub-step with all 192 accumulator registers alive
     auto kloop = [&](auto mc) {
@@ -265,6 +328,7 @@ __global__ __launch_bounds__(512) void experts_fused_kernel(const bf16_t* __rest
     if (my_blocks == 2) kloop(integral_constant<int, 2>{});
     else if (my_blocks == 1) kloop(integral_constant<int, 1>{});
     else kloop(integral_constant<int, 0>{});
+      }
   }
   wait_loads_and_sync();                   // every transfer has landed and every wave is done with the stages
 
@@ -506,7 +570,9 @@ template <int NT>
 void launch_fused_nt(const bf16_t* x, const bf16_t* wgu, const bf16_t* wd, const float* theta, const float* w,
                      const int32_t* offsets, const int32_t* perm_slot, const int32_t* perm_token, int S, int H, int E,
                      int act, unsigned x_bytes, bf16_t* yw, bf16_t* preact, hipStream_t s) {
-  if (H % 384 == 0) launch_fused_t<NT, 3>(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, S, H, E, act, x_bytes, yw, preact, s);
+  // (blocks of 256 columns leave room for the third x buffer of the deeper ring where I < 384)
+  if (H % 384 == 0 && (NT == 3 || H % 256 != 0))
+    launch_fused_t<NT, 3>(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, S, H, E, act, x_bytes, yw, preact, s);
   else if (H % 256 == 0) launch_fused_t<NT, 2>(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, S, H, E, act, x_bytes, yw, preact, s);
   else launch_fused_t<NT, 1>(x, wgu, wd, theta, w, offsets, perm_slot, perm_token, S, H, E, act, x_bytes, yw, preact, s);
 }

@@ -211,7 +211,8 @@ def test_mfma_and_generic_families_agree():
 @pytest.mark.parametrize("T,H,I,k,bias", [(1024, 768, 384, 6, "uniform"), (1024, 768, 384, 6, "hot4"),
                                           (333, 256, 128, 6, "uniform"), (130, 128, 256, 6, "zero"),
                                           (777, 512, 256, 6, "uniform"), (515, 640, 384, 8, "uniform"),
-                                          (1, 768, 384, 6, "zero")])
+                                          (600, 768, 256, 6, "uniform"), (400, 1024, 128, 6, "uniform"),
+                                          (450, 640, 256, 6, "uniform"), (1, 768, 384, 6, "zero")])
 def test_fused_kernel_matches_oracle_and_the_two_kernel_family(T, H, I, k, bias):
     """One launch for both GEMMs (activations never leave the CU): same operand rounding as the two MFMA
     kernels, another accumulation order in the down projection."""
