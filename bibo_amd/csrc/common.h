@@ -172,7 +172,7 @@ hipError_t launch_permute(const int32_t* idx, int T, int E, int k, int32_t* coun
                           int32_t* perm_slot, int32_t* perm_token, void* ws, hipStream_t s);
 size_t router_hist_bytes(int T);
 bool permute_takes_router_hist(int T, int k);
-hipError_t launch_permute_from_hist(const int32_t* idx, int T, int E, int k, const int32_t* hist, int hist_tokens,
+hipError_t launch_permute_from_hist(const int32_t* idx, int T, int E, int k, int32_t* hist, int hist_tokens,
                                     int32_t* counts, int32_t* offsets, int32_t* perm_slot, int32_t* perm_token,
                                     hipStream_t s);
 hipError_t launch_gateup_generic(const void* x, const void* wgu, const float* theta, const int32_t* offsets,

@@ -24,6 +24,31 @@ __global__ __launch_bounds__(256) void hist_kernel(const int32_t* __restrict__ i
   if (tid < kMaxE) block_hist[blockIdx.x * kMaxE + tid] = h[tid];
 }
 
+// Many histograms (large batches): sums over blocks of kHistBlock consecutive histograms, so that a scatter workgroup
+// adds up the block sums and the histograms of its own block instead of every histogram in front of it.
+constexpr int kHistBlock = 256;
+constexpr int kTwoLevelMin = 1024;                 // histograms from which the extra launch pays
+
+__global__ __launch_bounds__(256) void hist_blocksum_kernel(const int32_t* __restrict__ hist, int nhist,
+                                                            int32_t* __restrict__ block_sum) {
+  __shared__ int part[4][kMaxE];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int first = blockIdx.x * kHistBlock;
+  constexpr int kPer = kHistBlock / 4;
+  int v[kPer];
+#pragma unroll
+  for (int u = 0; u < kPer; ++u) {
+    const int bb = first + wave + 4 * u;
+    v[u] = bb < nhist ? hist[bb * kMaxE + lane] : 0;
+  }
+  int acc = 0;
+#pragma unroll
+  for (int u = 0; u < kPer; ++u) acc += v[u];
+  part[wave][lane] = acc;
+  __syncthreads();
+  if (wave == 0) block_sum[blockIdx.x * kMaxE + lane] = (part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane]);
+}
+
 // One workgroup per chunk of kPermTokens tokens, four waves of kPermTokens/4 tokens each, lane = expert for the
 // bookkeeping.  (1) every wave gets the per-expert counts of its own slots; (2) the chunk histograms are
 // summed (all chunks for the totals, earlier chunks for this workgroup's base), the loads issued in batches;
@@ -35,6 +60,7 @@ __global__ __launch_bounds__(256) void hist_kernel(const int32_t* __restrict__ i
 template <int HT>
 __global__ __launch_bounds__(256) void scatter_kernel(const int32_t* __restrict__ idx, int S, int E, int k,
                                                       const int32_t* __restrict__ hist, int nhist,
+                                                      const int32_t* __restrict__ block_sum,
                                                       int32_t* __restrict__ counts, int32_t* __restrict__ offsets,
                                                       int32_t* __restrict__ perm_slot, int32_t* __restrict__ perm_token) {
   static_assert(kPermTokens == 128 && (HT == kPermTokens || HT == 16 || HT == 32), "a wave owns 32 tokens");
@@ -78,18 +104,38 @@ __global__ __launch_bounds__(256) void scatter_kernel(const int32_t* __restrict_
 
   int tot = 0, bef = 0;
   constexpr int kBatch = 64;                       // histograms requested together: one memory latency per batch
-  for (int bb0 = wave; bb0 < nhist; bb0 += 4 * kBatch) {
+  if (block_sum == nullptr) {
+    for (int bb0 = wave; bb0 < nhist; bb0 += 4 * kBatch) {
+      int v[kBatch];
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) {
+        const int bb = bb0 + 4 * u;
+        v[u] = (bb < nhist) ? hist[bb * kMaxE + lane] : 0;
+      }
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) {
+        tot += v[u];
+        bef += (bb0 + 4 * u < h0) ? v[u] : 0;
+      }
+    }
+  } else {
+    // two levels: the sums of whole blocks of histograms, then the histograms of this workgroup's own block in front
+    // of its first one
+    static_assert(kHistBlock == 4 * kBatch, "one batch per wave covers a block");
+    const int nblk = (nhist + kHistBlock - 1) / kHistBlock, hb = h0 / kHistBlock;
     int v[kBatch];
 #pragma unroll
     for (int u = 0; u < kBatch; ++u) {
-      const int bb = bb0 + 4 * u;
-      v[u] = (bb < nhist) ? hist[bb * kMaxE + lane] : 0;
+      const int bb = hb * kHistBlock + wave + 4 * u;
+      v[u] = (bb < h0) ? hist[bb * kMaxE + lane] : 0;
+    }
+    for (int blk = wave; blk < nblk; blk += 4) {
+      const int bs = block_sum[blk * kMaxE + lane];
+      tot += bs;
+      bef += blk < hb ? bs : 0;
     }
 #pragma unroll
-    for (int u = 0; u < kBatch; ++u) {
-      tot += v[u];
-      bef += (bb0 + 4 * u < h0) ? v[u] : 0;
-    }
+    for (int u = 0; u < kBatch; ++u) bef += v[u];
   }
   part_tot[wave][lane] = tot;
   part_bef[wave][lane] = bef;
@@ -169,13 +215,23 @@ __global__ __launch_bounds__(64) void permute_small_kernel(const int32_t* __rest
 
 }  // namespace
 
+// the chunk histograms and, behind them, their block sums
 size_t permute_workspace_bytes(int T) {
   const size_t nblk = (size_t)(T + kPermTokens - 1) / kPermTokens;
-  return (nblk > 0 ? nblk : 1) * kMaxE * sizeof(int32_t);
+  return ((nblk > 0 ? nblk : 1) + nblk / kHistBlock + 1) * kMaxE * sizeof(int32_t);
 }
 
-// room for the histograms the router kernel writes, one per 16 tokens at the finest
+// room for the histograms the router kernel writes, one per 16 tokens at the finest (one per 32 tokens from 8192
+// tokens on, which leaves the upper half for their block sums)
 size_t router_hist_bytes(int T) { return ((size_t)(T + 15) / 16 + 1) * kMaxE * sizeof(int32_t); }
+
+// block sums of `nhist` histograms into the entries behind them, when there are enough of them to pay for the launch
+static const int32_t* block_sums(int32_t* hist, int nhist, hipStream_t s) {
+  if (nhist < kTwoLevelMin) return nullptr;
+  int32_t* sums = hist + (size_t)nhist * kMaxE;
+  hipLaunchKernelGGL(hist_blocksum_kernel, dim3((nhist + kHistBlock - 1) / kHistBlock), dim3(256), 0, s, hist, nhist, sums);
+  return sums;
+}
 
 hipError_t launch_permute(const int32_t* idx, int T, int E, int k, int32_t* counts, int32_t* offsets,
                           int32_t* perm_slot, int32_t* perm_token, void* ws, hipStream_t s) {
@@ -189,8 +245,8 @@ hipError_t launch_permute(const int32_t* idx, int T, int E, int k, int32_t* coun
   }
   const int grid = nblk;
   hipLaunchKernelGGL(hist_kernel, dim3(grid), dim3(256), 0, s, idx, S, E, k, block_hist);
-  hipLaunchKernelGGL(scatter_kernel<kPermTokens>, dim3(grid), dim3(256), 0, s, idx, S, E, k, block_hist, grid, counts,
-                     offsets, perm_slot, perm_token);
+  hipLaunchKernelGGL(scatter_kernel<kPermTokens>, dim3(grid), dim3(256), 0, s, idx, S, E, k, block_hist, grid,
+                     block_sums(block_hist, grid, s), counts, offsets, perm_slot, perm_token);
   return hipGetLastError();
 }
 
@@ -198,17 +254,17 @@ bool permute_takes_router_hist(int T, int k) { return T * k > kSmallSlots; }
 
 // The same permutation from the per-workgroup histograms the router kernel wrote (one per `hist_tokens` tokens):
 // no histogram launch and no counting pass.
-hipError_t launch_permute_from_hist(const int32_t* idx, int T, int E, int k, const int32_t* hist, int hist_tokens,
+hipError_t launch_permute_from_hist(const int32_t* idx, int T, int E, int k, int32_t* hist, int hist_tokens,
                                     int32_t* counts, int32_t* offsets, int32_t* perm_slot, int32_t* perm_token,
                                     hipStream_t s) {
   const int grid = (T + kPermTokens - 1) / kPermTokens;
   const int nhist = (T + hist_tokens - 1) / hist_tokens;
   if (hist_tokens == 32)
-    hipLaunchKernelGGL(scatter_kernel<32>, dim3(grid), dim3(256), 0, s, idx, T * k, E, k, hist, nhist, counts, offsets,
-                       perm_slot, perm_token);
-  else if (hist_tokens == 16)
-    hipLaunchKernelGGL(scatter_kernel<16>, dim3(grid), dim3(256), 0, s, idx, T * k, E, k, hist, nhist, counts, offsets,
-                       perm_slot, perm_token);
+    hipLaunchKernelGGL(scatter_kernel<32>, dim3(grid), dim3(256), 0, s, idx, T * k, E, k, hist, nhist,
+                       block_sums(hist, nhist, s), counts, offsets, perm_slot, perm_token);
+  else if (hist_tokens == 16)   // (fewer than 8192 tokens: never enough histograms for block sums, and no room for them)
+    hipLaunchKernelGGL(scatter_kernel<16>, dim3(grid), dim3(256), 0, s, idx, T * k, E, k, hist, nhist,
+                       static_cast<const int32_t*>(nullptr), counts, offsets, perm_slot, perm_token);
   else
     return hipErrorInvalidValue;
   return hipGetLastError();

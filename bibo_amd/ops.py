@@ -130,7 +130,8 @@ def permute(idx, E):
     offsets = torch.empty(E + 1, dtype=torch.int32, device=dev)
     perm_slot = torch.empty(T * k, dtype=torch.int32, device=dev)
     perm_token = torch.empty(T * k, dtype=torch.int32, device=dev)
-    nb = max(1, (T + 127) // 128) * 64 * 4          # one 64-entry histogram per 128 tokens
+    # one 64-entry histogram per 128 tokens and, for large batches, one sum per 256 histograms
+    nb = (max(1, (T + 127) // 128) + (T + 32767) // 32768 + 1) * 64 * 4
     ws = workspace(dev, nb)
     with torch.cuda.device(dev):
         L.check(L.lib().bibo_moe_permute(_ptr(idx), T, E, k, _ptr(counts), _ptr(offsets), _ptr(perm_slot),

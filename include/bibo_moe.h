@@ -149,7 +149,8 @@ int bibo_moe_router_fwd(const void* x, const void* w_router, const float* bias, 
  * bincount of BiBoMoELayer._balance_step (moe.py:141-145).
  *   idx int32 [T,k]; counts int32 [E]; offsets int32 [E+1]; perm_slot, perm_token int32 [T*k]
  * Indices outside [0,E) are ignored (their slots get no row and offsets[E] < T*k).
- * workspace: at least 256 * max(1, ceil(T / 128)) bytes (one 64-entry histogram per 128 tokens).
+ * workspace: at least 256 * (max(1, ceil(T / 128)) + ceil(T / 32768) + 1) bytes (one 64-entry histogram per 128 tokens
+ * and, for large batches, one sum per 256 histograms).
  */
 int bibo_moe_permute(const int32_t* idx, int T, int E, int k, int32_t* counts, int32_t* offsets,
                      int32_t* perm_slot, int32_t* perm_token, void* workspace, size_t workspace_bytes,

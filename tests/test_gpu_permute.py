@@ -32,6 +32,16 @@ def test_permutation_matches_oracle(T, E, k):
     _check(_random_idx(T, E, k, T + E + k), E)
 
 
+@pytest.mark.parametrize("T,E,k", [(131072, 64, 6), (140001, 64, 6), (200000, 7, 2)])
+def test_large_batches_take_the_block_sums(T, E, k):
+    """From 1024 chunk histograms on (131072 tokens) a launch sums them in blocks of 256 and every scatter workgroup
+    adds block sums plus the histograms of its own block; the permutation is the same, bit for bit."""
+    _check(_random_idx(T, E, k, T + E), E)
+    skew = _random_idx(T, E, k, 5)
+    skew[: T // 2] = np.arange(k)                                       # half of the tokens on the first k experts
+    _check(skew, E)
+
+
 def test_empty_and_skewed_and_repeated():
     _check(np.zeros((0, 6), dtype=np.int32), 64)                       # no tokens: counts and offsets all zero
     idx = _random_idx(4096, 64, 6, 1)
