@@ -183,3 +183,27 @@ def test_half_a_million_tokens_cross_the_4_gib_offsets():
         ops._workspaces.clear()                      # 20 GB of workspace: not kept for the tests that follow
         del x, d
         torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("T", [32768, 32768 + 40, 70000])
+def test_block_sums_of_the_router_histograms_from_1024_on(T):
+    """From 1024 router histograms on (32768 tokens) the permutation adds them up in two levels: counts and the
+    permutation against the oracle, bit for bit, and the ends of the output against the same tokens run alone."""
+    H, E, k, I, CH = 256, 64, 6, 128, 4096
+    p = O.make_inputs(T=64, H=H, E=E, k=k, I=I, bias="uniform", theta="normal", seed=91)
+    wts = [p[n].to(DEV) for n in ("w_router", "bias", "w_gate_up", "w_down", "theta")]
+    g = torch.Generator(device=DEV).manual_seed(T)
+    x = torch.randn(T, H, generator=g, device=DEV, dtype=torch.float32).to(torch.bfloat16)
+    out, idx, w, counts, _ = ops.moe_forward(x, *wts, k, want_routing=True, want_counts=True)
+    torch.cuda.synchronize()
+    idx_np = idx.cpu().numpy()
+    oc, _, oslot, otoken = O.permute(idx_np, E)
+    assert np.array_equal(counts.cpu().numpy(), oc)
+    # the permutation itself, through the stage entry point fed with the same indices (hist_kernel's histograms)
+    c2_, _, ps, pt = ops.permute(idx, E)
+    assert np.array_equal(c2_.cpu().numpy(), oc) and np.array_equal(ps.cpu().numpy(), oslot)
+    assert np.array_equal(pt.cpu().numpy(), otoken)
+    for a in (0, (T // 2) & ~127, T - CH):
+        oc_, ic_, wc_, _, _ = ops.moe_forward(x[a:a + CH], *wts, k, want_routing=True)
+        assert torch.equal(ic_, idx[a:a + CH]) and torch.equal(wc_, w[a:a + CH])
+        assert torch.equal(oc_, out[a:a + CH]), f"output of chunk {a}"
